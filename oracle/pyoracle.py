@@ -1,0 +1,285 @@
+"""numpy front end of libtsattn_oracle.so (the CPU checker).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline
+leg of bench.py.  The product package (tscale_amd) never imports this module.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtsattn_oracle.so")
+
+I8 = 0
+E4M3 = 1
+
+_c = ctypes
+_i64 = _c.c_int64
+_f32 = _c.c_float
+_int = _c.c_int
+_vp = _c.c_void_p
+
+
+def build():
+    """Compile the checker with gcc (make in this directory)."""
+    subprocess.check_call(["make", "-C", _HERE, "-B", "libtsattn_oracle.so"], stdout=subprocess.DEVNULL)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.tso_e4m3_to_float.restype = _f32
+        L.tso_e4m3_to_float.argtypes = [_c.c_uint8]
+        L.tso_float_to_e4m3.restype = _c.c_uint8
+        L.tso_float_to_e4m3.argtypes = [_f32]
+        L.tso_float_to_i8.restype = _c.c_int8
+        L.tso_float_to_i8.argtypes = [_f32]
+        L.tso_bf16_to_float.restype = _f32
+        L.tso_bf16_to_float.argtypes = [_c.c_uint16]
+        L.tso_float_to_bf16.restype = _c.c_uint16
+        L.tso_float_to_bf16.argtypes = [_f32]
+        L.tso_att_dot_scale.restype = _f32
+        L.tso_att_dot_scale.argtypes = [_int]
+        L.tso_quantize_rows.restype = None
+        L.tso_quantize_rows.argtypes = [_int, _vp, _i64, _i64, _int, _int, _vp, _i64, _vp, _i64]
+        L.tso_quantize_rows_bf16.restype = None
+        L.tso_quantize_rows_bf16.argtypes = [_int, _vp, _i64, _i64, _int, _int, _vp, _i64, _vp, _i64]
+        L.tso_make_spans.restype = None
+        L.tso_make_spans.argtypes = [_i64, _vp, _vp, _i64, _vp, _vp]
+        L.tso_init_alibi.restype = _int
+        L.tso_init_alibi.argtypes = [_int, _i64, _int, _vp, _vp]
+        L.tso_dot_i8.restype = _c.c_int32
+        L.tso_dot_i8.argtypes = [_vp, _vp, _int]
+        L.tso_dot_i8_simd.restype = _c.c_int32
+        L.tso_dot_i8_simd.argtypes = [_vp, _vp, _int]
+        L.tso_dot_e4m3.restype = _f32
+        L.tso_dot_e4m3.argtypes = [_vp, _vp, _int]
+        L.tso_qk_accum.restype = None
+        L.tso_qk_accum.argtypes = [_int, _vp, _i64, _vp, _i64, _int, _int, _i64, _i64, _i64, _i64, _vp]
+        L.tso_prefill_f32.restype = None
+        L.tso_prefill_f32.argtypes = [_i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _f32, _vp, _vp, _vp]
+        L.tso_prefill_q8.restype = None
+        L.tso_prefill_q8.argtypes = [_int, _i64, _int, _int, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64,
+                                     _f32, _f32, _f32, _vp, _vp, _f32, _vp, _i64, _vp, _int]
+        L.tso_decode.restype = None
+        L.tso_decode.argtypes = [_int, _i64, _int, _int, _vp, _vp, _f32, _vp, _vp, _i64, _i64, _i64,
+                                 _vp, _vp, _i64, _i64, _f32, _f32, _vp, _i64, _f32, _int, _int, _vp,
+                                 _vp, _i64, _int]
+        L.tso_softmax_buf.restype = _f32
+        L.tso_softmax_buf.argtypes = [_vp, _int, _int, _vp]
+        L.tso_simd_level.restype = _int
+        L.tso_max_threads.restype = _int
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+def _c_arr(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+# ---- formats ---------------------------------------------------------------------------------
+def e4m3_table():
+    L = lib()
+    return np.array([L.tso_e4m3_to_float(i) for i in range(256)], dtype=np.float32)
+
+
+def float_to_e4m3(x):
+    L = lib()
+    x = np.asarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint8)
+    xf, of = x.ravel(), out.ravel()
+    for i in range(xf.size):
+        of[i] = L.tso_float_to_e4m3(float(xf[i]))
+    return out
+
+
+def float_to_i8(x):
+    L = lib()
+    x = np.asarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.int8)
+    xf, of = x.ravel(), out.ravel()
+    for i in range(xf.size):
+        of[i] = L.tso_float_to_i8(float(xf[i]))
+    return out
+
+
+def att_dot_scale(d):
+    return np.float32(lib().tso_att_dot_scale(int(d)))
+
+
+def quantize_rows(dtype, x, n_heads):
+    """x: [n_rows, n_heads*d] float32 (or uint16 holding bf16 bits) -> (q uint8 [n_rows, H*d], scale f32 [H, n_rows])."""
+    L = lib()
+    n_rows, hd = x.shape
+    d = hd // n_heads
+    q = np.empty((n_rows, hd), dtype=np.uint8)
+    scale = np.empty((n_heads, n_rows), dtype=np.float32)
+    if x.dtype == np.uint16:
+        x = np.ascontiguousarray(x)
+        L.tso_quantize_rows_bf16(dtype, _p(x), hd, n_rows, n_heads, d, _p(q), hd, _p(scale), n_rows)
+    else:
+        x = _c_arr(x, np.float32)
+        L.tso_quantize_rows(dtype, _p(x), hd, n_rows, n_heads, d, _p(q), hd, _p(scale), n_rows)
+    return q, scale
+
+
+def float_to_bf16_bits(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    lsb = (u >> 16) & 1
+    r = ((u + 0x7FFF + lsb) >> 16).astype(np.uint16)
+    return r
+
+
+def bf16_bits_to_float(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+# ---- masks -----------------------------------------------------------------------------------
+def make_spans(seq_lens, window, doc_start_flag=None):
+    L = lib()
+    off = np.zeros(len(seq_lens) + 1, dtype=np.int64)
+    off[1:] = np.cumsum(seq_lens)
+    n = int(off[-1])
+    st = np.empty(n, dtype=np.int32)
+    fi = np.empty(n, dtype=np.int32)
+    flag = None if doc_start_flag is None else _c_arr(doc_start_flag, np.uint8)
+    L.tso_make_spans(len(seq_lens), _p(off), _p(flag), int(window), _p(st), _p(fi))
+    return st, fi
+
+
+def init_alibi(depth, wide):
+    L = lib()
+    w = np.zeros(depth + 2, dtype=np.int64)
+    s = np.zeros(depth + 2, dtype=np.float32)
+    n = L.tso_init_alibi(int(depth), int(wide), depth + 2, _p(w), _p(s))
+    return w[:n].copy(), s[:n].copy()
+
+
+# ---- dots ------------------------------------------------------------------------------------
+def dot_i8(a, b, simd=False):
+    L = lib()
+    a = _c_arr(a, np.int8)
+    b = _c_arr(b, np.int8)
+    f = L.tso_dot_i8_simd if simd else L.tso_dot_i8
+    return int(f(_p(a), _p(b), a.size))
+
+
+def dot_e4m3(a, b):
+    L = lib()
+    a = _c_arr(a, np.uint8)
+    b = _c_arr(b, np.uint8)
+    return np.float32(L.tso_dot_e4m3(_p(a), _p(b), a.size))
+
+
+def qk_accum(dtype, q, k, head, d, from0, n_from, to0, n_to):
+    L = lib()
+    q = _c_arr(q, np.uint8)
+    k = _c_arr(k, np.uint8)
+    acc = np.empty((n_from, n_to), dtype=np.int32 if dtype == I8 else np.float32)
+    L.tso_qk_accum(dtype, _p(q), q.shape[1], _p(k), k.shape[1], head, d, from0, n_from, to0, n_to, _p(acc))
+    return acc
+
+
+# ---- attention --------------------------------------------------------------------------------
+def prefill_f32(qk, qv, v, n_heads, span_ptr, spans, slope):
+    L = lib()
+    qk = _c_arr(qk, np.float32)
+    qv = _c_arr(qv, np.float32)
+    v = _c_arr(v, np.float32)
+    n = qk.shape[0]
+    q_dim = qk.shape[1] // n_heads
+    tt_dim = v.shape[1] // n_heads
+    span_ptr = _c_arr(span_ptr, np.int32)
+    spans = _c_arr(spans, np.int32)
+    out = np.empty((n, n_heads * tt_dim), dtype=np.float32)
+    sw = np.empty((n_heads, n), dtype=np.float32)
+    mx = np.empty((n_heads, n), dtype=np.float32)
+    L.tso_prefill_f32(n, n_heads, q_dim, tt_dim, _p(qk), _p(qv), _p(v), _p(span_ptr), _p(spans),
+                      float(slope), _p(out), _p(sw), _p(mx))
+    return out, sw, mx
+
+
+def _scale_args(s, default):
+    if s is None:
+        return None, float(default)
+    if np.isscalar(s):
+        return None, float(s)
+    return _c_arr(s, np.float32), 0.0
+
+
+def prefill_q8(dtype, q, k, v, n_heads, q_scale, k_scale, v_scale, span_start, span_finish, slope,
+               want_swl=False, n_threads=0):
+    """q,k,v: uint8 [n_tokens, H*d]; scales f32 [H, n_tokens] or python scalars."""
+    L = lib()
+    q = _c_arr(q, np.uint8)
+    k = _c_arr(k, np.uint8)
+    v = _c_arr(v, np.uint8)
+    n, hd = q.shape
+    d = hd // n_heads
+    qs, qc = _scale_args(q_scale, 1.0)
+    ks, kc = _scale_args(k_scale, 1.0)
+    vs, vc = _scale_args(v_scale, 1.0)
+    st = _c_arr(span_start, np.int32)
+    fi = _c_arr(span_finish, np.int32)
+    out = np.empty((n, hd), dtype=np.float32)
+    swl = np.empty((n_heads, n), dtype=np.float32) if want_swl else None
+    if n_threads <= 0:
+        n_threads = L.tso_max_threads()
+    L.tso_prefill_q8(dtype, n, n_heads, d, _p(q), _p(k), _p(v), hd, _p(qs), _p(ks), _p(vs), n,
+                     qc, kc, vc, _p(st), _p(fi), float(slope), _p(out), hd, _p(swl), n_threads)
+    return (out, swl) if want_swl else out
+
+
+def decode(dtype, q, q_scale, k_cache, v_cache, k_scale, v_scale, cache_len, window, slope,
+           exp2_mode=0, use_simd=False, want_acc=False, n_threads=0):
+    """Planar cache: k_cache, v_cache uint8 [B, H, L, d]; k_scale, v_scale f32 [B, H, L] (or scalars);
+    q uint8 [B, H*d]; q_scale f32 [B, H] or scalar; cache_len int32 [B]."""
+    L = lib()
+    k_cache = _c_arr(k_cache, np.uint8)
+    v_cache = _c_arr(v_cache, np.uint8)
+    B, H, Lmax, d = k_cache.shape
+    q = _c_arr(q, np.uint8)
+    qs, qc = _scale_args(q_scale, 1.0)
+    ks, kc = _scale_args(k_scale, 1.0)
+    vs, vc = _scale_args(v_scale, 1.0)
+    cl = _c_arr(cache_len, np.int32)
+    out = np.empty((B, H * d), dtype=np.float32)
+    acc = None
+    if want_acc:
+        acc = np.zeros((B, H, Lmax), dtype=np.int32 if dtype == I8 else np.float32)
+    if n_threads <= 0:
+        n_threads = L.tso_max_threads()
+    L.tso_decode(dtype, B, H, d, _p(q), _p(qs), qc, _p(k_cache), _p(v_cache), H * Lmax * d, Lmax * d, d,
+                 _p(ks), _p(vs), H * Lmax, Lmax, kc, vc, _p(cl), int(window), float(slope),
+                 int(exp2_mode), int(bool(use_simd)), _p(out), _p(acc), Lmax, n_threads)
+    return (out, acc) if want_acc else out
+
+
+def softmax_buf(logits, exp2_mode):
+    L = lib()
+    x = _c_arr(logits, np.float32)
+    w = np.empty_like(x)
+    scale = L.tso_softmax_buf(_p(x), x.size, int(exp2_mode), _p(w))
+    return w, np.float32(scale)
+
+
+def simd_level():
+    return lib().tso_simd_level()
+
+
+def max_threads():
+    return lib().tso_max_threads()

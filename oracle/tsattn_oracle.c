@@ -1,0 +1,701 @@
+/*
+ * tsattn_oracle.c -- CPU restatement of TScale's attention arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY (see tsattn_oracle.h).  Nothing in the product library depends on
+ * this file; it exists so that the HIP kernels can be compared with the reference algorithm on
+ * identical inputs, and so that the same algorithm can be timed on host cores.
+ *
+ * Reference lines restated (paths relative to the reference's code/ directory) and how each
+ * function is pinned by tests/test_oracle_*.py:
+ *
+ *   tso_e4m3_to_float      util/fp8.h:4-21               pinned: all 256 codes against the OCP e4m3fn
+ *                                                         table built from first principles and
+ *                                                         against torch.float8_e4m3fn
+ *   tso_float_to_e4m3      util/fp8.h:48-60 (cvt.rn.satfinite)  pinned: round trip of all codes, ties
+ *                                                         between neighbours go to even, saturation,
+ *                                                         and torch's float8_e4m3fn cast on a dense sweep
+ *   tso_float_to_i8        train/cpu_infer.cpp:88-92     pinned: ties-to-even and clamp cases
+ *   tso_quantize_rows      lib/cuda/cuda_matmul.cuh:237-249, cuda_util.cuh:290-297
+ *                                                         pinned: numpy restatement + absmax row maps
+ *                                                         to +-127 / +-256
+ *   tso_make_spans         att/sliding_window.cpp:80-87,150-154,205-223,253-290
+ *                                                         pinned: brute-force enumeration of allowed
+ *                                                         (from,to) pairs
+ *   tso_init_alibi         model_params/model_dim.cpp:55-97   pinned: doc/model.md layer pattern
+ *   tso_dot_i8(_simd)      train/cpu_infer.cpp:184-210   pinned: int64 brute force, extreme values
+ *   tso_dot_e4m3           (exact-sum definition)        pinned: Fraction arithmetic in Python
+ *   tso_prefill_f32        compute/gpt_cpu.cpp:374-441   pinned: closed forms (equal logits, single
+ *                                                         key, empty row, ALiBi geometric series),
+ *                                                         textbook softmax with an extra zero key
+ *   tso_prefill_q8         same + cpu_infer.cpp:448,454  pinned: equals tso_prefill_f32 on dequantised
+ *                                                         inputs; scale-shift invariance
+ *   tso_decode             train/cpu_infer.cpp:413-460   pinned: equals prefill row t on cache [0..t]
+ *   tso_softmax_buf        train/cpu_infer.cpp:220-281   pinned: against exp2 in double, |rel| < 1e-5
+ *
+ * The reference holds no golden vectors or known-answer tests for this path, and the two files
+ * that contain it (gpt_cpu.cpp, cpu_infer.cpp) cannot be compiled without the CUDA SDK, so the
+ * pins above are mathematical ones.
+ */
+#include "tsattn_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#if defined(__x86_64__)
+#include <immintrin.h>
+#endif
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* model_params/model_dim.h:19-31 */
+#define TS_LOG2 0.693147f
+#define TS_ATT_DOTPRODUCT_SCALE 0.5f
+
+float tso_att_dot_scale(int head_dim)
+{
+    float dot_scale = sqrtf(1.0f / (float)head_dim);          /* CalcDotScale */
+    float att_mult = TS_ATT_DOTPRODUCT_SCALE / TS_LOG2;       /* CalcAttentionMult */
+    return dot_scale * att_mult;                              /* gpt_cpu.cpp:376 */
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* element formats                                                                            */
+
+float tso_e4m3_to_float(uint8_t x)
+{
+    /* util/fp8.h:4-21: bias 7, 3 mantissa bits, subnormals at e==0, no infinities.  The reference
+     * decodes 0x7f/0xff as 480; OCP calls them NaN.  Quantised data never holds them. */
+    int e = (x >> 3) & 15;
+    int m = x & 7;
+    float sign = (x & 0x80) ? -1.0f : 1.0f;
+    if (e == 0) {
+        return sign * ldexpf((float)m, -9);
+    }
+    return sign * ldexpf(1.0f + (float)m * 0.125f, e - 7);
+}
+
+uint8_t tso_float_to_e4m3(float x)
+{
+    uint8_t sign = signbit(x) ? 0x80 : 0;
+    float a = fabsf(x);
+    if (isnan(x)) {
+        return (uint8_t)(sign | 0x7f);
+    }
+    if (a >= 448.0f) {
+        return (uint8_t)(sign | 0x7e); /* satfinite */
+    }
+    if (a < ldexpf(1.0f, -6)) {
+        /* subnormal range: step 2^-9, 8 steps reach the first normal */
+        int q = (int)nearbyintf(ldexpf(a, 9)); /* default rounding mode = nearest even */
+        return (uint8_t)(sign | q);             /* q == 8 encodes as e=1,m=0 automatically */
+    }
+    int e;
+    (void)frexpf(a, &e); /* a = f * 2^e, f in [0.5,1) -> floor(log2 a) = e-1 */
+    e -= 1;
+    int q = (int)nearbyintf(ldexpf(a, 3 - e)); /* in [8,16] */
+    if (q == 16) {
+        q = 8;
+        e += 1;
+    }
+    int code = ((e + 7) << 3) | (q - 8);
+    if (code > 0x7e) {
+        code = 0x7e;
+    }
+    return (uint8_t)(sign | code);
+}
+
+int8_t tso_float_to_i8(float x)
+{
+    /* cpu_infer.cpp:88-92: _mm_cvtss_si32 (nearest even) then clamp to [-127,127] */
+    float r = nearbyintf(x);
+    if (!(r <= 127.0f)) {
+        r = (r != r) ? 0.0f : 127.0f;
+    }
+    if (r < -127.0f) {
+        r = -127.0f;
+    }
+    return (int8_t)(int)r;
+}
+
+float tso_bf16_to_float(uint16_t x)
+{
+    uint32_t u = (uint32_t)x << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+uint16_t tso_float_to_bf16(float x)
+{
+    uint32_t u;
+    memcpy(&u, &x, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return (uint16_t)((u >> 16) | 0x40);
+    }
+    uint32_t lsb = (u >> 16) & 1;
+    u += 0x7fffu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* absmax row quantiser                                                                       */
+
+static void quantize_head_row(int dtype, const float *x, int head_dim, uint8_t *q, float *scale)
+{
+    /* cuda_matmul.cuh:237-249: maxVal = max |x|; discrScale = maxVal/127 (i8) or /256 (e4m3);
+     * values multiplied by 1/discrScale and converted round-to-nearest.  All-zero row: scale 0. */
+    float max_val = 0;
+    for (int i = 0; i < head_dim; ++i) {
+        max_val = fmaxf(max_val, fabsf(x[i]));
+    }
+    float discr = 0;
+    float mult = 0;
+    if (max_val > 0) {
+        discr = (dtype == TSO_I8) ? max_val / 127 : max_val / 256;
+        mult = 1 / discr;
+    }
+    for (int i = 0; i < head_dim; ++i) {
+        float y = x[i] * mult;
+        q[i] = (dtype == TSO_I8) ? (uint8_t)tso_float_to_i8(y) : tso_float_to_e4m3(y);
+    }
+    *scale = discr;
+}
+
+void tso_quantize_rows(int dtype, const float *x, int64_t x_pitch, int64_t n_rows, int n_heads,
+                       int head_dim, uint8_t *q, int64_t q_pitch, float *scale, int64_t scale_pitch)
+{
+    for (int64_t t = 0; t < n_rows; ++t) {
+        for (int h = 0; h < n_heads; ++h) {
+            quantize_head_row(dtype, x + t * x_pitch + (int64_t)h * head_dim, head_dim,
+                              q + t * q_pitch + (int64_t)h * head_dim, scale + h * scale_pitch + t);
+        }
+    }
+}
+
+void tso_quantize_rows_bf16(int dtype, const uint16_t *x, int64_t x_pitch, int64_t n_rows,
+                            int n_heads, int head_dim, uint8_t *q, int64_t q_pitch, float *scale,
+                            int64_t scale_pitch)
+{
+    float *tmp = (float *)malloc(sizeof(float) * (size_t)head_dim);
+    for (int64_t t = 0; t < n_rows; ++t) {
+        for (int h = 0; h < n_heads; ++h) {
+            const uint16_t *src = x + t * x_pitch + (int64_t)h * head_dim;
+            for (int i = 0; i < head_dim; ++i) {
+                tmp[i] = tso_bf16_to_float(src[i]);
+            }
+            quantize_head_row(dtype, tmp, head_dim, q + t * q_pitch + (int64_t)h * head_dim,
+                              scale + h * scale_pitch + t);
+        }
+    }
+    free(tmp);
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* spans and layer schedule                                                                   */
+
+void tso_make_spans(int64_t n_seq, const int64_t *seq_offset, const uint8_t *doc_start_flag,
+                    int64_t window, int32_t *span_start, int32_t *span_finish)
+{
+    for (int64_t s = 0; s < n_seq; ++s) {
+        int64_t ptr = seq_offset[s];                 /* sliding_window.cpp:260, span.Shift(ptr) :279 */
+        int64_t len = seq_offset[s + 1] - ptr;
+        int64_t doc_start = 0;                       /* :142 */
+        for (int64_t t = 0; t < len; ++t) {
+            if (doc_start_flag && t > 0 && doc_start_flag[ptr + t]) {
+                doc_start = t;                       /* :150-154 */
+            }
+            int64_t a, b;
+            if (window == 0) {
+                a = t;                               /* :213-216 self attention */
+                b = t;
+            } else {
+                a = (doc_start > t - window) ? doc_start : t - window; /* :82 */
+                b = t - 1;                                             /* :83, finishOffset = 1 */
+                if (b < a) {                                           /* :84 span omitted */
+                    a = t;
+                    b = t - 1;
+                }
+            }
+            span_start[ptr + t] = (int32_t)(a + ptr);
+            span_finish[ptr + t] = (int32_t)(b + ptr);
+        }
+    }
+}
+
+int tso_init_alibi(int depth, int64_t wide_window, int max_layers, int64_t *width, float *slope)
+{
+    int n = 0;
+    if (depth == 1) {                                /* model_dim.cpp:60-64 */
+        if (max_layers < 1) return 0;
+        width[0] = wide_window;
+        slope[0] = 0.1f;
+        return 1;
+    }
+    if (depth <= 0) {
+        return 0;
+    }
+    /* ALIBI_V3, model_dim.cpp:73-92: widths {0,1,64,wide}; ids 1,1 then alternating 2(0.5),3(0) */
+    int group_count = (depth + 1) / 2;
+    int w1count = group_count / 6;
+    if (w1count < 1) w1count = 1;
+    for (int k = 0; k < w1count && n + 2 <= max_layers; ++k) {
+        width[n] = 1; slope[n] = 0; ++n;
+        width[n] = 1; slope[n] = 0; ++n;
+    }
+    for (int k = w1count; k < group_count && n + 2 <= max_layers; ++k) {
+        width[n] = 64; slope[n] = 0.5f; ++n;
+        width[n] = wide_window; slope[n] = 0; ++n;
+    }
+    return n;
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* dot products                                                                               */
+
+int32_t tso_dot_i8(const int8_t *a, const int8_t *b, int n)
+{
+    int32_t sum = 0;
+    for (int i = 0; i < n; ++i) {
+        sum += (int32_t)a[i] * (int32_t)b[i];
+    }
+    return sum;
+}
+
+#if defined(__x86_64__)
+static inline int32_t hsum_epi32(__m256i v)
+{
+    /* cpu_infer.cpp:164-182 */
+    __m128i lo = _mm256_castsi256_si128(v);
+    __m128i hi = _mm256_extracti128_si256(v, 1);
+    lo = _mm_add_epi32(lo, hi);
+    __m128i sh = _mm_shuffle_epi32(lo, _MM_SHUFFLE(0, 3, 2, 1));
+    lo = _mm_add_epi32(lo, sh);
+    sh = _mm_shuffle_epi32(lo, _MM_SHUFFLE(1, 0, 3, 2));
+    lo = _mm_add_epi32(lo, sh);
+    return _mm_extract_epi32(lo, 0);
+}
+
+__attribute__((target("avx2"))) static int32_t dot_i8_avx2(const int8_t *a, const int8_t *b, int n)
+{
+    /* the sign trick of cpu_infer.cpp:184-196 (|x| as the unsigned operand, y*sign(x) as the
+     * signed one); vpmaddubsw + vpmaddwd stand in for vpdpbusd.  |x|,|y| <= 127 keeps the
+     * 16-bit pair sums below saturation (2*127*127 = 32258). */
+    __m256i sum = _mm256_setzero_si256();
+    const __m256i ones = _mm256_set1_epi16(1);
+    for (int i = 0; i < n; i += 32) {
+        __m256i x = _mm256_loadu_si256((const __m256i *)(a + i));
+        __m256i y = _mm256_loadu_si256((const __m256i *)(b + i));
+        __m256i ax = _mm256_sign_epi8(x, x);
+        __m256i sy = _mm256_sign_epi8(y, x);
+        __m256i p16 = _mm256_maddubs_epi16(ax, sy);
+        sum = _mm256_add_epi32(sum, _mm256_madd_epi16(p16, ones));
+    }
+    return hsum_epi32(sum);
+}
+
+__attribute__((target("avx2,avxvnni"))) static int32_t dot_i8_avxvnni(const int8_t *a, const int8_t *b, int n)
+{
+    /* cpu_infer.cpp:184-210 with the same instruction (vpdpbusd, VEX form) */
+    __m256i sum = _mm256_setzero_si256();
+    for (int i = 0; i < n; i += 32) {
+        __m256i x = _mm256_loadu_si256((const __m256i *)(a + i));
+        __m256i y = _mm256_loadu_si256((const __m256i *)(b + i));
+        __m256i ax = _mm256_sign_epi8(x, x);
+        __m256i sy = _mm256_sign_epi8(y, x);
+        sum = _mm256_dpbusd_avx_epi32(sum, ax, sy);
+    }
+    return hsum_epi32(sum);
+}
+
+__attribute__((target("avx2,avx512f,avx512vl,avx512vnni"))) static int32_t dot_i8_avx512vnni(const int8_t *a, const int8_t *b, int n)
+{
+    /* same, EVEX-encoded vpdpbusd on 256-bit registers */
+    __m256i sum = _mm256_setzero_si256();
+    for (int i = 0; i < n; i += 32) {
+        __m256i x = _mm256_loadu_si256((const __m256i *)(a + i));
+        __m256i y = _mm256_loadu_si256((const __m256i *)(b + i));
+        __m256i ax = _mm256_sign_epi8(x, x);
+        __m256i sy = _mm256_sign_epi8(y, x);
+        sum = _mm256_dpbusd_epi32(sum, ax, sy);
+    }
+    return hsum_epi32(sum);
+}
+#endif
+
+static int g_simd_level = -1;
+
+int tso_simd_level(void)
+{
+    if (g_simd_level < 0) {
+        int lvl = 0;
+#if defined(__x86_64__)
+        __builtin_cpu_init();
+        if (__builtin_cpu_supports("avx2")) {
+            lvl = 1;
+            if (__builtin_cpu_supports("avx512vnni") && __builtin_cpu_supports("avx512vl")) {
+                lvl = 3;
+            } else if (__builtin_cpu_supports("avxvnni")) {
+                lvl = 2;
+            }
+        }
+#endif
+        g_simd_level = lvl;
+    }
+    return g_simd_level;
+}
+
+int32_t tso_dot_i8_simd(const int8_t *a, const int8_t *b, int n)
+{
+#if defined(__x86_64__)
+    if ((n & 31) == 0) {
+        switch (tso_simd_level()) {
+        case 3: return dot_i8_avx512vnni(a, b, n);
+        case 2: return dot_i8_avxvnni(a, b, n);
+        case 1: return dot_i8_avx2(a, b, n);
+        default: break;
+        }
+    }
+#endif
+    return tso_dot_i8(a, b, n);
+}
+
+static int32_t g_e4m3_fix[256]; /* value * 2^9 as an integer; every e4m3 value is a multiple of 2^-9 */
+static float g_e4m3_f32[256];
+static int g_e4m3_ready = 0;
+
+static void e4m3_tables(void)
+{
+    if (!g_e4m3_ready) {
+        for (int i = 0; i < 256; ++i) {
+            float f = tso_e4m3_to_float((uint8_t)i);
+            g_e4m3_f32[i] = f;
+            g_e4m3_fix[i] = (int32_t)ldexpf(f, 9);
+        }
+        g_e4m3_ready = 1;
+    }
+}
+
+float tso_dot_e4m3(const uint8_t *a, const uint8_t *b, int n)
+{
+    e4m3_tables();
+    int64_t sum = 0; /* products are multiples of 2^-18, |sum| < 2^43 for n <= 4096: exact */
+    for (int i = 0; i < n; ++i) {
+        sum += (int64_t)g_e4m3_fix[a[i]] * (int64_t)g_e4m3_fix[b[i]];
+    }
+    return (float)ldexp((double)sum, -18); /* one rounding, to nearest even */
+}
+
+void tso_qk_accum(int dtype, const uint8_t *q, int64_t q_pitch, const uint8_t *k, int64_t k_pitch,
+                  int head, int head_dim, int64_t from0, int64_t n_from, int64_t to0, int64_t n_to,
+                  void *acc)
+{
+    int64_t off = (int64_t)head * head_dim;
+    for (int64_t i = 0; i < n_from; ++i) {
+        for (int64_t j = 0; j < n_to; ++j) {
+            const uint8_t *qa = q + (from0 + i) * q_pitch + off;
+            const uint8_t *kb = k + (to0 + j) * k_pitch + off;
+            if (dtype == TSO_I8) {
+                ((int32_t *)acc)[i * n_to + j] = tso_dot_i8((const int8_t *)qa, (const int8_t *)kb, head_dim);
+            } else {
+                ((float *)acc)[i * n_to + j] = tso_dot_e4m3(qa, kb, head_dim);
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* prefill, fp32 inputs (compute/gpt_cpu.cpp:374-441)                                         */
+
+static float calc_dp_f32(const float *qk, const float *qv, int64_t pitch, int head_q_dim, int64_t q_offset,
+                         int64_t from, int64_t to, float att_dot_scale, float alibi_slope)
+{
+    /* gpt_cpu.cpp:379-389 */
+    float sum = 0;
+    for (int x = 0; x < head_q_dim; ++x) {
+        sum += qk[from * pitch + q_offset + x] * qv[to * pitch + q_offset + x];
+    }
+    float dp = sum * att_dot_scale;
+    dp += -(alibi_slope) * (float)(from - to); /* GetAttentionDecay, model_dim.h:33 */
+    return dp;
+}
+
+void tso_prefill_f32(int64_t len, int n_heads, int q_dim, int tt_dim, const float *qk,
+                     const float *qv, const float *v, const int32_t *span_ptr,
+                     const int32_t *spans, float alibi_slope, float *out, float *sum_weight,
+                     float *max_dp_out)
+{
+    float att_dot_scale = tso_att_dot_scale(q_dim);
+    int64_t q_pitch = (int64_t)n_heads * q_dim;
+    int64_t tt_pitch = (int64_t)n_heads * tt_dim;
+    float *val = (float *)malloc(sizeof(float) * (size_t)tt_dim);
+    for (int head = 0; head < n_heads; ++head) {
+        int64_t q_offset = (int64_t)head * q_dim;
+        int64_t tt_offset = (int64_t)head * tt_dim;
+        for (int64_t from = 0; from < len; ++from) {
+            float max_dp = 0; /* :410 the zero vector's logit takes part in the max */
+            for (int32_t ai = span_ptr[from]; ai < span_ptr[from + 1]; ++ai) {
+                for (int64_t to = spans[2 * ai]; to <= spans[2 * ai + 1]; ++to) {
+                    float dp = calc_dp_f32(qk, qv, q_pitch, q_dim, q_offset, from, to, att_dot_scale, alibi_slope);
+                    max_dp = fmaxf(max_dp, dp);
+                }
+            }
+            float sw = exp2f(-max_dp); /* :419 zero vector of weight 1 */
+            memset(val, 0, sizeof(float) * (size_t)tt_dim);
+            for (int32_t ai = span_ptr[from]; ai < span_ptr[from + 1]; ++ai) {
+                for (int64_t to = spans[2 * ai]; to <= spans[2 * ai + 1]; ++to) {
+                    float dp = calc_dp_f32(qk, qv, q_pitch, q_dim, q_offset, from, to, att_dot_scale, alibi_slope);
+                    float w = exp2f(dp - max_dp);
+                    sw += w;
+                    for (int x = 0; x < tt_dim; ++x) {
+                        val[x] += w * v[to * tt_pitch + tt_offset + x];
+                    }
+                }
+            }
+            if (sum_weight) sum_weight[(int64_t)head * len + from] = sw;
+            if (max_dp_out) max_dp_out[(int64_t)head * len + from] = max_dp;
+            float inv = 1 / sw;
+            for (int x = 0; x < tt_dim; ++x) {
+                out[from * tt_pitch + tt_offset + x] = val[x] * inv;
+            }
+        }
+    }
+    free(val);
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* prefill, 8-bit inputs with per-row scales                                                  */
+
+static inline float acc_to_float(int dtype, const uint8_t *a, const uint8_t *b, int d)
+{
+    if (dtype == TSO_I8) {
+        return (float)tso_dot_i8((const int8_t *)a, (const int8_t *)b, d);
+    }
+    return tso_dot_e4m3(a, b, d);
+}
+
+void tso_prefill_q8(int dtype, int64_t n_tokens, int n_heads, int head_dim, const uint8_t *q,
+                    const uint8_t *k, const uint8_t *v, int64_t pitch, const float *q_scale,
+                    const float *k_scale, const float *v_scale, int64_t scale_pitch,
+                    float q_scale_const, float k_scale_const, float v_scale_const,
+                    const int32_t *span_start, const int32_t *span_finish, float alibi_slope,
+                    float *out, int64_t out_pitch, float *sum_weight_log, int n_threads)
+{
+    e4m3_tables();
+    float att_dot_scale = tso_att_dot_scale(head_dim);
+    if (n_threads < 1) n_threads = 1;
+    int64_t n_jobs = (int64_t)n_heads * n_tokens;
+#pragma omp parallel num_threads(n_threads)
+    {
+        float *val = (float *)malloc(sizeof(float) * (size_t)head_dim);
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t job = 0; job < n_jobs; ++job) {
+            int head = (int)(job / n_tokens);
+            int64_t from = job % n_tokens;
+            int64_t off = (int64_t)head * head_dim;
+            const uint8_t *qrow = q + from * pitch + off;
+            float qs = q_scale ? q_scale[head * scale_pitch + from] : q_scale_const;
+            int64_t lo = span_start[from], hi = span_finish[from];
+            /* pass 1: maximum, the zero vector's logit 0 included (gpt_cpu.cpp:410-417) */
+            float max_dp = 0;
+            for (int64_t to = lo; to <= hi; ++to) {
+                float ks = k_scale ? k_scale[head * scale_pitch + to] : k_scale_const;
+                float acc = acc_to_float(dtype, qrow, k + to * pitch + off, head_dim);
+                float dp = acc * ks * att_dot_scale * qs - alibi_slope * (float)(from - to); /* cpu_infer.cpp:448 */
+                max_dp = fmaxf(max_dp, dp);
+            }
+            /* pass 2: weights and weighted values (gpt_cpu.cpp:419-431) */
+            float sw = exp2f(-max_dp);
+            memset(val, 0, sizeof(float) * (size_t)head_dim);
+            for (int64_t to = lo; to <= hi; ++to) {
+                float ks = k_scale ? k_scale[head * scale_pitch + to] : k_scale_const;
+                float vs = v_scale ? v_scale[head * scale_pitch + to] : v_scale_const;
+                float acc = acc_to_float(dtype, qrow, k + to * pitch + off, head_dim);
+                float dp = acc * ks * att_dot_scale * qs - alibi_slope * (float)(from - to);
+                float w = exp2f(dp - max_dp);
+                sw += w;
+                float wv = w * vs; /* cpu_infer.cpp:454: weight times value scale, then times the 8-bit value */
+                const uint8_t *vrow = v + to * pitch + off;
+                if (dtype == TSO_I8) {
+                    for (int x = 0; x < head_dim; ++x) {
+                        val[x] += wv * (float)(int8_t)vrow[x];
+                    }
+                } else {
+                    for (int x = 0; x < head_dim; ++x) {
+                        val[x] += wv * g_e4m3_f32[vrow[x]];
+                    }
+                }
+            }
+            float inv = 1 / sw;
+            for (int x = 0; x < head_dim; ++x) {
+                out[from * out_pitch + off + x] = val[x] * inv;
+            }
+            if (sum_weight_log) {
+                sum_weight_log[head * scale_pitch + from] = max_dp + log2f(sw); /* gpt_att_fp16.cuh:249 */
+            }
+        }
+        free(val);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* softmax buffer (train/cpu_infer.cpp:220-281)                                               */
+
+static float exp2_poly_lane(float x_minus_max)
+{
+    /* one lane of cpu_infer.cpp:254-275 */
+    float x = x_minus_max;
+    x = (x > -127.0f) ? x : -127.0f; /* _mm256_max_ps(x, -127): NaN in x yields -127 as well */
+    float xf = floorf(x);
+    x = x - xf;
+    int32_t xfi = (int32_t)nearbyintf(xf); /* cvtps_epi32 */
+    float x2 = x * x;
+    const float c0 = -3.069678791803394491901405992213472390777e-1f;
+    const float c1 = -6.558811624324781017147952441210509604385e-2f;
+    const float c2 = -1.355574723481491770403079319055785445381e-2f;
+    float res = fmaf(fmaf(c2, x, c1), x, c0);
+    float x_by_1_minus_x = x - x2;
+    res = fmaf(res, x_by_1_minus_x, x);
+    res = res + 1.0f;
+    int32_t bits;
+    memcpy(&bits, &res, 4);
+    bits += (int32_t)((uint32_t)xfi << 23);
+    memcpy(&res, &bits, 4);
+    return res;
+}
+
+static float hsum8(const float *x)
+{
+    /* sse_utils.h:208-230: (x0+x4)+(x2+x6) then + ((x1+x5)+(x3+x7)) */
+    float s0 = x[0] + x[4], s1 = x[1] + x[5], s2 = x[2] + x[6], s3 = x[3] + x[7];
+    float d0 = s0 + s2, d1 = s1 + s3;
+    return d0 + d1;
+}
+
+/* buf must hold ceil(n/8)*8 floats; entries beyond n are the -1e38 padding of TSoftMaxBuf.
+ * Overwrites buf with the un-normalised weights and returns Scale = 1/sum. */
+static float softmax_buf_inplace(float *buf, int n, float max_value, int exp2_mode)
+{
+    int groups = (n + 7) / 8;
+    if (exp2_mode == 1) {
+        float lane_sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int i = 0; i < groups; ++i) {
+            for (int j = 0; j < 8; ++j) {
+                float r = exp2_poly_lane(buf[i * 8 + j] - max_value);
+                buf[i * 8 + j] = r;
+                lane_sum[j] += r;
+            }
+        }
+        return 1 / hsum8(lane_sum);
+    }
+    float sum = 0;
+    for (int i = 0; i < n; ++i) {
+        float r = exp2f(buf[i] - max_value);
+        buf[i] = r;
+        sum += r;
+    }
+    return 1 / sum;
+}
+
+float tso_softmax_buf(const float *logits, int n, int exp2_mode, float *weights)
+{
+    int cap = ((n + 7) / 8) * 8;
+    if (cap < 8) cap = 8;
+    float *buf = (float *)malloc(sizeof(float) * (size_t)cap);
+    float max_value = 0; /* TSoftMaxBuf::Clear: MaxValue = 0 */
+    for (int i = 0; i < cap; ++i) buf[i] = -1e38f;
+    for (int i = 0; i < n; ++i) {
+        buf[i] = logits[i];
+        max_value = (max_value > logits[i]) ? max_value : logits[i];
+    }
+    float scale = softmax_buf_inplace(buf, n, max_value, exp2_mode);
+    for (int i = 0; i < n; ++i) weights[i] = buf[i] * scale;
+    free(buf);
+    return scale;
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* decode over a KV cache (train/cpu_infer.cpp:413-460)                                       */
+
+void tso_decode(int dtype, int64_t n_seq, int n_heads, int head_dim, const uint8_t *q,
+                const float *q_scale, float q_scale_const, const uint8_t *k, const uint8_t *v,
+                int64_t seq_stride, int64_t head_stride, int64_t tok_stride, const float *k_scale,
+                const float *v_scale, int64_t s_seq_stride, int64_t s_head_stride,
+                float k_scale_const, float v_scale_const, const int32_t *cache_len, int64_t window,
+                float alibi_slope, int exp2_mode, int use_simd, float *out, void *qk_acc,
+                int64_t qk_acc_pitch, int n_threads)
+{
+    e4m3_tables();
+    float att_dot_scale = tso_att_dot_scale(head_dim);
+    if (n_threads < 1) n_threads = 1;
+    int64_t n_jobs = n_seq * n_heads;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(n_threads)
+    for (int64_t job = 0; job < n_jobs; ++job) {
+        int64_t s = job / n_heads;
+        int head = (int)(job % n_heads);
+        int64_t cur = (int64_t)cache_len[s] - 1; /* :422 */
+        float *o = out + (s * n_heads + head) * head_dim;
+        for (int x = 0; x < head_dim; ++x) o[x] = 0;
+        if (cur < 0) {
+            continue;
+        }
+        /* :423-431 the key list: self only for width 0, else cur-1 ... cur-min(cur,width) */
+        int64_t to_count, to_first, to_step;
+        if (window == 0) {
+            to_count = 1; to_first = cur; to_step = 0;
+        } else {
+            to_count = (cur < window) ? cur : window; to_first = cur - 1; to_step = -1;
+        }
+        int cap = (int)(((to_count + 1 + 7) / 8) * 8);
+        float *buf = (float *)malloc(sizeof(float) * (size_t)cap);
+        for (int i = 0; i < cap; ++i) buf[i] = -1e38f;
+        const uint8_t *qrow = q + (s * n_heads + head) * head_dim;
+        float qs = q_scale ? q_scale[s * n_heads + head] : q_scale_const;
+        const uint8_t *kbase = k + s * seq_stride + head * head_stride;
+        const uint8_t *vbase = v + s * seq_stride + head * head_stride;
+        const float *ksb = k_scale ? k_scale + s * s_seq_stride + head * s_head_stride : NULL;
+        const float *vsb = v_scale ? v_scale + s * s_seq_stride + head * s_head_stride : NULL;
+        float max_value = 0;
+        buf[0] = 0; /* :444 softMax.Add(0) */
+        for (int64_t z = 0; z < to_count; ++z) {
+            int64_t to = to_first + z * to_step;
+            const uint8_t *krow = kbase + to * tok_stride;
+            float accf;
+            if (dtype == TSO_I8) {
+                int32_t acc = use_simd ? tso_dot_i8_simd((const int8_t *)qrow, (const int8_t *)krow, head_dim)
+                                       : tso_dot_i8((const int8_t *)qrow, (const int8_t *)krow, head_dim);
+                if (qk_acc) ((int32_t *)qk_acc)[(s * n_heads + head) * qk_acc_pitch + to] = acc;
+                accf = (float)acc;
+            } else {
+                accf = tso_dot_e4m3(qrow, krow, head_dim);
+                if (qk_acc) ((float *)qk_acc)[(s * n_heads + head) * qk_acc_pitch + to] = accf;
+            }
+            float ks = ksb ? ksb[to] : k_scale_const;
+            float logit = accf * ks * att_dot_scale * qs - alibi_slope * (float)(cur - to); /* :448 */
+            buf[z + 1] = logit;
+            max_value = (max_value > logit) ? max_value : logit;
+        }
+        float scale = softmax_buf_inplace(buf, (int)to_count + 1, max_value, exp2_mode); /* :450 */
+        for (int64_t z = 0; z < to_count; ++z) {
+            int64_t to = to_first + z * to_step;
+            float vs = vsb ? vsb[to] : v_scale_const;
+            float w = buf[z + 1] * scale * vs; /* :454 */
+            const uint8_t *vrow = vbase + to * tok_stride;
+            if (dtype == TSO_I8) {
+                for (int x = 0; x < head_dim; ++x) o[x] += w * (float)(int8_t)vrow[x];
+            } else {
+                for (int x = 0; x < head_dim; ++x) o[x] += w * g_e4m3_f32[vrow[x]];
+            }
+        }
+        free(buf);
+    }
+}
+
+int tso_max_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
