@@ -1,0 +1,180 @@
+/*
+ * tsattn.h -- C ABI of the MI355X (gfx950) implementation of TScale's quantized attention.
+ *
+ * Plain C: pointers, sizes and a stream handle; no C++ or framework types cross this boundary.
+ * All data pointers are DEVICE pointers unless stated otherwise.  Every call that takes a stream is
+ * asynchronous on that stream (pass the hipStream_t as void*, NULL = the default stream), never
+ * synchronises, never allocates and never reads device data on the host, so it can be captured
+ * into a HIP graph.  A handle belongs to one device and one host thread at a time.
+ *
+ * Reference lines are given relative to the reference's code/ directory.
+ *
+ * Attention definition (per sequence, head, query row `from`):
+ *     keys   to in [span_start[from], span_finish[from]]   (inclusive; finish < start = no keys)
+ *     acc    = sum_x q[from][x] * k[to][x]                 (int8: exact int32; e4m3: fp32 MFMA sum)
+ *     dp     = acc * ks[to] * sqrtf(1/d)*(0.5f/0.693147f) * qs[from] - slope * (from - to)
+ *     m      = max(0, max_to dp)                           (a zero vector of logit 0 always takes part)
+ *     l      = exp2(-m) + sum_to exp2(dp - m)
+ *     out[x] = sum_to exp2(dp - m) * vs[to] * v[to][x] / l
+ *     sum_weight_log = m + log2(l)
+ */
+#ifndef TSATTN_H
+#define TSATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tsattn_ctx *tsattn_handle_t;
+
+enum tsattn_status {
+    TSATTN_OK = 0,
+    TSATTN_ERR_BAD_ARG = 1,     /* null pointer, negative size, misaligned pitch */
+    TSATTN_ERR_UNSUPPORTED = 2, /* head_dim other than 64/128, unknown dtype */
+    TSATTN_ERR_HIP = 3,         /* the HIP runtime reported an error; see tsattn_last_error */
+    TSATTN_ERR_SCRATCH = 4      /* sizes exceed what the handle was created for */
+};
+
+enum tsattn_dtype { TSATTN_I8 = 0, TSATTN_E4M3 = 1 };               /* Q/K/V element type */
+enum tsattn_out_dtype { TSATTN_OUT_F32 = 0, TSATTN_OUT_F16 = 1 };   /* prefill output type */
+enum tsattn_src_dtype { TSATTN_SRC_F32 = 0, TSATTN_SRC_BF16 = 1 };  /* quantiser input type */
+enum tsattn_q_dtype { TSATTN_Q_8BIT = 0, TSATTN_Q_BF16 = 1 };       /* decode query type */
+
+/* Sizes the handle's one-time scratch is provisioned for (decode split partials). */
+typedef struct tsattn_config {
+    int device;            /* HIP device ordinal */
+    int max_seqs;          /* decode: sequences per call */
+    int max_heads;
+    int max_head_dim;      /* 64 or 128 */
+    int max_splits;        /* decode: KV splits per (sequence, head); 0 = library default */
+} tsattn_config;
+
+/* Context lifetime.  Replaces the per-context arena of the reference
+ * (TAttentionComputeCtx::AllocateCuda, gpt/compute/gpt_cuda.cu:231-302): the only allocation the
+ * library ever makes happens in tsattn_create. */
+size_t tsattn_scratch_bytes(const tsattn_config *cfg);
+int tsattn_create(const tsattn_config *cfg, tsattn_handle_t *out);
+int tsattn_destroy(tsattn_handle_t h);
+/* Text of the last error on the calling thread (never NULL).  The reference aborts instead
+ * (Y_VERIFY, util/eden_core.h:111). */
+const char *tsattn_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Prefill.  Replaces
+ *   GPU: CudaCall(c, Fp8Att)...(scaleQV, QK, QV, QVscale)(VT)(AttSpans, AttSpanPtr, AlibiSlope)
+ *        .Write(&ValLookup, &SumWeightLog)              gpt/compute/gpt_cuda.cu:503-507
+ *        and the Fp16Att int8 variant                    gpt/compute/gpt_cuda.cu:511-515
+ *        (kernels gpt/compute/gpt_att_fp8.cuh:43-248, gpt_att_fp16.cuh:120-318)
+ *   CPU: TAttentionComputer::ComputeValLookup            gpt/compute/gpt_cpu.cpp:391-441, call :633
+ * Unlike Fp8Att, V is taken in the same [token][head*d] layout as Q and K: no transposed copy
+ * (gpt_cuda.cu:501) is needed.
+ */
+typedef struct tsattn_prefill_args {
+    int dtype;                 /* tsattn_dtype of q, k, v */
+    int out_dtype;             /* tsattn_out_dtype */
+    int64_t n_tokens;          /* all sequences of the batch concatenated */
+    int n_heads;
+    int head_dim;              /* 64 or 128 */
+    const void *q, *k, *v;     /* [n_tokens][n_heads*head_dim] 8-bit */
+    int64_t q_pitch, k_pitch, v_pitch;   /* row pitch in bytes, multiple of 16 */
+    const float *q_scale, *k_scale, *v_scale; /* [n_heads][n_tokens] or NULL = the constant below */
+    int64_t scale_pitch;       /* floats between heads */
+    float q_scale_const, k_scale_const, v_scale_const;
+    const float *k_global_scale; /* optional device float multiplied into every key scale
+                                    (the QV matrix scale, gpt_cuda.cu:476) */
+    const int32_t *span_start;   /* [n_tokens] inclusive first key of each row */
+    const int32_t *span_finish;  /* [n_tokens] inclusive last key; < start = row sees no key */
+    float alibi_slope;
+    void *out;                   /* [n_tokens][n_heads*head_dim] f32 or f16 */
+    int64_t out_pitch;           /* bytes */
+    float *sum_weight_log;       /* optional [n_heads][n_tokens] (pitch scale_pitch) */
+    void *debug_qk_acc;          /* optional raw QK^T accumulators, [n_heads][n_tokens][debug_pitch]
+                                    int32 (int8 inputs) or f32 (e4m3); only in-span pairs are written */
+    int64_t debug_pitch;         /* elements per (head, from) row of debug_qk_acc */
+} tsattn_prefill_args;
+
+int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Decode of one new token per sequence over a KV cache.  Replaces
+ *   ComputeValLookup(att.AttentionWidth, att.AlibiSlope, dims, kvCache, qk, &valLookup)
+ *                                                        gpt/train/cpu_infer.cpp:413-460, call :509
+ * The cache is planar: element (seq, head, to, x) lives at
+ *   cache + seq*seq_stride + head*head_stride + to*tok_stride + x      (bytes)
+ * and its row scale at  scale + seq*s_seq_stride + head*s_head_stride + to   (floats).
+ * cache_len[seq] counts valid rows INCLUDING the current token, which the caller appended first
+ * (cpu_infer.cpp:506); the token attends to rows cache_len-2 ... cache_len-1-min(cache_len-1, window),
+ * or to itself only when window == 0 (cpu_infer.cpp:423-431).
+ */
+typedef struct tsattn_decode_args {
+    int dtype;                 /* tsattn_dtype of the cache (and of q when q_dtype == TSATTN_Q_8BIT) */
+    int q_dtype;               /* tsattn_q_dtype; BF16 queries are quantised per head with the absmax
+                                  rule (scale = absmax/127 or /256) before the dot products */
+    int n_seqs, n_heads, head_dim;
+    const void *q;             /* [n_seqs][n_heads*head_dim] */
+    int64_t q_pitch;           /* bytes per sequence */
+    const float *q_scale;      /* [n_seqs][n_heads] or NULL = constant; ignored for BF16 queries */
+    float q_scale_const;
+    const void *k_cache, *v_cache;
+    int64_t seq_stride, head_stride, tok_stride; /* bytes; tok_stride multiple of 16 */
+    const float *k_scale, *v_scale;              /* NULL = constant */
+    int64_t s_seq_stride, s_head_stride;         /* floats */
+    float k_scale_const, v_scale_const;
+    const int32_t *cache_len;  /* device [n_seqs] */
+    int max_len;               /* host-side upper bound of cache_len (sizes the grid) */
+    int64_t window;
+    float alibi_slope;
+    float *out;                /* [n_seqs][n_heads*head_dim] f32 */
+    int n_splits;              /* KV splits per (seq, head); 0 = choose from max_len */
+    void *debug_qk_acc;        /* optional [n_seqs][n_heads][debug_pitch] int32 / f32 */
+    int64_t debug_pitch;
+} tsattn_decode_args;
+
+int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream);
+
+/* Append one token per sequence to the cache at row cache_len[seq], then increment cache_len[seq]
+ * on the device.  Replaces TAttentionVecHistory::AddVectors, gpt/train/cpu_infer.cpp:403-408
+ * (call :506).  k_new, v_new: [n_seqs][n_heads*head_dim] 8-bit; *_scale_new: [n_seqs][n_heads]. */
+typedef struct tsattn_append_args {
+    int n_seqs, n_heads, head_dim;
+    const void *k_new, *v_new;
+    int64_t new_pitch;         /* bytes per sequence */
+    const float *k_scale_new, *v_scale_new; /* NULL = leave the scale planes untouched */
+    void *k_cache, *v_cache;
+    int64_t seq_stride, head_stride, tok_stride;
+    float *k_scale, *v_scale;
+    int64_t s_seq_stride, s_head_stride;
+    int32_t *cache_len;        /* device [n_seqs], updated in place */
+    int max_len;               /* rows per (seq, head) plane; a full cache is left unchanged */
+} tsattn_append_args;
+
+int tsattn_cache_append(tsattn_handle_t h, const tsattn_append_args *a, void *stream);
+
+/* Per-(row, head) absmax quantiser: scale = absmax/127 (int8) or absmax/256 (e4m3), values
+ * round-to-nearest-even, int8 clamped to [-127,127].  Replaces NormalizeVecsRowTileMax /
+ * TStoreRowTileMaxNormalize (gpt/compute/row_tile_scale.cuh:59-81, lib/cuda/cuda_matmul.cuh:207-260,
+ * lib/cuda/cuda_util.cuh:286-297).  src: [n_rows][n_heads*head_dim] f32 or bf16;
+ * scale written to scale[head*scale_pitch + row]. */
+int tsattn_quantize_rows(tsattn_handle_t h, int src_dtype, int dst_dtype, const void *src,
+                         int64_t src_pitch, int64_t n_rows, int n_heads, int head_dim, void *dst,
+                         int64_t dst_pitch, float *scale, int64_t scale_pitch, void *stream);
+
+/* Window metadata on the device: one inclusive key span per token from the window width, the
+ * sequence boundaries and optional in-sequence document starts.  Replaces the host-side span
+ * emission of GenerateAttentionGraph / AddAttSpans (gpt/att/sliding_window.cpp:80-87,150-154,
+ * 205-223) and the fragment shift of InitLabelData (:253-290).  seq_offset: device int32
+ * [n_seqs+1] first token of each sequence; doc_start_flag: optional device uint8 [n_tokens]. */
+int tsattn_build_spans(tsattn_handle_t h, int n_seqs, const int32_t *seq_offset, int64_t n_tokens,
+                       const uint8_t *doc_start_flag, int64_t window, int32_t *span_start,
+                       int32_t *span_finish, void *stream);
+
+/* Library build identification (kernel set and target), for logs. */
+const char *tsattn_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,152 @@
+"""GPU: MFMA prefill through the C ABI against the prefill oracle (compute/gpt_cpu.cpp:391-441 with
+8-bit operands).  int8 QK^T accumulators bit-exact; e4m3 accumulators within a few fp32 ulps of the
+exact sum; outputs within max-abs 2e-2 / mean-abs 2e-3 on unit-variance outputs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import pyoracle as orc
+from tests.common import assert_within_tolerance, make_qkv
+from tscale_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from tscale_amd import AttentionContext
+    c = AttentionContext(0, max_seqs=1, max_heads=16, max_head_dim=128)
+    yield c
+    c.close()
+
+
+def run_gpu(ctx, dtype, H, q, qs, k, ks, v, vs, st, fi, slope, out_f16=False, want_acc=False, want_swl=False):
+    n = q.shape[0]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    sc = lambda s: t(s) if isinstance(s, np.ndarray) else s
+    dbg = None
+    if want_acc:
+        dbg = torch.zeros((H, n, n), dtype=torch.int32 if dtype == capi.I8 else torch.float32, device="cuda")
+        dbg = dbg.view(H * n, n).unsqueeze(0)[0].view(H, n, n)
+    swl = torch.zeros((H, n), dtype=torch.float32, device="cuda") if want_swl else None
+    out = ctx.compute_val_lookup(dtype, H, t(q), t(k), t(v), sc(qs), sc(ks), sc(vs), t(st), t(fi), slope,
+                                 out_f16=out_f16, sum_weight_log=swl,
+                                 debug_qk_acc=None if dbg is None else dbg.view(H * n, n).view(H, n, n))
+    torch.cuda.synchronize()
+    res = [out.float().cpu().numpy()]
+    if want_acc:
+        res.append(dbg.cpu().numpy())
+    if want_swl:
+        res.append(swl.cpu().numpy())
+    return res if len(res) > 1 else res[0]
+
+
+@pytest.mark.parametrize("dtype", [capi.I8, capi.E4M3])
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("window,slope", [(10 ** 6, 0.0), (64, 0.5), (0, 0.0), (1, 0.0), (256, 0.5)])
+def test_prefill_parity_small(ctx, dtype, d, window, slope):
+    H = 2
+    seq_lens = [300, 1, 129, 70]  # ragged: sequence boundaries inside query tiles
+    n = sum(seq_lens)
+    q, qs, k, ks, v, vs = make_qkv(50 + d, n, H, d, dtype)
+    st, fi = orc.make_spans(seq_lens, window)
+    want, want_swl = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, slope, want_swl=True)
+    out, acc, swl = run_gpu(ctx, dtype, H, q, qs, k, ks, v, vs, st, fi, slope, want_acc=True, want_swl=True)
+    for h in range(H):
+        for f in range(0, n, 7):
+            if fi[f] < st[f]:
+                continue
+            ref = orc.qk_accum(dtype, q, k, h, d, f, 1, int(st[f]), int(fi[f] - st[f] + 1))[0]
+            got = acc[h, f, st[f]:fi[f] + 1]
+            if dtype == capi.I8:
+                assert np.array_equal(got, ref), "int32 QK^T accumulators differ"
+            else:
+                # v_mfma_f32_32x32x64_f8f6f4 aligns the 64 products of a step to their largest exponent and
+                # keeps fewer bits than fp32 there: the error is relative to the largest product a row pair
+                # can hold (256*256 after absmax scaling), not to the sum.  2^-12 of that, measured ~2^-13.
+                assert np.all(np.abs(got - ref) <= 2.0 ** -12 * 65536.0 + 2.0 ** -12 * np.abs(ref))
+    assert_within_tolerance(out, want, "prefill")
+    assert np.abs(swl - want_swl).max() < 1e-3
+    empty = fi < st
+    assert not out[empty].any()
+
+
+@pytest.mark.parametrize("dtype", [capi.I8, capi.E4M3])
+def test_prefill_doc_boundaries_and_f16_out(ctx, dtype):
+    H, d = 3, 128
+    seq_lens = [513, 255]
+    n = sum(seq_lens)
+    flags = (np.random.default_rng(2).random(n) < 0.01).astype(np.uint8)
+    q, qs, k, ks, v, vs = make_qkv(61, n, H, d, dtype)
+    st, fi = orc.make_spans(seq_lens, 10 ** 6, flags)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, 0.0)
+    out = run_gpu(ctx, dtype, H, q, qs, k, ks, v, vs, st, fi, 0.0, out_f16=True)
+    assert_within_tolerance(out, want, "prefill f16 out")
+
+
+def test_prefill_mask_probe_one_hot_values(ctx):
+    """V = one-hot(to) makes the output equal to the weight vector: pins which keys each row sees."""
+    H, d, n = 1, 128, 128
+    rng = np.random.default_rng(3)
+    q = rng.integers(-20, 21, (n, d)).astype(np.int8).view(np.uint8)
+    k = rng.integers(-20, 21, (n, d)).astype(np.int8).view(np.uint8)
+    v = np.eye(n, d, dtype=np.int8).view(np.uint8)  # key t has value e_t (t < 128)
+    for window in (0, 1, 5, 64, 1000):
+        st, fi = orc.make_spans([70, 58], window)
+        out = run_gpu(ctx, capi.I8, H, q, 0.01, k, 0.02, v, 1.0, st, fi, 0.25)
+        for f in range(n):
+            seen = set(np.nonzero(out[f] > 0)[0].tolist())
+            assert seen == set(range(st[f], fi[f] + 1)), (window, f)
+
+
+def test_prefill_constant_scales_and_global_key_scale(ctx):
+    H, d, n = 2, 128, 200
+    rng = np.random.default_rng(4)
+    q, k, v = (rng.integers(-127, 128, (n, H * d)).astype(np.int8).view(np.uint8) for _ in range(3))
+    ks = (rng.random((H, n)).astype(np.float32) + 0.5) / 24
+    VEC = 1.0 / 24
+    st, fi = orc.make_spans([n], 64)
+    want = orc.prefill_q8(orc.I8, q, k, v, H, VEC, ks * np.float32(0.37), VEC, st, fi, 0.5)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    out = ctx.compute_val_lookup(capi.I8, H, t(q), t(k), t(v), VEC, t(ks), VEC, t(st), t(fi), 0.5,
+                                 k_global_scale=torch.tensor([0.37], device="cuda")).cpu().numpy()
+    assert_within_tolerance(out, want, "constant scales")
+
+
+@pytest.mark.parametrize("dtype,B,S,H,d,window,slope", [
+    (capi.I8, 1, 1024, 12, 64, 1024, 0.0),     # the CPU-reference configuration, full size
+    (capi.E4M3, 2, 1024, 12, 64, 64, 0.5),     # 125M-style short-window layer, reduced batch
+    (capi.E4M3, 2, 1024, 12, 64, 1024, 0.0),   # 125M-style wide layer, reduced batch
+    (capi.E4M3, 1, 2048, 4, 128, 256, 0.5),    # 1.5B-style layers, reduced batch / heads / length
+    (capi.E4M3, 1, 2048, 4, 128, 2048, 0.0),
+])
+def test_prefill_parity_benchmark_shapes(ctx, dtype, B, S, H, d, window, slope):
+    n = B * S
+    q, qs, k, ks, v, vs = make_qkv(1313, n, H, d, dtype)
+    st, fi = orc.make_spans([S] * B, window)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, slope)
+    out = run_gpu(ctx, dtype, H, q, qs, k, ks, v, vs, st, fi, slope)
+    mx, mean = assert_within_tolerance(out, want, "benchmark shape")
+    print(f"unit-variance error: max {mx:.2e} mean {mean:.2e}")
+
+
+def test_prefill_full_size_properties(ctx):
+    """1.5B-style shape at full size (B8 S4096 H16 d128 e4m3): V = ones of scale 1 gives
+    out = 1 - 2^-sum_weight_log in every column, and row 0 of every sequence is zero."""
+    B, S, H, d = 8, 4096, 16, 128
+    n = B * S
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn((n, H * d), device="cuda", generator=g)
+    q, qs = ctx.quantize_rows(x, H, capi.E4M3)
+    k, ks = ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g), H, capi.E4M3)
+    v = torch.full((n, H * d), 0x38, dtype=torch.uint8, device="cuda")  # e4m3 1.0
+    off = torch.arange(0, n + 1, S, dtype=torch.int32, device="cuda")
+    st, fi = ctx.build_spans(off, n, S)
+    swl = torch.zeros((H, n), device="cuda")
+    out = ctx.compute_val_lookup(capi.E4M3, H, q, k, v, qs, ks, 1.0, st, fi, 0.0, sum_weight_log=swl)
+    torch.cuda.synchronize()
+    o = out.view(n, H, d)
+    assert (o[::S] == 0).all()
+    want = 1 - torch.exp2(-swl).t()
+    assert (o - want[:, :, None]).abs().max().item() < 2e-3
+    assert (o.max(dim=2).values - o.min(dim=2).values).max().item() < 1e-6

@@ -1,0 +1,170 @@
+"""Host-side mirror of the reference's attention call sites on top of the C ABI.
+
+`AttentionContext.compute_val_lookup` has the argument meaning of
+TAttentionComputer::ComputeValLookup (gpt/compute/gpt_cpu.cpp:391-441) / the Fp8Att launch
+(gpt/compute/gpt_cuda.cu:503-507); `AttentionContext.compute_val_lookup_decode` that of
+ComputeValLookup in gpt/train/cpu_infer.cpp:413-460 and `KVCache.add_vectors` that of
+TAttentionVecHistory::AddVectors (:403-408).  torch tensors are used for device memory only; all
+arithmetic happens in libtsattn.so.  There is no fallback path: a missing library raises.
+"""
+import ctypes
+
+import torch
+
+from . import capi
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream_ptr():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _scale_arg(s):
+    """tensor -> (pointer, 0.0); python number -> (None, value)."""
+    if isinstance(s, torch.Tensor):
+        assert s.dtype == torch.float32 and s.is_cuda and s.is_contiguous()
+        return _ptr(s), 0.0
+    return None, float(s)
+
+
+class AttentionContext:
+    """One per device, like the reference's per-device compute context (gpt_cuda.cu:1478-1573)."""
+
+    def __init__(self, device=0, max_seqs=64, max_heads=16, max_head_dim=128, max_splits=32):
+        self.lib = capi.load()
+        if not torch.cuda.is_available():
+            raise RuntimeError("tscale_amd needs a HIP device; there is no CPU path")
+        cfg = capi.Config(device, max_seqs, max_heads, max_head_dim, max_splits)
+        h = ctypes.c_void_p()
+        capi.check(self.lib.tsattn_create(ctypes.byref(cfg), ctypes.byref(h)))
+        self.handle = h
+        self.device = torch.device("cuda", device)
+
+    def close(self):
+        if self.handle:
+            self.lib.tsattn_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ---- producers of the path's inputs -------------------------------------------------------
+    def quantize_rows(self, x, n_heads, dtype):
+        """x: [n_rows, n_heads*d] float32 or bfloat16 -> (uint8 [n_rows, n_heads*d], f32 [n_heads, n_rows])."""
+        assert x.is_cuda and x.is_contiguous() and x.dim() == 2
+        n_rows, hd = x.shape
+        src = capi.SRC_F32 if x.dtype == torch.float32 else capi.SRC_BF16
+        assert x.dtype in (torch.float32, torch.bfloat16)
+        q = torch.empty((n_rows, hd), dtype=torch.uint8, device=x.device)
+        scale = torch.empty((n_heads, n_rows), dtype=torch.float32, device=x.device)
+        capi.check(self.lib.tsattn_quantize_rows(self.handle, src, dtype, _ptr(x), hd * x.element_size(), n_rows,
+                                                 n_heads, hd // n_heads, _ptr(q), hd, _ptr(scale), n_rows,
+                                                 _stream_ptr()))
+        return q, scale
+
+    def build_spans(self, seq_offset, n_tokens, window, doc_start_flag=None):
+        """seq_offset: int32 [n_seqs+1] on the device.  Returns (span_start, span_finish) int32 [n_tokens]."""
+        st = torch.empty(n_tokens, dtype=torch.int32, device=self.device)
+        fi = torch.empty(n_tokens, dtype=torch.int32, device=self.device)
+        capi.check(self.lib.tsattn_build_spans(self.handle, seq_offset.numel() - 1, _ptr(seq_offset), n_tokens,
+                                               _ptr(doc_start_flag), int(window), _ptr(st), _ptr(fi), _stream_ptr()))
+        return st, fi
+
+    # ---- prefill --------------------------------------------------------------------------------
+    def compute_val_lookup(self, dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, span_start, span_finish,
+                           alibi_slope, out=None, out_f16=False, sum_weight_log=None, k_global_scale=None,
+                           debug_qk_acc=None):
+        """q,k,v: uint8 [n_tokens, n_heads*d] (row pitch = stride(0)); scales f32 [n_heads, n_tokens] or numbers."""
+        n_tokens, hd = q.shape
+        d = hd // n_heads
+        if out is None:
+            out = torch.empty((n_tokens, hd), dtype=torch.float16 if out_f16 else torch.float32, device=q.device)
+        a = capi.PrefillArgs()
+        a.dtype = dtype
+        a.out_dtype = capi.OUT_F16 if out.dtype == torch.float16 else capi.OUT_F32
+        a.n_tokens, a.n_heads, a.head_dim = n_tokens, n_heads, d
+        a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
+        a.q_pitch, a.k_pitch, a.v_pitch = q.stride(0), k.stride(0), v.stride(0)
+        a.q_scale, a.q_scale_const = _scale_arg(q_scale)
+        a.k_scale, a.k_scale_const = _scale_arg(k_scale)
+        a.v_scale, a.v_scale_const = _scale_arg(v_scale)
+        pitches = [s.stride(0) for s in (q_scale, k_scale, v_scale, sum_weight_log) if isinstance(s, torch.Tensor)]
+        assert len(set(pitches)) <= 1, "all scale planes must share one pitch"
+        a.scale_pitch = pitches[0] if pitches else n_tokens
+        a.k_global_scale = _ptr(k_global_scale)
+        a.span_start, a.span_finish = _ptr(span_start), _ptr(span_finish)
+        a.alibi_slope = float(alibi_slope)
+        a.out, a.out_pitch = _ptr(out), out.stride(0) * out.element_size()
+        a.sum_weight_log = _ptr(sum_weight_log)
+        if debug_qk_acc is not None:
+            a.debug_qk_acc, a.debug_pitch = _ptr(debug_qk_acc), debug_qk_acc.stride(1)
+        capi.check(self.lib.tsattn_prefill(self.handle, ctypes.byref(a), _stream_ptr()))
+        return out
+
+    # ---- decode ---------------------------------------------------------------------------------
+    def compute_val_lookup_decode(self, cache, q, q_scale, window, alibi_slope, out=None, n_splits=0,
+                                  debug_qk_acc=None, max_len=None):
+        """q: uint8 [B, H*d] with q_scale f32 [B, H] (or a number), or bfloat16 [B, H*d] (quantised in the kernel)."""
+        B, H, d = cache.n_seqs, cache.n_heads, cache.head_dim
+        if out is None:
+            out = torch.empty((B, H * d), dtype=torch.float32, device=q.device)
+        a = capi.DecodeArgs()
+        a.dtype = cache.dtype
+        a.q_dtype = capi.Q_BF16 if q.dtype == torch.bfloat16 else capi.Q_8BIT
+        a.n_seqs, a.n_heads, a.head_dim = B, H, d
+        a.q, a.q_pitch = _ptr(q), q.stride(0) * q.element_size()
+        a.q_scale, a.q_scale_const = _scale_arg(q_scale if q_scale is not None else 1.0)
+        a.k_cache, a.v_cache = _ptr(cache.k), _ptr(cache.v)
+        a.seq_stride, a.head_stride, a.tok_stride = cache.k.stride(0), cache.k.stride(1), cache.k.stride(2)
+        a.k_scale, a.k_scale_const = _scale_arg(cache.k_scale)
+        a.v_scale, a.v_scale_const = _scale_arg(cache.v_scale)
+        if isinstance(cache.k_scale, torch.Tensor):
+            a.s_seq_stride, a.s_head_stride = cache.k_scale.stride(0), cache.k_scale.stride(1)
+        a.cache_len = _ptr(cache.cache_len)
+        a.max_len = cache.max_len if max_len is None else int(max_len)
+        a.window = int(window)
+        a.alibi_slope = float(alibi_slope)
+        a.out = _ptr(out)
+        a.n_splits = int(n_splits)
+        if debug_qk_acc is not None:
+            a.debug_qk_acc, a.debug_pitch = _ptr(debug_qk_acc), debug_qk_acc.stride(1)
+        capi.check(self.lib.tsattn_decode(self.handle, ctypes.byref(a), _stream_ptr()))
+        return out
+
+
+class KVCache:
+    """Planar KV cache [n_seqs][n_heads][max_len][d] 8-bit with f32 row scales [n_seqs][n_heads][max_len];
+    the device-resident counterpart of TAttentionVecHistory (gpt/train/cpu_infer.cpp:397-410)."""
+
+    def __init__(self, ctx, dtype, n_seqs, n_heads, max_len, head_dim, const_scales=None):
+        dev = ctx.device
+        self.ctx, self.dtype = ctx, dtype
+        self.n_seqs, self.n_heads, self.max_len, self.head_dim = n_seqs, n_heads, max_len, head_dim
+        self.k = torch.zeros((n_seqs, n_heads, max_len, head_dim), dtype=torch.uint8, device=dev)
+        self.v = torch.zeros_like(self.k)
+        if const_scales is None:
+            self.k_scale = torch.zeros((n_seqs, n_heads, max_len), dtype=torch.float32, device=dev)
+            self.v_scale = torch.zeros_like(self.k_scale)
+        else:
+            self.k_scale, self.v_scale = const_scales
+        self.cache_len = torch.zeros(n_seqs, dtype=torch.int32, device=dev)
+
+    def add_vectors(self, k_new, k_scale_new, v_new, v_scale_new=None):
+        """k_new, v_new: uint8 [n_seqs, n_heads*d]; scales f32 [n_seqs, n_heads] (None with constant scales)."""
+        a = capi.AppendArgs()
+        a.n_seqs, a.n_heads, a.head_dim = self.n_seqs, self.n_heads, self.head_dim
+        a.k_new, a.v_new, a.new_pitch = _ptr(k_new), _ptr(v_new), k_new.stride(0)
+        a.k_scale_new, a.v_scale_new = _ptr(k_scale_new), _ptr(v_scale_new)
+        a.k_cache, a.v_cache = _ptr(self.k), _ptr(self.v)
+        a.seq_stride, a.head_stride, a.tok_stride = self.k.stride(0), self.k.stride(1), self.k.stride(2)
+        if isinstance(self.k_scale, torch.Tensor):
+            a.k_scale, a.v_scale = _ptr(self.k_scale), _ptr(self.v_scale)
+            a.s_seq_stride, a.s_head_stride = self.k_scale.stride(0), self.k_scale.stride(1)
+        a.cache_len, a.max_len = _ptr(self.cache_len), self.max_len
+        capi.check(self.ctx.lib.tsattn_cache_append(self.ctx.handle, ctypes.byref(a), _stream_ptr()))

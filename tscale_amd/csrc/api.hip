@@ -1,0 +1,241 @@
+// C ABI of the library (declared in include/tsattn.h): argument checks, the handle and the
+// launches.  Nothing here allocates, frees or synchronises except tsattn_create / tsattn_destroy.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/tsattn.h"
+#include "kernels.hpp"
+
+struct tsattn_ctx {
+    int device;
+    int max_seqs, max_heads, max_head_dim, max_splits;
+    float *part_acc;
+    float *part_ml;
+};
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char *what)
+{
+    return fail(TSATTN_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+constexpr int DEFAULT_MAX_SPLITS = 32;
+
+int cfg_splits(const tsattn_config *cfg) { return cfg->max_splits > 0 ? cfg->max_splits : DEFAULT_MAX_SPLITS; }
+
+bool head_dim_ok(int d) { return d == 64 || d == 128; }
+bool dtype_ok(int t) { return t == TSATTN_I8 || t == TSATTN_E4M3; }
+bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
+
+} // namespace
+
+extern "C" {
+
+const char *tsattn_last_error(void) { return g_err; }
+
+const char *tsattn_version(void) { return "tsattn 0.1 gfx950 (hip; mfma f8f6f4/i8 prefill, split-kv decode)"; }
+
+size_t tsattn_scratch_bytes(const tsattn_config *cfg)
+{
+    if (!cfg || cfg->max_seqs < 0 || cfg->max_heads < 0 || cfg->max_head_dim < 0) return 0;
+    size_t parts = (size_t)cfg->max_seqs * cfg->max_heads * cfg_splits(cfg);
+    return parts * ((size_t)cfg->max_head_dim + 2) * sizeof(float);
+}
+
+int tsattn_create(const tsattn_config *cfg, tsattn_handle_t *out)
+{
+    if (!cfg || !out) return fail(TSATTN_ERR_BAD_ARG, "tsattn_create: null argument");
+    if (cfg->max_seqs < 0 || cfg->max_heads < 0 || cfg->max_head_dim < 0 || cfg->max_splits < 0)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_create: negative size");
+    if (cfg->max_head_dim != 0 && !head_dim_ok(cfg->max_head_dim))
+        return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_create: head_dim %d (64 or 128 supported)", cfg->max_head_dim);
+    int n_dev = 0;
+    hipError_t e = hipGetDeviceCount(&n_dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDeviceCount");
+    if (cfg->device < 0 || cfg->device >= n_dev) return fail(TSATTN_ERR_BAD_ARG, "tsattn_create: device %d of %d", cfg->device, n_dev);
+    e = hipSetDevice(cfg->device);
+    if (e != hipSuccess) return hip_fail(e, "hipSetDevice");
+    tsattn_ctx *c = new tsattn_ctx();
+    c->device = cfg->device;
+    c->max_seqs = cfg->max_seqs;
+    c->max_heads = cfg->max_heads;
+    c->max_head_dim = cfg->max_head_dim;
+    c->max_splits = cfg_splits(cfg);
+    c->part_acc = nullptr;
+    c->part_ml = nullptr;
+    size_t parts = (size_t)c->max_seqs * c->max_heads * c->max_splits;
+    if (parts > 0 && c->max_head_dim > 0) {
+        e = hipMalloc((void **)&c->part_acc, parts * c->max_head_dim * sizeof(float));
+        if (e != hipSuccess) { delete c; return hip_fail(e, "hipMalloc(split partials)"); }
+        e = hipMalloc((void **)&c->part_ml, parts * 2 * sizeof(float));
+        if (e != hipSuccess) { (void)hipFree(c->part_acc); delete c; return hip_fail(e, "hipMalloc(split max/sum)"); }
+    }
+    *out = c;
+    return TSATTN_OK;
+}
+
+int tsattn_destroy(tsattn_handle_t h)
+{
+    if (!h) return TSATTN_OK;
+    if (h->part_acc) (void)hipFree(h->part_acc);
+    if (h->part_ml) (void)hipFree(h->part_ml);
+    delete h;
+    return TSATTN_OK;
+}
+
+int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: null argument");
+    if (!dtype_ok(a->dtype)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_prefill: dtype %d", a->dtype);
+    if (a->out_dtype != TSATTN_OUT_F32 && a->out_dtype != TSATTN_OUT_F16)
+        return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_prefill: out_dtype %d", a->out_dtype);
+    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_prefill: head_dim %d (64 or 128 supported)", a->head_dim);
+    if (a->n_tokens < 0 || a->n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: n_tokens %lld n_heads %d", (long long)a->n_tokens, a->n_heads);
+    if (a->n_tokens > 0x7fffffff - 256) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: n_tokens too large");
+    if (a->n_tokens == 0) return TSATTN_OK;
+    if (!a->q || !a->k || !a->v || !a->out || !a->span_start || !a->span_finish)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: null data pointer");
+    const int64_t row = (int64_t)a->n_heads * a->head_dim;
+    if (a->q_pitch < row || a->k_pitch < row || a->v_pitch < row || (a->q_pitch | a->k_pitch | a->v_pitch) % 16)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: input pitch must be >= %lld and a multiple of 16", (long long)row);
+    const int64_t out_row = row * (a->out_dtype == TSATTN_OUT_F16 ? 2 : 4);
+    if (a->out_pitch < out_row || a->out_pitch % 16) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: out_pitch must be >= %lld and a multiple of 16", (long long)out_row);
+    if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: q, k, v, out must be 16-byte aligned");
+    if ((a->q_scale || a->k_scale || a->v_scale || a->sum_weight_log) && a->scale_pitch < a->n_tokens)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: scale_pitch %lld < n_tokens", (long long)a->scale_pitch);
+    if (a->debug_qk_acc && a->debug_pitch < a->n_tokens) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: debug_pitch < n_tokens");
+
+    tsattn::PrefillParams p;
+    p.q = (const uint8_t *)a->q; p.k = (const uint8_t *)a->k; p.v = (const uint8_t *)a->v;
+    p.q_pitch = a->q_pitch; p.k_pitch = a->k_pitch; p.v_pitch = a->v_pitch;
+    p.qs = a->q_scale; p.ks = a->k_scale; p.vs = a->v_scale;
+    p.scale_pitch = a->scale_pitch;
+    p.qs_const = a->q_scale_const; p.ks_const = a->k_scale_const; p.vs_const = a->v_scale_const;
+    p.k_global_scale = a->k_global_scale;
+    p.span_start = a->span_start; p.span_finish = a->span_finish;
+    p.slope = a->alibi_slope;
+    p.out = a->out; p.out_pitch = a->out_pitch;
+    p.sum_weight_log = a->sum_weight_log;
+    p.dbg = a->debug_qk_acc; p.dbg_pitch = a->debug_pitch;
+    p.n_tokens = (int)a->n_tokens; p.n_heads = a->n_heads;
+    hipError_t e = tsattn::launch_prefill(p, a->dtype, a->head_dim, a->out_dtype, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "prefill launch");
+    return TSATTN_OK;
+}
+
+int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: null argument");
+    if (!dtype_ok(a->dtype)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: dtype %d", a->dtype);
+    if (a->q_dtype != TSATTN_Q_8BIT && a->q_dtype != TSATTN_Q_BF16) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: q_dtype %d", a->q_dtype);
+    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: head_dim %d (64 or 128 supported)", a->head_dim);
+    if (a->n_seqs < 0 || a->n_heads <= 0 || a->max_len < 0 || a->window < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: negative size");
+    if (a->n_seqs == 0) return TSATTN_OK;
+    if (!a->q || !a->k_cache || !a->v_cache || !a->cache_len || !a->out) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: null data pointer");
+    const int qbytes = a->q_dtype == TSATTN_Q_BF16 ? 2 : 1;
+    if (a->q_pitch < (int64_t)a->n_heads * a->head_dim * qbytes || a->q_pitch % 16) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: q_pitch");
+    if (a->tok_stride < a->head_dim || a->tok_stride % 16 || a->head_stride % 16 || a->seq_stride % 16)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: cache strides must be multiples of 16 bytes, tok_stride >= head_dim");
+    if (!aligned16(a->q) || !aligned16(a->k_cache) || !aligned16(a->v_cache)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: q and caches must be 16-byte aligned");
+    if (a->debug_qk_acc && a->debug_pitch < a->max_len) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: debug_pitch < max_len");
+    if (a->n_seqs > h->max_seqs || a->n_heads > h->max_heads || a->head_dim > h->max_head_dim)
+        return fail(TSATTN_ERR_SCRATCH, "tsattn_decode: %d seqs x %d heads x d%d exceeds the handle's %d x %d x d%d", a->n_seqs, a->n_heads,
+                    a->head_dim, h->max_seqs, h->max_heads, h->max_head_dim);
+    int splits = a->n_splits;
+    if (splits < 0 || splits > h->max_splits) return fail(TSATTN_ERR_SCRATCH, "tsattn_decode: n_splits %d exceeds the handle's %d", splits, h->max_splits);
+    if (splits == 0) {
+        // enough workgroups to fill 256 CUs several times over, but at least 512 cache rows per split
+        const int64_t pairs = (int64_t)a->n_seqs * a->n_heads;
+        int64_t want = (4096 + pairs - 1) / pairs;
+        int64_t by_len = ((int64_t)a->max_len + 511) / 512;
+        if (want > by_len) want = by_len;
+        if (want < 1) want = 1;
+        if (want > h->max_splits) want = h->max_splits;
+        splits = (int)want;
+    }
+    tsattn::DecodeParams p;
+    p.q = (const uint8_t *)a->q; p.q_pitch = a->q_pitch; p.q_scale = a->q_scale; p.q_scale_const = a->q_scale_const;
+    p.k = (const uint8_t *)a->k_cache; p.v = (const uint8_t *)a->v_cache;
+    p.seq_stride = a->seq_stride; p.head_stride = a->head_stride; p.tok_stride = a->tok_stride;
+    p.ks = a->k_scale; p.vs = a->v_scale; p.s_seq_stride = a->s_seq_stride; p.s_head_stride = a->s_head_stride;
+    p.ks_const = a->k_scale_const; p.vs_const = a->v_scale_const;
+    p.cache_len = a->cache_len; p.window = a->window; p.slope = a->alibi_slope;
+    p.n_heads = a->n_heads; p.n_splits = splits;
+    p.part_acc = h->part_acc; p.part_ml = h->part_ml;
+    p.dbg = a->debug_qk_acc; p.dbg_pitch = a->debug_pitch;
+    hipError_t e = tsattn::launch_decode(p, a->dtype, a->head_dim, a->q_dtype == TSATTN_Q_BF16, a->n_seqs, a->out, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "decode launch");
+    return TSATTN_OK;
+}
+
+int tsattn_cache_append(tsattn_handle_t h, const tsattn_append_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_append: null argument");
+    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_cache_append: head_dim %d (64 or 128 supported)", a->head_dim);
+    if (a->n_seqs < 0 || a->n_heads <= 0 || a->max_len < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_append: negative size");
+    if (a->n_seqs == 0) return TSATTN_OK;
+    if (!a->k_new || !a->v_new || !a->k_cache || !a->v_cache || !a->cache_len) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_append: null data pointer");
+    if ((a->k_scale_new && !a->k_scale) || (a->v_scale_new && !a->v_scale)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_append: new scales given without scale planes");
+    if (a->new_pitch % 16 || a->tok_stride % 16 || a->head_stride % 16 || a->seq_stride % 16 || a->tok_stride < a->head_dim)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_append: pitches and strides must be multiples of 16 bytes");
+    if (!aligned16(a->k_new) || !aligned16(a->v_new) || !aligned16(a->k_cache) || !aligned16(a->v_cache))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_append: pointers must be 16-byte aligned");
+    tsattn::AppendParams p;
+    p.k_new = (const uint8_t *)a->k_new; p.v_new = (const uint8_t *)a->v_new; p.new_pitch = a->new_pitch;
+    p.ks_new = a->k_scale_new; p.vs_new = a->v_scale_new;
+    p.k = (uint8_t *)a->k_cache; p.v = (uint8_t *)a->v_cache;
+    p.seq_stride = a->seq_stride; p.head_stride = a->head_stride; p.tok_stride = a->tok_stride;
+    p.ks = a->k_scale; p.vs = a->v_scale; p.s_seq_stride = a->s_seq_stride; p.s_head_stride = a->s_head_stride;
+    p.cache_len = a->cache_len; p.max_len = a->max_len; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
+    hipError_t e = tsattn::launch_cache_append(p, a->n_seqs, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "cache append launch");
+    return TSATTN_OK;
+}
+
+int tsattn_quantize_rows(tsattn_handle_t h, int src_dtype, int dst_dtype, const void *src, int64_t src_pitch, int64_t n_rows,
+                         int n_heads, int head_dim, void *dst, int64_t dst_pitch, float *scale, int64_t scale_pitch, void *stream)
+{
+    if (!h) return fail(TSATTN_ERR_BAD_ARG, "tsattn_quantize_rows: null handle");
+    if (!dtype_ok(dst_dtype) || (src_dtype != TSATTN_SRC_F32 && src_dtype != TSATTN_SRC_BF16))
+        return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_quantize_rows: dtypes %d -> %d", src_dtype, dst_dtype);
+    if (head_dim <= 0 || head_dim % 64 || head_dim > 256) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_quantize_rows: head_dim %d (multiple of 64 up to 256)", head_dim);
+    if (n_rows < 0 || n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_quantize_rows: negative size");
+    if (n_rows == 0) return TSATTN_OK;
+    if (!src || !dst || !scale) return fail(TSATTN_ERR_BAD_ARG, "tsattn_quantize_rows: null data pointer");
+    const int64_t row = (int64_t)n_heads * head_dim;
+    if (src_pitch < row * (src_dtype == TSATTN_SRC_F32 ? 4 : 2) || dst_pitch < row || scale_pitch < n_rows)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_quantize_rows: pitch too small");
+    hipError_t e = tsattn::launch_quantize_rows(src_dtype, dst_dtype, src, src_pitch, n_rows, n_heads, head_dim, dst, dst_pitch, scale,
+                                                scale_pitch, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "quantize launch");
+    return TSATTN_OK;
+}
+
+int tsattn_build_spans(tsattn_handle_t h, int n_seqs, const int32_t *seq_offset, int64_t n_tokens, const uint8_t *doc_start_flag,
+                       int64_t window, int32_t *span_start, int32_t *span_finish, void *stream)
+{
+    if (!h) return fail(TSATTN_ERR_BAD_ARG, "tsattn_build_spans: null handle");
+    if (n_seqs < 0 || n_tokens < 0 || window < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_build_spans: negative size");
+    if (n_tokens == 0) return TSATTN_OK;
+    if (n_seqs == 0 || !seq_offset || !span_start || !span_finish) return fail(TSATTN_ERR_BAD_ARG, "tsattn_build_spans: null data pointer");
+    hipError_t e = tsattn::launch_build_spans(n_seqs, seq_offset, n_tokens, doc_start_flag, window, span_start, span_finish, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "build spans launch");
+    return TSATTN_OK;
+}
+
+} // extern "C"

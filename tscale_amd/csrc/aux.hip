@@ -1,0 +1,147 @@
+// Small kernels around the attention path: the absmax row quantiser, the span (window metadata)
+// builder and the KV-cache append.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace tsattn {
+
+// One wave per (row, head).  scale = absmax/127 (int8) or absmax/256 (e4m3); values times 1/scale,
+// rounded to nearest even (lib/cuda/cuda_matmul.cuh:237-249, lib/cuda/cuda_util.cuh:286-297).
+template <int SRC, int DST>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const uint8_t *src, int64_t src_pitch, int64_t n_rows, int n_heads,
+                                                            int head_dim, uint8_t *dst, int64_t dst_pitch, float *scale,
+                                                            int64_t scale_pitch)
+{
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int64_t job = (int64_t)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+    if (job >= n_rows * n_heads) return;
+    const int64_t row = job / n_heads;
+    const int head = (int)(job % n_heads);
+    const int per = head_dim / WAVE; // head_dim is a multiple of 64, at most 256
+    float x[4];
+    float amax = 0;
+    for (int i = 0; i < per; ++i) {
+        int e = head * head_dim + i * WAVE + lane;
+        if (SRC == TSATTN_SRC_F32) x[i] = ((const float *)(src + row * src_pitch))[e];
+        else x[i] = bf16_to_float(((const uint16_t *)(src + row * src_pitch))[e]);
+        amax = fmaxf(amax, fabsf(x[i]));
+    }
+    amax = wave_max(amax);
+    float discr = 0, mult = 0;
+    if (amax > 0) {
+        discr = (DST == TSATTN_I8) ? amax / 127.0f : amax / 256.0f;
+        mult = 1.0f / discr;
+    }
+    for (int i = 0; i < per; ++i) {
+        float y = x[i] * mult;
+        uint8_t b = (DST == TSATTN_I8) ? (uint8_t)float_to_i8(y) : float_to_e4m3(y);
+        dst[row * dst_pitch + head * head_dim + i * WAVE + lane] = b;
+    }
+    if (lane == 0) scale[head * scale_pitch + row] = discr;
+}
+
+hipError_t launch_quantize_rows(int src_dtype, int dst_dtype, const void *src, int64_t src_pitch, int64_t n_rows,
+                                int n_heads, int head_dim, void *dst, int64_t dst_pitch, float *scale,
+                                int64_t scale_pitch, hipStream_t st)
+{
+    int64_t jobs = n_rows * n_heads;
+    if (jobs == 0) return hipSuccess;
+    dim3 grid((unsigned)((jobs + 3) / 4)), block(256);
+#define TSATTN_QR(S, D)                                                                                              \
+    hipLaunchKernelGGL((quantize_rows_kernel<S, D>), grid, block, 0, st, (const uint8_t *)src, src_pitch, n_rows,   \
+                       n_heads, head_dim, (uint8_t *)dst, dst_pitch, scale, scale_pitch)
+    if (src_dtype == TSATTN_SRC_F32 && dst_dtype == TSATTN_I8) TSATTN_QR(TSATTN_SRC_F32, TSATTN_I8);
+    else if (src_dtype == TSATTN_SRC_F32 && dst_dtype == TSATTN_E4M3) TSATTN_QR(TSATTN_SRC_F32, TSATTN_E4M3);
+    else if (src_dtype == TSATTN_SRC_BF16 && dst_dtype == TSATTN_I8) TSATTN_QR(TSATTN_SRC_BF16, TSATTN_I8);
+    else if (src_dtype == TSATTN_SRC_BF16 && dst_dtype == TSATTN_E4M3) TSATTN_QR(TSATTN_SRC_BF16, TSATTN_E4M3);
+    else return hipErrorInvalidValue;
+#undef TSATTN_QR
+    return hipGetLastError();
+}
+
+// One thread per token: span = [max(docStart, t - W), t - 1] shifted by the sequence's first token;
+// W == 0 means the token itself (gpt/att/sliding_window.cpp:80-87, 213-220).  A flagged token
+// starts a document unless it is the first token of its sequence (:150-154).
+__global__ __launch_bounds__(256) void build_spans_kernel(int n_seqs, const int32_t *seq_offset, int64_t n_tokens,
+                                                          const uint8_t *flag, int64_t window, int32_t *span_start,
+                                                          int32_t *span_finish)
+{
+    const int64_t tok = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tok >= n_tokens) return;
+    int lo = 0, hi = n_seqs; // last sequence whose offset <= tok
+    while (hi - lo > 1) {
+        int mid = (lo + hi) / 2;
+        if (seq_offset[mid] <= tok) lo = mid; else hi = mid;
+    }
+    const int64_t base = seq_offset[lo];
+    const int64_t t = tok - base;
+    int64_t a, b;
+    if (window == 0) {
+        a = t; b = t;
+    } else {
+        a = t - window;
+        if (a < 0) a = 0;
+        b = t - 1;
+        if (flag) {
+            // the latest document start in (a, t] clips the span
+            for (int64_t u = t; u > a; --u) {
+                if (flag[base + u]) { a = u; break; }
+            }
+        }
+        if (b < a) { a = t; b = t - 1; }
+    }
+    span_start[tok] = (int32_t)(a + base);
+    span_finish[tok] = (int32_t)(b + base);
+}
+
+hipError_t launch_build_spans(int n_seqs, const int32_t *seq_offset, int64_t n_tokens, const uint8_t *doc_start_flag,
+                              int64_t window, int32_t *span_start, int32_t *span_finish, hipStream_t st)
+{
+    if (n_tokens == 0) return hipSuccess;
+    hipLaunchKernelGGL(build_spans_kernel, dim3((unsigned)((n_tokens + 255) / 256)), dim3(256), 0, st, n_seqs, seq_offset,
+                       n_tokens, doc_start_flag, window, span_start, span_finish);
+    return hipGetLastError();
+}
+
+// TAttentionVecHistory::AddVectors (gpt/train/cpu_infer.cpp:403-408) for a planar cache: one thread
+// copies 16 bytes of the new K and V rows to row cache_len[seq]; a second kernel bumps the lengths.
+__global__ __launch_bounds__(256) void cache_append_kernel(AppendParams p, int n_seqs)
+{
+    const int chunks = p.head_dim / 16;
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = (int64_t)n_seqs * p.n_heads * chunks;
+    if (id >= total) return;
+    const int c = (int)(id % chunks);
+    const int head = (int)((id / chunks) % p.n_heads);
+    const int seq = (int)(id / ((int64_t)chunks * p.n_heads));
+    const int pos = p.cache_len[seq];
+    if (pos < 0 || pos >= p.max_len) return;
+    const int64_t src = (int64_t)seq * p.new_pitch + head * p.head_dim + c * 16;
+    const int64_t dst = (int64_t)seq * p.seq_stride + (int64_t)head * p.head_stride + (int64_t)pos * p.tok_stride + c * 16;
+    *(v4i *)(p.k + dst) = *(const v4i *)(p.k_new + src);
+    *(v4i *)(p.v + dst) = *(const v4i *)(p.v_new + src);
+    if (c == 0) {
+        const int64_t sd = (int64_t)seq * p.s_seq_stride + (int64_t)head * p.s_head_stride + pos;
+        if (p.ks_new) p.ks[sd] = p.ks_new[seq * p.n_heads + head];
+        if (p.vs_new) p.vs[sd] = p.vs_new[seq * p.n_heads + head];
+    }
+}
+
+__global__ void cache_len_bump_kernel(int32_t *cache_len, int n_seqs, int max_len)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_seqs && cache_len[i] >= 0 && cache_len[i] < max_len) cache_len[i] += 1;
+}
+
+hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st)
+{
+    if (n_seqs == 0) return hipSuccess;
+    const int64_t total = (int64_t)n_seqs * p.n_heads * (p.head_dim / 16);
+    hipLaunchKernelGGL(cache_append_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, p, n_seqs);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(cache_len_bump_kernel, dim3((unsigned)((n_seqs + 255) / 256)), dim3(256), 0, st, p.cache_len, n_seqs, p.max_len);
+    return hipGetLastError();
+}
+
+} // namespace tsattn

@@ -1,0 +1,75 @@
+// Parameter blocks and host-side launchers shared between the kernel files and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tsattn {
+
+struct DecodeParams {
+    const uint8_t *q;
+    int64_t q_pitch;
+    const float *q_scale;
+    float q_scale_const;
+    const uint8_t *k, *v;
+    int64_t seq_stride, head_stride, tok_stride;
+    const float *ks, *vs;
+    int64_t s_seq_stride, s_head_stride;
+    float ks_const, vs_const;
+    const int32_t *cache_len;
+    int64_t window;
+    float slope;
+    int n_heads;
+    int n_splits;
+    float *part_acc; // [seq][head][split][d]
+    float *part_ml;  // [seq][head][split][2] = running max, sum
+    void *dbg;
+    int64_t dbg_pitch;
+};
+
+hipError_t launch_decode(const DecodeParams &p, int dtype, int head_dim, bool qbf16, int n_seqs, float *out, hipStream_t st);
+
+struct PrefillParams {
+    const uint8_t *q, *k, *v;
+    int64_t q_pitch, k_pitch, v_pitch;
+    const float *qs, *ks, *vs;
+    int64_t scale_pitch;
+    float qs_const, ks_const, vs_const;
+    const float *k_global_scale;
+    const int32_t *span_start, *span_finish;
+    float slope;
+    void *out;
+    int64_t out_pitch;
+    float *sum_weight_log;
+    void *dbg;
+    int64_t dbg_pitch;
+    int n_tokens;
+    int n_heads;
+};
+
+hipError_t launch_prefill(const PrefillParams &p, int dtype, int head_dim, int out_dtype, hipStream_t st);
+
+hipError_t launch_quantize_rows(int src_dtype, int dst_dtype, const void *src, int64_t src_pitch, int64_t n_rows,
+                                int n_heads, int head_dim, void *dst, int64_t dst_pitch, float *scale,
+                                int64_t scale_pitch, hipStream_t st);
+
+hipError_t launch_build_spans(int n_seqs, const int32_t *seq_offset, int64_t n_tokens, const uint8_t *doc_start_flag,
+                              int64_t window, int32_t *span_start, int32_t *span_finish, hipStream_t st);
+
+struct AppendParams {
+    const uint8_t *k_new, *v_new;
+    int64_t new_pitch;
+    const float *ks_new, *vs_new;
+    uint8_t *k, *v;
+    int64_t seq_stride, head_stride, tok_stride;
+    float *ks, *vs;
+    int64_t s_seq_stride, s_head_stride;
+    int32_t *cache_len;
+    int max_len;
+    int n_heads;
+    int head_dim;
+};
+
+hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st);
+
+} // namespace tsattn
