@@ -1,0 +1,274 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized attention path on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
+  prefill (the headline `value`): the 125M-style configuration -- batch 16, seq 1024, 12 heads,
+      head_dim 64, e4m3 Q/K/V with per-row fp32 scales, 12 layers alternating (window 64, slope 0.5)
+      and (full causal window, slope 0) -- one step = the 12 attention launches of one forward pass,
+      each layer on its own Q/K/V buffers.
+  decode (reported in the same line under "decode"): batch 64, one bf16 query per sequence, int8 KV
+      cache of 4096 rows, 16 heads x 128, per-row scales; one step = one decode launch pair
+      (split kernel + merge), rotating over 4 caches so that no launch finds its cache in the
+      Infinity Cache.
+Algorithmic work: FLOPs = 4*d*sum_rows min(row, W) per (sequence, head) (masked tiles count zero,
+the zero vector adds none); decode bytes = K + V planes + both scale planes + q + out.
+
+Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this build uses one GPU.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA
+PEAK_I8_TOPS = 5000.0
+PEAK_HBM_GBPS = 8000.0
+
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, scaled
+# by what the same counters read for a copy kernel of known size).  None until measured; the numbers
+# and commands are in profiles/.
+MEASURED_TRAFFIC = {"prefill_c2": None, "decode_c3": None}
+
+
+def pairs(S, W):
+    """sum over rows of min(row, W): (query, key) pairs of one sequence and head."""
+    W = min(W, S)
+    return W * (W - 1) // 2 + (S - W) * W
+
+
+def prefill_flops(B, S, H, d, W):
+    return 4.0 * d * pairs(S, W) * B * H
+
+
+def layer_schedule(n_layers, wide, short):
+    return [(short, 0.5) if i % 2 == 0 else (wide, 0.0) for i in range(n_layers)]
+
+
+def gpu_time_ms(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+class PrefillWorkload:
+    def __init__(self, ctx, dtype, B, S, H, d, n_layers, seed, short=64):
+        import torch
+        self.ctx, self.dtype, self.B, self.S, self.H, self.d = ctx, dtype, B, S, H, d
+        self.layers = layer_schedule(n_layers, S, short)
+        n = B * S
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        self.inputs = []
+        for _ in range(n_layers):
+            qkv = []
+            for _ in range(3):
+                x = torch.randn((n, H * d), device="cuda", generator=g)
+                qkv.append(ctx.quantize_rows(x, H, dtype))
+                del x
+            self.inputs.append(qkv)
+        off = torch.arange(0, n + 1, S, dtype=torch.int32, device="cuda")
+        self.spans = {W: ctx.build_spans(off, n, W) for W in {w for w, _ in self.layers}}
+        self.out = torch.empty((n, H * d), dtype=torch.float16, device="cuda")
+        self.flops_layer = [prefill_flops(B, S, H, d, W) for W, _ in self.layers]
+        self.flops = sum(self.flops_layer)
+        torch.cuda.synchronize()
+
+    def run_layer(self, i):
+        (q, qs), (k, ks), (v, vs) = self.inputs[i]
+        W, slope = self.layers[i]
+        st, fi = self.spans[W]
+        self.ctx.compute_val_lookup(self.dtype, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out)
+
+    def step(self):
+        for i in range(len(self.layers)):
+            self.run_layer(i)
+
+
+class DecodeWorkload:
+    def __init__(self, ctx, B, L, H, d, n_caches, seed):
+        import torch
+        from tscale_amd import KVCache, capi
+        self.ctx, self.B, self.L, self.H, self.d = ctx, B, L, H, d
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        self.caches = []
+        for _ in range(n_caches):
+            c = KVCache(ctx, capi.I8, B, H, L, d)
+            for plane, scale in ((c.k, c.k_scale), (c.v, c.v_scale)):
+                for b0 in range(0, B, 8):  # bounded temporaries
+                    x = torch.randn((8 * H * L, d), device="cuda", generator=g)
+                    q8, s = ctx.quantize_rows(x, 1, capi.I8)
+                    plane[b0:b0 + 8].copy_(q8.view(8, H, L, d))
+                    scale[b0:b0 + 8].copy_(s.view(8, H, L))
+                    del x, q8, s
+            c.cache_len.fill_(L)
+            self.caches.append(c)
+        self.q = torch.randn((B, H * d), device="cuda", generator=g).to(torch.bfloat16)
+        self.out = torch.empty((B, H * d), dtype=torch.float32, device="cuda")
+        self.i = 0
+        # K + V planes, two scale planes, bf16 q, f32 out
+        self.bytes = 2 * B * H * L * d + 2 * B * H * L * 4 + B * H * d * 2 + B * H * d * 4
+        torch.cuda.synchronize()
+
+    def step(self):
+        c = self.caches[self.i % len(self.caches)]
+        self.i += 1
+        self.ctx.compute_val_lookup_decode(c, self.q, None, 10 ** 6, 0.0, out=self.out)
+
+
+def cpu_baseline_prefill(wl, n_seq_sample):
+    """The oracle (a port of the reference's CPU attention) on the first sequences of layer 0 (window 64)
+    and layer 1 (full causal window), all host threads."""
+    import numpy as np
+    from oracle import pyoracle as orc
+    S, H, d = wl.S, wl.H, wl.d
+    n = n_seq_sample * S
+    threads = orc.max_threads()
+    flops = 0.0
+    t_total = 0.0
+    for li in (0, 1):
+        (q, qs), (k, ks), (v, vs) = wl.inputs[li]
+        W, slope = wl.layers[li]
+        hq, hk, hv = (x[:n].cpu().numpy() for x in (q, k, v))
+        hqs, hks, hvs = (np.ascontiguousarray(x[:, :n].cpu().numpy()) for x in (qs, ks, vs))
+        st, fi = orc.make_spans([S] * n_seq_sample, W)
+        t0 = time.perf_counter()
+        orc.prefill_q8(wl.dtype, hq, hk, hv, H, hqs, hks, hvs, st, fi, slope, n_threads=threads)
+        t_total += time.perf_counter() - t0
+        flops += prefill_flops(n_seq_sample, S, H, d, W)
+    t1 = None
+    # single thread (the reference's CPU path has no threading): one sequence of the wide layer
+    (q, qs), (k, ks), (v, vs) = wl.inputs[1]
+    hq, hk, hv = (x[:S].cpu().numpy() for x in (q, k, v))
+    hqs, hks, hvs = (np.ascontiguousarray(x[:, :S].cpu().numpy()) for x in (qs, ks, vs))
+    st, fi = orc.make_spans([S], S)
+    t0 = time.perf_counter()
+    orc.prefill_q8(wl.dtype, hq, hk, hv, H, hqs, hks, hvs, st, fi, 0.0, n_threads=1)
+    t1 = time.perf_counter() - t0
+    return {
+        "value": flops / t_total / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"{n_seq_sample} of {wl.B} sequences, one window-64 layer + one full-window layer, "
+                  f"{threads} OpenMP threads, {t_total:.2f} s",
+        "single_thread_value": prefill_flops(1, S, H, d, S) / t1 / 1e12,
+        "single_thread_sample": f"1 sequence, full-window layer, {t1:.2f} s",
+    }
+
+
+def cpu_baseline_decode(wl, n_seq_sample, reps):
+    import numpy as np
+    from oracle import pyoracle as orc
+    c = wl.caches[0]
+    k = c.k[:n_seq_sample].cpu().numpy(); v = c.v[:n_seq_sample].cpu().numpy()
+    ks = c.k_scale[:n_seq_sample].cpu().numpy(); vs = c.v_scale[:n_seq_sample].cpu().numpy()
+    import torch
+    bits = wl.q[:n_seq_sample].cpu().view(torch.int16).numpy().view(np.uint16)
+    q8, qs = orc.quantize_rows(orc.I8, bits, wl.H)
+    qs = np.ascontiguousarray(qs.T)
+    lens = np.full(n_seq_sample, wl.L, np.int32)
+    threads = orc.max_threads()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        orc.decode(orc.I8, q8, qs, k, v, ks, vs, lens, 10 ** 6, 0.0, exp2_mode=1, use_simd=True, n_threads=threads)
+    t = (time.perf_counter() - t0) / reps
+    nbytes = wl.bytes * n_seq_sample / wl.B
+    return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{n_seq_sample} of {wl.B} sequences, {reps} repetitions, vpdpbusd level {orc.simd_level()}, "
+                      f"{threads} OpenMP threads, {t * reps:.2f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--extra", action="store_true", help="also time the 1.5B-style prefill shapes")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from tscale_amd import AttentionContext, capi
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device", file=sys.stderr)
+        sys.exit(1)
+    ctx = AttentionContext(0, max_seqs=64, max_heads=16, max_head_dim=128, max_splits=32)
+
+    # ---- prefill, 125M-style -----------------------------------------------------------------
+    B, S, H, d, NL = 16, 1024, 12, 64, 12
+    wl = PrefillWorkload(ctx, capi.E4M3, B, S, H, d, NL, seed=1313 + 2)
+    ms = gpu_time_ms(wl.step, args.steps, args.warmup)
+    tflops = wl.flops / (ms * 1e-3) / 1e12
+    ms_short = gpu_time_ms(lambda: wl.run_layer(0), args.steps, 2)
+    ms_wide = gpu_time_ms(lambda: wl.run_layer(1), args.steps, 2)
+    launch_ms = ms / NL
+    ach = (wl.flops / NL) / (launch_ms * 1e-3) / 1e12
+    result = {
+        "metric": "prefill attn TFLOP/s + decode attn HBM GB/s (% of MI355X peak), 1 GPU",
+        "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "e4m3 (fp32 accumulate; f16 P.V)", "data": "synthetic",
+        "config": {"workload": "prefill-125M-style: B16 S1024 H12 d64 e4m3 + per-row f32 scales, 12 layers "
+                               "alternating (W=64, slope 0.5)/(W=1024, slope 0), f16 out; 173.18 GFLOP per step",
+                   "layer_ms": {"window64": round(ms_short, 5), "full": round(ms_wide, 5)},
+                   "layer_tflops": {"window64": round(wl.flops_layer[0] / ms_short / 1e9, 2),
+                                    "full": round(wl.flops_layer[1] / ms_wide / 1e9, 2)}},
+        "roofline": {"kernel": "prefill_kernel<e4m3, d64>", "bound": "mfma", "achieved": round(ach, 3),
+                     "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_FP8_TFLOPS, 5),
+                     "traffic": MEASURED_TRAFFIC["prefill_c2"],
+                     "launch_ms": round(launch_ms, 5), "flops_per_launch": wl.flops / NL},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline_prefill(wl, 4)
+    del wl
+    torch.cuda.empty_cache()
+
+    # ---- decode, int8 KV ----------------------------------------------------------------------
+    if not args.no_decode:
+        dw = DecodeWorkload(ctx, 64, 4096, 16, 128, n_caches=4, seed=1313 + 3)
+        dsteps = max(args.steps, 20)
+        dms = gpu_time_ms(dw.step, dsteps, max(args.warmup, 4))
+        gbps = dw.bytes / (dms * 1e-3) / 1e9
+        dec = {"value": round(gbps, 2), "unit": "GB/s", "ms_per_step": round(dms, 5), "steps": dsteps, "dtype": "int8",
+               "config": {"workload": "decode: B64, 1 bf16 query/seq, int8 KV cache L=4096, H16 d128, per-row f32 scales; "
+                                      "1108.08 MB per step; 4 caches in rotation"},
+               "roofline": {"kernel": "decode_split_kernel<int8, d128>", "bound": "hbm", "achieved": round(gbps, 2),
+                            "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(gbps / PEAK_HBM_GBPS, 5),
+                            "traffic": MEASURED_TRAFFIC["decode_c3"], "bytes_per_launch": dw.bytes}}
+        if not args.no_cpu:
+            dec["cpu_baseline"] = cpu_baseline_decode(dw, 8, 3)
+        result["decode"] = dec
+        del dw
+        torch.cuda.empty_cache()
+
+    # ---- optional: 1.5B-style prefill shapes ---------------------------------------------------------
+    if args.extra:
+        B, S, H, d = 8, 4096, 16, 128
+        wl = PrefillWorkload(ctx, capi.E4M3, B, S, H, d, 2, seed=1313 + 4, short=256)
+        steps = max(10, args.steps // 5)
+        ms_s = gpu_time_ms(lambda: wl.run_layer(0), steps, 2)
+        ms_w = gpu_time_ms(lambda: wl.run_layer(1), steps, 2)
+        result["prefill_1p5B_style"] = {
+            "config": "B8 S4096 H16 d128 e4m3, W=256 (slope 0.5) / full (slope 0)",
+            "layer_ms": {"window256": round(ms_s, 5), "full": round(ms_w, 5)},
+            "layer_tflops": {"window256": round(wl.flops_layer[0] / ms_s / 1e9, 2), "full": round(wl.flops_layer[1] / ms_w / 1e9, 2)},
+            "frac_of_fp8_peak_full": round(wl.flops_layer[1] / ms_w / 1e9 / PEAK_FP8_TFLOPS, 5)}
+        del wl
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -14,6 +14,8 @@
 //                   when the tile is staged, and read back transposed with ds_read_b64_tr_b16.
 // Semantics: gpt/compute/gpt_cpu.cpp:391-441 (two-pass form of the same sums) with the 8-bit
 // operand handling of gpt/compute/gpt_att_fp8.cuh:139-152 / gpt_att_fp16.cuh:184-189.
+#include <type_traits>
+
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -96,46 +98,54 @@ struct QkMma<TSATTN_I8, D> {
     __device__ static float bits(const acc_t &a, int r) { return __int_as_float(a[r]); }
 };
 
-// 16 bytes of one V row -> 16 halves scaled by the row's value scale
+// 16 bytes of one V row -> 16 halves scaled by the row's value scale.
+// e4m3: v_cvt_scalef32_pk_f16_fp8 (exact widening, unit scale) then a packed f16 multiply.
+// int8: byte b -> f16 bits 0x6400 | (b ^ 0x80) = 1024 + (b + 128); a packed add of -1152 gives b
+//       exactly, then the packed multiply.
 template <int DTYPE>
 __device__ inline void widen_v(v4i raw, float vs, v8h &lo, v8h &hi)
 {
+    const _Float16 vsh = (_Float16)vs;
+    const v2h vs2 = v2h{vsh, vsh};
     int w[4] = {raw.x, raw.y, raw.z, raw.w};
-    _Float16 h[16];
+    v2h h[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float f0, f1, f2, f3;
         if (DTYPE == TSATTN_I8) {
-            f0 = (float)(int8_t)(w[i] & 0xff);
-            f1 = (float)(int8_t)((w[i] >> 8) & 0xff);
-            f2 = (float)(int8_t)((w[i] >> 16) & 0xff);
-            f3 = (float)(w[i] >> 24);
+            const unsigned u = (unsigned)w[i] ^ 0x80808080u;
+            const unsigned a = __builtin_amdgcn_perm(u, 0x64646464u, 0x00050004u);
+            const unsigned b = __builtin_amdgcn_perm(u, 0x64646464u, 0x00070006u);
+            const v2h off = v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
+            h[2 * i] = (__builtin_bit_cast(v2h, a) + off) * vs2;
+            h[2 * i + 1] = (__builtin_bit_cast(v2h, b) + off) * vs2;
         } else {
-            v2f a = e4m3x2_to_float(w[i], false), b = e4m3x2_to_float(w[i], true);
-            f0 = a.x; f1 = a.y; f2 = b.x; f3 = b.y;
+            h[2 * i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, false) * vs2;
+            h[2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, true) * vs2;
         }
-        h[4 * i + 0] = (_Float16)(f0 * vs);
-        h[4 * i + 1] = (_Float16)(f1 * vs);
-        h[4 * i + 2] = (_Float16)(f2 * vs);
-        h[4 * i + 3] = (_Float16)(f3 * vs);
     }
-    lo = v8h{h[0], h[1], h[2], h[3], h[4], h[5], h[6], h[7]};
-    hi = v8h{h[8], h[9], h[10], h[11], h[12], h[13], h[14], h[15]};
+    lo = v8h{h[0][0], h[0][1], h[1][0], h[1][1], h[2][0], h[2][1], h[3][0], h[3][1]};
+    hi = v8h{h[4][0], h[4][1], h[5][0], h[5][1], h[6][0], h[6][1], h[7][0], h[7][1]};
 }
 
 typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
 
-template <int DTYPE, int D, bool OUT_F16, bool DUMP>
-__global__ __launch_bounds__(PF_THREADS) void prefill_kernel(PrefillParams p)
+// A logit may exceed the reference maximum by this much (log2 units) before the accumulators are
+// rescaled: weights then stay below 2^8, far inside f16 and f32 range, and ordinary inputs never
+// trigger a rescale because the reference maximum starts at the zero vector's logit 0.
+constexpr float PF_RESCALE_THRESHOLD = 8.0f;
+
+template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP>
+__global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p)
 {
     typedef PfLayout<D> L;
     typedef QkMma<DTYPE, D> Qk;
-    constexpr int DT = D / 32;       // 32-row tiles of O^T
-    constexpr int CHUNKS = D / 16;   // 16-byte chunks per 8-bit row
+    constexpr int DT = D / 32;                               // 32-row tiles of O^T
+    constexpr int CHUNKS = D / 16;                           // 16-byte chunks per 8-bit row
+    constexpr int NLD = (PF_BN * CHUNKS) / PF_THREADS;       // 16-byte chunks per thread per tile
 
-    __shared__ __attribute__((aligned(16))) uint8_t k_lds[L::K_BYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t v_lds[L::V_BYTES];
-    __shared__ __attribute__((aligned(16))) float ks_lds[PF_BN];
+    __shared__ __attribute__((aligned(16))) uint8_t k_lds[2][L::K_BYTES];
+    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2][L::V_BYTES];
+    __shared__ __attribute__((aligned(16))) float ks_lds[2][PF_BN];
     __shared__ int red_lds[2 * PF_WAVES];
 
     const int tid = threadIdx.x;
@@ -188,109 +198,146 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_kernel(PrefillParams p)
     v16f o_acc[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i) o_acc[i] = v16f{0};
-    float m = 0.0f; // the zero vector's logit takes part in the maximum
-    float l = 0.0f; // this lane's share of the sum (its 32 of every 64 keys)
+    float m_ref = 0.0f; // reference maximum: starts at the zero vector's logit
+    float l = 0.0f;     // this lane's share of the weight sum (its 32 of every 64 keys)
 
     if (b_max_b >= b_min_a) {
         const int kb_first = (b_min_a / PF_BN) * PF_BN;
-        for (int kb = kb_first; kb <= b_max_b; kb += PF_BN) {
-            // ---- stage K (8-bit, as is) and V (f16 * row scale) in LDS ----------------------------------
-            __syncthreads();
+        const int n_tiles = (b_max_b - kb_first) / PF_BN + 1;
+
+        // ---- staging: global -> registers -> LDS (K as is; V widened to f16 * row scale) -----------------
+        v4i rk[NLD], rv[NLD];
+        float rvs[NLD], rks = 0.0f;
+        auto load_tile = [&](int kb) {
 #pragma unroll
-            for (int i = 0; i < (PF_BN * CHUNKS) / PF_THREADS; ++i) {
-                int ch = tid + i * PF_THREADS;
-                int r = ch / CHUNKS, c = ch % CHUNKS;
-                int key = min(kb + r, p.n_tokens - 1);
-                v4i kraw = *(const v4i *)(p.k + (int64_t)key * p.k_pitch + hoff + c * 16);
-                v4i vraw = *(const v4i *)(p.v + (int64_t)key * p.v_pitch + hoff + c * 16);
-                float vs = p.vs ? p.vs[(int64_t)head * p.scale_pitch + key] : p.vs_const;
-                *(v4i *)(k_lds + r * L::K_PITCH + c * 16) = kraw;
-                v8h lo, hi;
-                widen_v<DTYPE>(vraw, vs, lo, hi);
-                *(v8h *)(v_lds + r * L::V_PITCH + c * 32) = lo;
-                *(v8h *)(v_lds + r * L::V_PITCH + c * 32 + 16) = hi;
+            for (int i = 0; i < NLD; ++i) {
+                const int ch = tid + i * PF_THREADS;
+                const int r = ch / CHUNKS, c = ch % CHUNKS;
+                const int key = min(kb + r, p.n_tokens - 1);
+                rk[i] = *(const v4i *)(p.k + (int64_t)key * p.k_pitch + hoff + c * 16);
+                rv[i] = *(const v4i *)(p.v + (int64_t)key * p.v_pitch + hoff + c * 16);
+                rvs[i] = p.vs ? p.vs[(int64_t)head * p.scale_pitch + key] : p.vs_const;
             }
             if (tid < PF_BN) {
-                int key = min(kb + tid, p.n_tokens - 1);
-                float ks = p.ks ? p.ks[(int64_t)head * p.scale_pitch + key] : p.ks_const;
-                ks_lds[tid] = ks * ads;
+                const int key = min(kb + tid, p.n_tokens - 1);
+                rks = p.ks ? p.ks[(int64_t)head * p.scale_pitch + key] : p.ks_const;
             }
-            __syncthreads();
+        };
+        auto store_tile = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int ch = tid + i * PF_THREADS;
+                const int r = ch / CHUNKS, c = ch % CHUNKS;
+                *(v4i *)(k_lds[buf] + r * L::K_PITCH + c * 16) = rk[i];
+                v8h lo, hi;
+                widen_v<DTYPE>(rv[i], rvs[i], lo, hi);
+                *(v8h *)(v_lds[buf] + r * L::V_PITCH + c * 32) = lo;
+                *(v8h *)(v_lds[buf] + r * L::V_PITCH + c * 32 + 16) = hi;
+            }
+            if (tid < PF_BN) ks_lds[buf][tid] = rks * ads;
+        };
 
-            // ---- does this wave need the tile at all, and does it need the mask? -----------------------
-            if (kb + PF_BN - 1 < w_min_a || kb > w_max_b) continue;
-            const bool interior = w_all_have_keys && (kb >= w_max_a) && (kb + PF_BN - 1 <= w_min_b);
-
-            // ---- S^T = K . Q^T, scale, mask ---------------------------------------------------------------
-            float s[2][16];
+        // ---- one 64-key tile for this wave's 32 queries ---------------------------------------------------
+        auto compute_tile = [&](auto interior_tag, int buf, int kb) {
+            constexpr bool INTERIOR = decltype(interior_tag)::value;
+            float t[2][16];
             float tmax = -INFINITY;
+            // keys of register r of sub-tile kt: kb + kt*32 + 8*(r/4) + 4*g + r%4
+            const int rel_a = sp_a - kb - 4 * g;            // span start relative to this lane's first key
+            const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
+            const float dist0 = (float)(from - kb - 4 * g);
+            const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
-                typename Qk::acc_t acc = qk.mma(k_lds + (kt * 32 + qi) * L::K_PITCH, g);
+                typename Qk::acc_t acc = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
 #pragma unroll
                 for (int c4 = 0; c4 < 4; ++c4) {
-                    const int koff = kt * 32 + 8 * c4 + 4 * g;
-                    v4f ksv = *(const v4f *)(ks_lds + koff);
+                    const int off0 = kt * 32 + 8 * c4;
+                    v4f ksv = *(const v4f *)(ks_lds[buf] + off0 + 4 * g);
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const int r = c4 * 4 + j;
-                        const int key = kb + koff + j;
+                        const int off = off0 + j;
+                        const bool in_span = INTERIOR || ((unsigned)(off - rel_a) <= span_w && has_keys);
                         if (DUMP) {
-                            if (row_ok && key >= sp_a && key <= sp_b) {
-                                ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + key] = Qk::bits(acc, r);
+                            if (in_span) {
+                                ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + kb + off + 4 * g] = Qk::bits(acc, r);
                             }
                         }
-                        float dp = Qk::to_float(acc, r) * ksv[j] * qs - p.slope * (float)(from - key);
-                        if (!interior) {
-                            dp = (key >= sp_a && key <= sp_b) ? dp : -INFINITY;
-                        }
-                        s[kt][r] = dp;
-                        tmax = fmaxf(tmax, dp);
+                        float x = Qk::to_float(acc, r) * ksv[j];
+                        float tv = fmaf(x, qs, base);
+                        if (SLOPE) tv += p.slope * (float)off;
+                        if (!INTERIOR) tv = in_span ? tv : -INFINITY;
+                        t[kt][r] = tv;
+                        tmax = fmaxf(tmax, tv);
                     }
                 }
             }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-            const float m_new = fmaxf(m, tmax);
-            if (__any(m_new != m)) {
-                const float alpha = fast_exp2(m - m_new);
+            if (__any(tmax > PF_RESCALE_THRESHOLD)) {
+                const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
+                const float alpha = fast_exp2(-shift);
+                m_ref += shift;
                 l *= alpha;
 #pragma unroll
                 for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) t[kt][r] -= shift;
             }
-            m = m_new;
-
-            // ---- P = 2^(S - m), O^T += V^T . P^T --------------------------------------------------------------
+            // P = 2^t ; O^T += V^T . P^T
+            const int i16 = lane & 15, dh = (lane >> 4) & 1;
+            const v2h ones = v2h{(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    float pw[8];
+                    v2h pp[4];
 #pragma unroll
-                    for (int x = 0; x < 8; ++x) {
-                        pw[x] = fast_exp2(s[kt][8 * i + x] - m_new);
-                        l += pw[x];
+                    for (int x = 0; x < 4; ++x) {
+                        const float p0 = fast_exp2(t[kt][8 * i + 2 * x]);
+                        const float p1 = fast_exp2(t[kt][8 * i + 2 * x + 1]);
+                        pp[x] = v2h{(_Float16)p0, (_Float16)p1};
+                        l = __builtin_amdgcn_fdot2(pp[x], ones, l, false); // sum of the weights the MFMA sees
                     }
-                    v8h pb = v8h{(_Float16)pw[0], (_Float16)pw[1], (_Float16)pw[2], (_Float16)pw[3],
-                                 (_Float16)pw[4], (_Float16)pw[5], (_Float16)pw[6], (_Float16)pw[7]};
+                    const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
                     // keys of this MFMA for lane group g: kt*32 + 16*i + 4*g + {0..3} and the same + 8
-                    const int i16 = lane & 15, dh = (lane >> 4) & 1;
                     const int key0 = kt * 32 + 16 * i + 4 * g + (i16 >> 2);
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
-                        const uint8_t *base = v_lds + key0 * L::V_PITCH + (dt * 32 + 16 * dh + 4 * (i16 & 3)) * 2;
-                        v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(base));
-                        v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(base + 8 * L::V_PITCH));
+                        const uint8_t *vb = v_lds[buf] + key0 * L::V_PITCH + (dt * 32 + 16 * dh + 4 * (i16 & 3)) * 2;
+                        v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb));
+                        v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb + 8 * L::V_PITCH));
                         v8h va = __builtin_bit_cast(v8h, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
                         o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb, o_acc[dt], 0, 0, 0);
                     }
                 }
             }
+        };
+
+        load_tile(kb_first);
+        store_tile(0);
+        if (n_tiles > 1) load_tile(kb_first + PF_BN);
+        __syncthreads();
+        for (int it = 0; it < n_tiles; ++it) {
+            const int buf = it & 1;
+            const int kb = kb_first + it * PF_BN;
+            // does this wave need the tile at all, and does it need the per-element mask?
+            if (!(kb + PF_BN - 1 < w_min_a || kb > w_max_b)) {
+                const bool interior = w_all_have_keys && (kb >= w_max_a) && (kb + PF_BN - 1 <= w_min_b);
+                if (interior) compute_tile(std::true_type{}, buf, kb);
+                else compute_tile(std::false_type{}, buf, kb);
+            }
+            if (it + 1 < n_tiles) store_tile(buf ^ 1);
+            if (it + 2 < n_tiles) load_tile(kb + 2 * PF_BN);
+            __syncthreads();
         }
     }
 
     // ---- epilogue: add the zero vector's weight, normalise, store -----------------------------------
     float l_all = l + __shfl_xor(l, 32, WAVE);
-    l_all += fast_exp2(-m);
+    l_all += fast_exp2(-m_ref);
     const float inv = 1.0f / l_all;
     if (row_ok) {
 #pragma unroll
@@ -309,24 +356,32 @@ __global__ __launch_bounds__(PF_THREADS) void prefill_kernel(PrefillParams p)
             }
         }
         if (p.sum_weight_log && g == 0) {
-            p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m + __log2f(l_all);
+            p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m_ref + __log2f(l_all);
         }
+    }
+}
+
+template <int DTYPE, int D, bool OUT_F16>
+static void launch_prefill_do(const PrefillParams &p, dim3 grid, hipStream_t st)
+{
+    const bool dump = p.dbg != nullptr;
+    const bool slope = p.slope != 0.0f;
+    dim3 block(PF_THREADS);
+    if (dump) {
+        // the debug variant always takes the general (slope) path
+        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true>), grid, block, 0, st, p);
+    } else if (slope) {
+        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false>), grid, block, 0, st, p);
+    } else {
+        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false>), grid, block, 0, st, p);
     }
 }
 
 template <int DTYPE, int D>
 static void launch_prefill_dd(const PrefillParams &p, int out_dtype, dim3 grid, hipStream_t st)
 {
-    const bool dump = p.dbg != nullptr;
-    const bool f16 = out_dtype == TSATTN_OUT_F16;
-    dim3 block(PF_THREADS);
-    if (f16) {
-        if (dump) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, true, true>), grid, block, 0, st, p);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, true, false>), grid, block, 0, st, p);
-    } else {
-        if (dump) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, false, true>), grid, block, 0, st, p);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, false, false>), grid, block, 0, st, p);
-    }
+    if (out_dtype == TSATTN_OUT_F16) launch_prefill_do<DTYPE, D, true>(p, grid, st);
+    else launch_prefill_do<DTYPE, D, false>(p, grid, st);
 }
 
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int head_dim, int out_dtype, hipStream_t st)
