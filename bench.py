@@ -128,8 +128,9 @@ class DecodeWorkload:
 
 
 def cpu_baseline_prefill(wl, n_seq_sample):
-    """The oracle (a port of the reference's CPU attention) on the first sequences of layer 0 (window 64)
-    and layer 1 (full causal window), all host threads."""
+    """The oracle (a port of the reference's CPU attention) on the same quantised inputs: the first
+    `n_seq_sample` sequences of every layer of the pass, all host threads; plus one sequence of one
+    full-window layer on a single thread (the reference's CPU path has no threading)."""
     import numpy as np
     from oracle import pyoracle as orc
     S, H, d = wl.S, wl.H, wl.d
@@ -137,7 +138,8 @@ def cpu_baseline_prefill(wl, n_seq_sample):
     threads = orc.max_threads()
     flops = 0.0
     t_total = 0.0
-    for li in (0, 1):
+    layers_done = 0
+    for li in range(len(wl.layers)):
         (q, qs), (k, ks), (v, vs) = wl.inputs[li]
         W, slope = wl.layers[li]
         hq, hk, hv = (x[:n].cpu().numpy() for x in (q, k, v))
@@ -147,8 +149,9 @@ def cpu_baseline_prefill(wl, n_seq_sample):
         orc.prefill_q8(wl.dtype, hq, hk, hv, H, hqs, hks, hvs, st, fi, slope, n_threads=threads)
         t_total += time.perf_counter() - t0
         flops += prefill_flops(n_seq_sample, S, H, d, W)
-    t1 = None
-    # single thread (the reference's CPU path has no threading): one sequence of the wide layer
+        layers_done += 1
+        if t_total > 20.0 and layers_done % 2 == 0:
+            break
     (q, qs), (k, ks), (v, vs) = wl.inputs[1]
     hq, hk, hv = (x[:S].cpu().numpy() for x in (q, k, v))
     hqs, hks, hvs = (np.ascontiguousarray(x[:, :S].cpu().numpy()) for x in (qs, ks, vs))
@@ -158,10 +161,10 @@ def cpu_baseline_prefill(wl, n_seq_sample):
     t1 = time.perf_counter() - t0
     return {
         "value": flops / t_total / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "sample": f"{n_seq_sample} of {wl.B} sequences, one window-64 layer + one full-window layer, "
+        "sample": f"{n_seq_sample} of {wl.B} sequences, {layers_done} of {len(wl.layers)} layers, "
                   f"{threads} OpenMP threads, {t_total:.2f} s",
         "single_thread_value": prefill_flops(1, S, H, d, S) / t1 / 1e12,
-        "single_thread_sample": f"1 sequence, full-window layer, {t1:.2f} s",
+        "single_thread_sample": f"1 sequence, one full-window layer, 1 thread, {t1:.2f} s",
     }
 
 
@@ -187,6 +190,36 @@ def cpu_baseline_decode(wl, n_seq_sample, reps):
                       f"{threads} OpenMP threads, {t * reps:.2f} s"}
 
 
+def run_only(ctx, args):
+    """Profiling aid: one kind of launch, repeated; used for the rocprofv3 runs recorded in profiles/."""
+    from tscale_amd import capi
+    name = args.only
+    if args.calibrate:
+        # a plain copy of known size in the same profile: 256 MiB read + 256 MiB written
+        import torch
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+    if name == "decode":
+        dw = DecodeWorkload(ctx, 64, 4096, 16, 128, n_caches=4, seed=1313 + 3)
+        ms = gpu_time_ms(dw.step, args.steps, args.warmup)
+        print(json.dumps({"only": name, "ms": ms, "GB/s": dw.bytes / ms / 1e6}))
+        return
+    if name == "c1-int8":
+        wl = PrefillWorkload(ctx, capi.I8, 1, 1024, 12, 64, 2, seed=1313 + 1)
+        li = 1
+    elif name.startswith("c2"):
+        wl = PrefillWorkload(ctx, capi.E4M3, 16, 1024, 12, 64, 2, seed=1313 + 2)
+        li = 0 if name.endswith("short") else 1
+    else:
+        wl = PrefillWorkload(ctx, capi.E4M3, 8, 4096, 16, 128, 2, seed=1313 + 4, short=256)
+        li = 0 if name.endswith("short") else 1
+    ms = gpu_time_ms(lambda: wl.run_layer(li), args.steps, args.warmup)
+    print(json.dumps({"only": name, "ms": ms, "TFLOP/s": wl.flops_layer[li] / ms / 1e9}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -195,6 +228,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--extra", action="store_true", help="also time the 1.5B-style prefill shapes")
+    ap.add_argument("--only", default=None,
+                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode"],
+                    help="profiling aid: run just this launch --steps times and print its timing")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="with --only: first run three 256 MiB device copies (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -206,6 +244,9 @@ def main():
         print("bench.py: no HIP device", file=sys.stderr)
         sys.exit(1)
     ctx = AttentionContext(0, max_seqs=64, max_heads=16, max_head_dim=128, max_splits=32)
+    if args.only:
+        run_only(ctx, args)
+        return
 
     # ---- prefill, 125M-style -----------------------------------------------------------------
     B, S, H, d, NL = 16, 1024, 12, 64, 12
@@ -232,7 +273,7 @@ def main():
                      "launch_ms": round(launch_ms, 5), "flops_per_launch": wl.flops / NL},
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline_prefill(wl, 4)
+        result["cpu_baseline"] = cpu_baseline_prefill(wl, 16)
     del wl
     torch.cuda.empty_cache()
 
@@ -249,7 +290,7 @@ def main():
                             "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(gbps / PEAK_HBM_GBPS, 5),
                             "traffic": MEASURED_TRAFFIC["decode_c3"], "bytes_per_launch": dw.bytes}}
         if not args.no_cpu:
-            dec["cpu_baseline"] = cpu_baseline_decode(dw, 8, 3)
+            dec["cpu_baseline"] = cpu_baseline_decode(dw, 64, 200)
         result["decode"] = dec
         del dw
         torch.cuda.empty_cache()

@@ -135,7 +135,7 @@ typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
 constexpr float PF_RESCALE_THRESHOLD = 8.0f;
 
 template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP>
-__global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p)
+__global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p, int n_qtiles)
 {
     typedef PfLayout<D> L;
     typedef QkMma<DTYPE, D> Qk;
@@ -153,8 +153,13 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p)
     const int wave = tid / WAVE;
     const int qi = lane & 31; // query column of this lane
     const int g = lane >> 5;  // which half of the contraction this lane feeds
-    const int head = blockIdx.y;
-    const int tile = (int)gridDim.x - 1 - (int)blockIdx.x; // long rows first
+    // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of
+    // (head, query tile) pairs: equal work per XCD, and the K/V rows a run shares stay in its L2.
+    int wg = blockIdx.x;
+    const int n_wg = gridDim.x;
+    if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
+    const int head = wg / n_qtiles;
+    const int tile = n_qtiles - 1 - (wg % n_qtiles); // long rows first
     const int q0 = tile * PF_BM + wave * 32;
     const int from = q0 + qi;
     const bool row_ok = from < p.n_tokens;
@@ -208,19 +213,39 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p)
         // ---- staging: global -> registers -> LDS (K as is; V widened to f16 * row scale) -----------------
         v4i rk[NLD], rv[NLD];
         float rvs[NLD], rks = 0.0f;
-        auto load_tile = [&](int kb) {
+        // Row offsets advance by one tile per load; rows past the last token re-read the last row
+        // (their logits are masked), so no multiply is needed inside the loop.
+        const int64_t k_last = (int64_t)(p.n_tokens - 1) * p.k_pitch, v_last = (int64_t)(p.n_tokens - 1) * p.v_pitch;
+        int64_t k_off[NLD], v_off[NLD];
+        int s_idx[NLD];
+        const uint8_t *k_base[NLD], *v_base[NLD];
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int ch = tid + i * PF_THREADS;
+            const int r = ch / CHUNKS, c = ch % CHUNKS;
+            k_off[i] = (int64_t)(kb_first + r) * p.k_pitch;
+            v_off[i] = (int64_t)(kb_first + r) * p.v_pitch;
+            s_idx[i] = kb_first + r;
+            k_base[i] = p.k + hoff + c * 16;
+            v_base[i] = p.v + hoff + c * 16;
+        }
+        int ks_idx = kb_first + tid;
+        const float *vs_row = p.vs ? p.vs + (int64_t)head * p.scale_pitch : nullptr;
+        const float *ks_row = p.ks ? p.ks + (int64_t)head * p.scale_pitch : nullptr;
+        const int64_t k_step = (int64_t)PF_BN * p.k_pitch, v_step = (int64_t)PF_BN * p.v_pitch;
+        auto load_tile = [&]() { // loads the next tile in sequence
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
-                const int ch = tid + i * PF_THREADS;
-                const int r = ch / CHUNKS, c = ch % CHUNKS;
-                const int key = min(kb + r, p.n_tokens - 1);
-                rk[i] = *(const v4i *)(p.k + (int64_t)key * p.k_pitch + hoff + c * 16);
-                rv[i] = *(const v4i *)(p.v + (int64_t)key * p.v_pitch + hoff + c * 16);
-                rvs[i] = p.vs ? p.vs[(int64_t)head * p.scale_pitch + key] : p.vs_const;
+                rk[i] = *(const v4i *)(k_base[i] + (k_off[i] < k_last ? k_off[i] : k_last));
+                rv[i] = *(const v4i *)(v_base[i] + (v_off[i] < v_last ? v_off[i] : v_last));
+                rvs[i] = vs_row ? vs_row[min(s_idx[i], p.n_tokens - 1)] : p.vs_const;
+                k_off[i] += k_step;
+                v_off[i] += v_step;
+                s_idx[i] += PF_BN;
             }
             if (tid < PF_BN) {
-                const int key = min(kb + tid, p.n_tokens - 1);
-                rks = p.ks ? p.ks[(int64_t)head * p.scale_pitch + key] : p.ks_const;
+                rks = ks_row ? ks_row[min(ks_idx, p.n_tokens - 1)] : p.ks_const;
+                ks_idx += PF_BN;
             }
         };
         auto store_tile = [&](int buf) {
@@ -316,9 +341,9 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p)
             }
         };
 
-        load_tile(kb_first);
+        load_tile();
         store_tile(0);
-        if (n_tiles > 1) load_tile(kb_first + PF_BN);
+        if (n_tiles > 1) load_tile();
         __syncthreads();
         for (int it = 0; it < n_tiles; ++it) {
             const int buf = it & 1;
@@ -330,7 +355,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p)
                 else compute_tile(std::false_type{}, buf, kb);
             }
             if (it + 1 < n_tiles) store_tile(buf ^ 1);
-            if (it + 2 < n_tiles) load_tile(kb + 2 * PF_BN);
+            if (it + 2 < n_tiles) load_tile();
             __syncthreads();
         }
     }
@@ -362,18 +387,20 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p)
 }
 
 template <int DTYPE, int D, bool OUT_F16>
-static void launch_prefill_do(const PrefillParams &p, dim3 grid, hipStream_t st)
+static void launch_prefill_do(const PrefillParams &p, dim3 grid2, hipStream_t st)
 {
+    const int n_qtiles = (int)grid2.x;
+    dim3 grid(grid2.x * grid2.y);
     const bool dump = p.dbg != nullptr;
     const bool slope = p.slope != 0.0f;
     dim3 block(PF_THREADS);
     if (dump) {
         // the debug variant always takes the general (slope) path
-        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true>), grid, block, 0, st, p, n_qtiles);
     } else if (slope) {
-        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false>), grid, block, 0, st, p, n_qtiles);
     } else {
-        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false>), grid, block, 0, st, p, n_qtiles);
     }
 }
 
