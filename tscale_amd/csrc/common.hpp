@@ -33,6 +33,15 @@ __device__ inline float fast_exp2(float x)
     return __builtin_amdgcn_exp2f(x); // v_exp_f32
 }
 
+// Two-operand maximum kept out of the compiler's v_max3_f32 fusion: VALU instructions that read
+// three different VGPRs do not execute alongside an MFMA on gfx950, two-operand ones do.
+__device__ inline float max2(float a, float b)
+{
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 __device__ inline float bf16_to_float(uint16_t b)
 {
     return __uint_as_float((uint32_t)b << 16);

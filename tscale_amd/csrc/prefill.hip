@@ -204,7 +204,8 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
 #pragma unroll
     for (int i = 0; i < DT; ++i) o_acc[i] = v16f{0};
     float m_ref = 0.0f; // reference maximum: starts at the zero vector's logit
-    float l = 0.0f;     // this lane's share of the weight sum (its 32 of every 64 keys)
+    bool have_ref = false; // wave-uniform: some lane of this wave has m_ref != 0
+    float l = 0.0f, l2 = 0.0f; // this lane's share of the weight sum (its 32 of every 64 keys), in two chains
 
     if (b_max_b >= b_min_a) {
         const int kb_first = (b_min_a / PF_BN) * PF_BN;
@@ -262,9 +263,25 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
             if (tid < PF_BN) ks_lds[buf][tid] = rks * ads;
         };
 
+        // V^T operands (A of the P.V MFMA) of one group: keys kt*32 + 16*i + 4*g + {0..3} and the same + 8
+        const int i16 = lane & 15, dh = (lane >> 4) & 1;
+        v8h va[2][DT];
+        auto vload = [&](int slot, int grp, int buf) {
+            const int kt = grp >> 1, i = grp & 1;
+            const int key0 = kt * 32 + 16 * i + 4 * g + (i16 >> 2);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint8_t *vb = v_lds[buf] + key0 * L::V_PITCH + (dt * 32 + 16 * dh + 4 * (i16 & 3)) * 2;
+                v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb));
+                v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb + 8 * L::V_PITCH));
+                va[slot][dt] = __builtin_bit_cast(v8h, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+            }
+        };
+
         // ---- one 64-key tile for this wave's 32 queries ---------------------------------------------------
-        auto compute_tile = [&](auto interior_tag, int buf, int kb) {
+        auto compute_tile = [&](auto interior_tag, auto ref_tag, int buf, int kb) {
             constexpr bool INTERIOR = decltype(interior_tag)::value;
+            constexpr bool REF = decltype(ref_tag)::value || SLOPE; // general form: logit * qs + base
             float t[2][16];
             float tmax = -INFINITY;
             // keys of register r of sub-tile kt: kb + kt*32 + 8*(r/4) + 4*g + r%4
@@ -272,9 +289,15 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
             const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
             const float dist0 = (float)(from - kb - 4 * g);
             const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
+            typename Qk::acc_t accs[2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) accs[kt] = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
+            vload(0, 0, buf);
+            vload(1, 1, buf);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
-                typename Qk::acc_t acc = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
+                typename Qk::acc_t acc = accs[kt];
 #pragma unroll
                 for (int c4 = 0; c4 < 4; ++c4) {
                     const int off0 = kt * 32 + 8 * c4;
@@ -289,12 +312,13 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
                                 ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + kb + off + 4 * g] = Qk::bits(acc, r);
                             }
                         }
+                        // while the reference maximum is still 0 (no slope): two 2-operand multiplies
                         float x = Qk::to_float(acc, r) * ksv[j];
-                        float tv = fmaf(x, qs, base);
+                        float tv = REF ? fmaf(x, qs, base) : x * qs;
                         if (SLOPE) tv += p.slope * (float)off;
                         if (!INTERIOR) tv = in_span ? tv : -INFINITY;
                         t[kt][r] = tv;
-                        tmax = fmaxf(tmax, tv);
+                        tmax = max2(tmax, tv);
                     }
                 }
             }
@@ -302,8 +326,10 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
             if (__any(tmax > PF_RESCALE_THRESHOLD)) {
                 const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
                 const float alpha = fast_exp2(-shift);
+                have_ref = true;
                 m_ref += shift;
                 l *= alpha;
+                l2 *= alpha;
 #pragma unroll
                 for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
 #pragma unroll
@@ -311,33 +337,25 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
 #pragma unroll
                     for (int r = 0; r < 16; ++r) t[kt][r] -= shift;
             }
-            // P = 2^t ; O^T += V^T . P^T
-            const int i16 = lane & 15, dh = (lane >> 4) & 1;
-            const v2h ones = v2h{(_Float16)1.0f, (_Float16)1.0f};
+            // P = 2^t ; O^T += V^T . P^T in four groups of DT MFMAs (16 keys each).  The V^T operands of a
+            // group are read from LDS two groups ahead (ring of two register sets) so that no MFMA waits
+            // for an LDS round trip.
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
+            for (int grp = 0; grp < 4; ++grp) {
+                const int kt = grp >> 1, i = grp & 1;
+                v2h pp[4];
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    v2h pp[4];
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        const float p0 = fast_exp2(t[kt][8 * i + 2 * x]);
-                        const float p1 = fast_exp2(t[kt][8 * i + 2 * x + 1]);
-                        pp[x] = v2h{(_Float16)p0, (_Float16)p1};
-                        l = __builtin_amdgcn_fdot2(pp[x], ones, l, false); // sum of the weights the MFMA sees
-                    }
-                    const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
-                    // keys of this MFMA for lane group g: kt*32 + 16*i + 4*g + {0..3} and the same + 8
-                    const int key0 = kt * 32 + 16 * i + 4 * g + (i16 >> 2);
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        const uint8_t *vb = v_lds[buf] + key0 * L::V_PITCH + (dt * 32 + 16 * dh + 4 * (i16 & 3)) * 2;
-                        v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb));
-                        v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb + 8 * L::V_PITCH));
-                        v8h va = __builtin_bit_cast(v8h, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
-                        o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb, o_acc[dt], 0, 0, 0);
-                    }
+                for (int x = 0; x < 4; ++x) {
+                    const float p0 = fast_exp2(t[kt][8 * i + 2 * x]);
+                    const float p1 = fast_exp2(t[kt][8 * i + 2 * x + 1]);
+                    pp[x] = v2h{(_Float16)p0, (_Float16)p1};
+                    l += p0;
+                    l2 += p1;
                 }
+                const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[grp & 1][dt], pb, o_acc[dt], 0, 0, 0);
+                if (grp + 2 < 4) vload(grp & 1, grp + 2, buf);
             }
         };
 
@@ -351,8 +369,9 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
             // does this wave need the tile at all, and does it need the per-element mask?
             if (!(kb + PF_BN - 1 < w_min_a || kb > w_max_b)) {
                 const bool interior = w_all_have_keys && (kb >= w_max_a) && (kb + PF_BN - 1 <= w_min_b);
-                if (interior) compute_tile(std::true_type{}, buf, kb);
-                else compute_tile(std::false_type{}, buf, kb);
+                if (interior && !have_ref) compute_tile(std::true_type{}, std::false_type{}, buf, kb);
+                else if (interior) compute_tile(std::true_type{}, std::true_type{}, buf, kb);
+                else compute_tile(std::false_type{}, std::true_type{}, buf, kb);
             }
             if (it + 1 < n_tiles) store_tile(buf ^ 1);
             if (it + 2 < n_tiles) load_tile();
@@ -361,6 +380,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
     }
 
     // ---- epilogue: add the zero vector's weight, normalise, store -----------------------------------
+    l += l2;
     float l_all = l + __shfl_xor(l, 32, WAVE);
     l_all += fast_exp2(-m_ref);
     const float inv = 1.0f / l_all;
