@@ -1,0 +1,183 @@
+// GPU test of the C++ host mirror (tscale_amd/host/att_compute.h) against the CPU oracle, written
+// the way the reference drives its own contexts: build the attention spans of a batch of fragments,
+// run the prefill attention of one layer, then replay the same tokens one at a time through the
+// KV cache and compare every decoded row with its prefill row (the comparison NCPUInfer::Check
+// makes at model level, gpt/train/cpu_infer.cpp:658-683).
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+#include "../../oracle/tsattn_oracle.h"
+#include "../../tscale_amd/host/att_compute.h"
+
+using namespace NTsAttn;
+
+#define HIP_OK(x)                                                                 \
+    do {                                                                          \
+        hipError_t e_ = (x);                                                      \
+        if (e_ != hipSuccess) {                                                   \
+            printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            exit(2);                                                              \
+        }                                                                         \
+    } while (0)
+
+template <class T>
+static T *ToDevice(const std::vector<T> &v)
+{
+    T *d = nullptr;
+    HIP_OK(hipMalloc((void **)&d, v.size() * sizeof(T)));
+    HIP_OK(hipMemcpy(d, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice));
+    return d;
+}
+
+static float Gauss(unsigned &s)
+{
+    float u = 0;
+    for (int i = 0; i < 12; ++i) {
+        s = s * 1664525u + 1013904223u;
+        u += (s >> 8) * (1.0f / 16777216.0f);
+    }
+    return u - 6.0f;
+}
+
+static int RunCase(int dtype, int window, float slope)
+{
+    const int H = 2, d = 128;
+    const int fragLen[2] = {150, 90};
+    const int len = fragLen[0] + fragLen[1];
+    TModelDims dims;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = H * d;
+
+    // inputs: N(0,1) rows quantised with the absmax rule
+    unsigned seed = 1313u + dtype * 7 + window;
+    std::vector<float> x((size_t)len * H * d);
+    std::vector<uint8_t> q(x.size()), k(x.size()), v(x.size());
+    std::vector<float> qs((size_t)H * len), ks(qs.size()), vs(qs.size());
+    for (auto *dst : {&q, &k, &v}) {
+        for (float &f : x) f = Gauss(seed);
+        float *sc = dst == &q ? qs.data() : dst == &k ? ks.data() : vs.data();
+        tso_quantize_rows(dtype, x.data(), H * d, len, H, d, dst->data(), H * d, sc, len);
+    }
+
+    // spans of the batch, fragment by fragment
+    TAttentionInfo att;
+    att.Init();
+    AddWindowSpans(0, fragLen[0], window, nullptr, &att);
+    AddWindowSpans(fragLen[0], fragLen[1], window, nullptr, &att);
+    std::vector<int32_t> st(len), fi(len);
+    for (int t = 0; t < len; ++t) {
+        int a = att.SpanPtr[t], b = att.SpanPtr[t + 1];
+        st[t] = b > a ? att.Spans[a].Start : t;
+        fi[t] = b > a ? att.Spans[a].Finish : t - 1;
+    }
+
+    // oracle
+    std::vector<float> want((size_t)len * H * d);
+    tso_prefill_q8(dtype, len, H, d, q.data(), k.data(), v.data(), H * d, qs.data(), ks.data(), vs.data(), len, 0, 0, 0,
+                   st.data(), fi.data(), slope, want.data(), H * d, nullptr, 4);
+
+    // GPU prefill through the host mirror
+    TAttentionComputer attComp(dims, slope, 0, len, 2);
+    attComp.SetAttention(att, nullptr);
+    uint8_t *dq = ToDevice(q), *dk = ToDevice(k), *dv = ToDevice(v);
+    float *dqs = ToDevice(qs), *dks = ToDevice(ks), *dvs = ToDevice(vs);
+    float *dout = nullptr;
+    HIP_OK(hipMalloc((void **)&dout, want.size() * sizeof(float)));
+    TQuantRows rq, rk, rv;
+    rq.Data = dq; rq.PitchBytes = H * d; rq.Scale = dqs;
+    rk.Data = dk; rk.PitchBytes = H * d; rk.Scale = dks;
+    rv.Data = dv; rv.PitchBytes = H * d; rv.Scale = dvs;
+    attComp.ComputeValLookup(len, dtype, rq, rk, rv, nullptr, dout, (int64_t)H * d * sizeof(float), false, nullptr);
+    std::vector<float> got(want.size());
+    HIP_OK(hipMemcpy(got.data(), dout, got.size() * sizeof(float), hipMemcpyDeviceToHost));
+
+    double sum = 0, sum2 = 0;
+    for (float f : want) { sum += f; sum2 += (double)f * f; }
+    double sd = sqrt(sum2 / want.size() - (sum / want.size()) * (sum / want.size()));
+    double maxErr = 0, meanErr = 0;
+    for (size_t i = 0; i < want.size(); ++i) {
+        double e = fabs(got[i] - want[i]) / sd;
+        maxErr = e > maxErr ? e : maxErr;
+        meanErr += e;
+    }
+    meanErr /= want.size();
+    int fails = 0;
+    if (!(maxErr <= 2e-2 && meanErr <= 2e-3)) {
+        printf("  prefill mismatch: max %.3e mean %.3e\n", maxErr, meanErr);
+        ++fails;
+    }
+
+    // decode replay: both fragments advance in lock step through a two-sequence cache
+    const int steps = fragLen[1];
+    TAttentionVecHistory cache(attComp.GetHandle(), dtype, 2, H, steps, d);
+    std::vector<uint8_t> stepK(2 * H * d), stepV(2 * H * d), stepQ(2 * H * d);
+    std::vector<float> stepKs(2 * H), stepVs(2 * H), stepQs(2 * H);
+    uint8_t *dsk, *dsv, *dsq;
+    float *dsks, *dsvs, *dsqs, *dval;
+    HIP_OK(hipMalloc((void **)&dsk, stepK.size()));
+    HIP_OK(hipMalloc((void **)&dsv, stepV.size()));
+    HIP_OK(hipMalloc((void **)&dsq, stepQ.size()));
+    HIP_OK(hipMalloc((void **)&dsks, stepKs.size() * 4));
+    HIP_OK(hipMalloc((void **)&dsvs, stepVs.size() * 4));
+    HIP_OK(hipMalloc((void **)&dsqs, stepQs.size() * 4));
+    HIP_OK(hipMalloc((void **)&dval, 2 * H * d * sizeof(float)));
+    std::vector<float> val(2 * H * d);
+    double decMax = 0;
+    for (int t = 0; t < steps; ++t) {
+        for (int s = 0; s < 2; ++s) {
+            int row = (s == 0 ? 0 : fragLen[0]) + t;
+            memcpy(&stepK[s * H * d], &k[(size_t)row * H * d], H * d);
+            memcpy(&stepV[s * H * d], &v[(size_t)row * H * d], H * d);
+            memcpy(&stepQ[s * H * d], &q[(size_t)row * H * d], H * d);
+            for (int h = 0; h < H; ++h) {
+                stepKs[s * H + h] = ks[(size_t)h * len + row];
+                stepVs[s * H + h] = vs[(size_t)h * len + row];
+                stepQs[s * H + h] = qs[(size_t)h * len + row];
+            }
+        }
+        HIP_OK(hipMemcpy(dsk, stepK.data(), stepK.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dsv, stepV.data(), stepV.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dsq, stepQ.data(), stepQ.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dsks, stepKs.data(), stepKs.size() * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dsvs, stepVs.data(), stepVs.size() * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dsqs, stepQs.data(), stepQs.size() * 4, hipMemcpyHostToDevice));
+        cache.AddVectors(dsk, dsks, dsv, dsvs, nullptr);            // cpu_infer.cpp:506
+        ComputeValLookup(window, slope, cache, dsq, dsqs, 0, dval, nullptr); // cpu_infer.cpp:509
+        HIP_OK(hipMemcpy(val.data(), dval, val.size() * sizeof(float), hipMemcpyDeviceToHost));
+        for (int s = 0; s < 2; ++s) {
+            int row = (s == 0 ? 0 : fragLen[0]) + t;
+            for (int i = 0; i < H * d; ++i) {
+                double e = fabs(val[s * H * d + i] - want[(size_t)row * H * d + i]);
+                decMax = e > decMax ? e : decMax;
+            }
+        }
+    }
+    if (!(decMax < 1e-4)) {
+        printf("  decode replay mismatch: max abs %.3e\n", decMax);
+        ++fails;
+    }
+    printf("dtype %d window %d slope %.2f: prefill max %.2e mean %.2e, decode replay max abs %.2e %s\n", dtype, window, slope,
+           maxErr, meanErr, decMax, fails ? "FAIL" : "ok");
+    for (void *p : {(void *)dq, (void *)dk, (void *)dv, (void *)dqs, (void *)dks, (void *)dvs, (void *)dout, (void *)dsk, (void *)dsv,
+                    (void *)dsq, (void *)dsks, (void *)dsvs, (void *)dsqs, (void *)dval}) {
+        HIP_OK(hipFree(p));
+    }
+    return fails;
+}
+
+int main()
+{
+    int fails = 0;
+    for (int dtype : {TSATTN_I8, TSATTN_E4M3}) {
+        fails += RunCase(dtype, 64, 0.5f);
+        fails += RunCase(dtype, 1000, 0.0f);
+        fails += RunCase(dtype, 1, 0.0f);
+        fails += RunCase(dtype, 0, 0.0f);
+    }
+    printf(fails ? "FAILED %d\n" : "ALL OK\n", fails);
+    return fails ? 1 : 0;
+}

@@ -1,0 +1,129 @@
+// C++ host side of the attention path: keeps the shape of the reference's attention call sites so
+// that a model/layer implementation written against them can switch to the gfx950 kernels.
+//
+//   reference                                                     here
+//   TAttentionSpan / TAttentionInfo        gpt/att/att.h:4-47      NTsAttn::TAttentionSpan / TAttentionInfo
+//   AddAttSpans + GenerateAttentionGraph   gpt/att/sliding_window.cpp:80-87,205-223   NTsAttn::AddWindowSpans
+//   TAttentionComputer::ComputeValLookup   gpt/compute/gpt_cpu.cpp:391-441 (call :633),
+//   CudaCall(c, Fp8Att)...                 gpt/compute/gpt_cuda.cu:503-507            TAttentionComputer::ComputeValLookup
+//   TAttentionVecHistory::AddVectors       gpt/train/cpu_infer.cpp:397-410            TAttentionVecHistory::AddVectors
+//   ComputeValLookup (KV cache)            gpt/train/cpu_infer.cpp:413-460 (call :509) NTsAttn::ComputeValLookup
+//
+// All arithmetic runs in libtsattn.so through the C ABI of include/tsattn.h; this layer owns the
+// per-context device buffers (allocated once, like TAttentionComputeCtx::AllocateCuda,
+// gpt/compute/gpt_cuda.cu:231-302) and aborts on errors the way the reference's Y_VERIFY does.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include <vector>
+
+#include "../../include/tsattn.h"
+
+namespace NTsAttn {
+
+struct TAttentionSpan {
+    // inclusive borders
+    int Start = 0;
+    int Finish = 0;
+    TAttentionSpan() {}
+    TAttentionSpan(int start, int finish) : Start(start), Finish(finish) {}
+};
+
+struct TAttentionInfo {
+    std::vector<TAttentionSpan> Spans;
+    std::vector<int> SpanPtr;
+
+    void Init()
+    {
+        Spans.resize(0);
+        SpanPtr.assign(1, 0);
+    }
+    size_t GetSampleCount() const { return SpanPtr.size() - 1; }
+    bool IsEmpty() const { return SpanPtr.size() <= 1; }
+    void AddSpan(const TAttentionSpan &span) { Spans.push_back(span); }
+    void AddSample() { SpanPtr.push_back((int)Spans.size()); }
+};
+
+struct TModelDims {
+    int Dim = 256;
+    int QDim = 128;
+    int TTDim = 128;
+    int HeadCount = 1;
+    int GetQSum() const { return QDim * HeadCount; }
+    int GetTTSum() const { return TTDim * HeadCount; }
+};
+
+// Appends the samples of one fragment of `len` tokens that starts at node `ptr` of the batch:
+// token t sees [max(docStart, t - limitWindow), t - 1]; limitWindow == 0 means itself only;
+// docStartFlag (nullable, per token of the fragment) marks document starts inside the fragment.
+void AddWindowSpans(int ptr, int len, int limitWindow, const uint8_t *docStartFlag, TAttentionInfo *pAtt);
+
+// Quantised per-row operands as the projection epilogues leave them on the device.
+struct TQuantRows {
+    const void *Data = nullptr;   // [len][headCount*dim] 8-bit, device
+    int64_t PitchBytes = 0;
+    const float *Scale = nullptr; // [headCount][scalePitch] device, or nullptr = ConstScale
+    float ConstScale = 1;
+};
+
+class TAttentionComputer
+{
+    tsattn_handle_t Handle = nullptr;
+    TModelDims Dims;
+    float AlibiSlope = 0;
+    int MaxLen = 0;
+    int Len = 0;
+    int32_t *SpanStart = nullptr; // device
+    int32_t *SpanFinish = nullptr;
+    float *SumWeightLog = nullptr; // device [headCount][MaxLen]
+
+  public:
+    // maxSeqs > 0 also provisions the handle for KV-cache decode of that many sequences
+    TAttentionComputer(const TModelDims &dims, float alibiSlope, int deviceId, int maxLen, int maxSeqs = 0);
+    ~TAttentionComputer();
+    TAttentionComputer(const TAttentionComputer &) = delete;
+    TAttentionComputer &operator=(const TAttentionComputer &) = delete;
+
+    // Per batch, like TComputeContext::Init copying the spans to the device (gpt_cuda.cu:1362-1376).
+    // Rows with more than one span are not supported by the kernels and abort.
+    void SetAttention(const TAttentionInfo &attInfo, void *stream);
+
+    // valLookup: device [len][headCount*TTDim] fp32 (outF16 = false) or fp16.
+    void ComputeValLookup(int len, int dtype, const TQuantRows &qk, const TQuantRows &qv, const TQuantRows &v,
+                          const float *qvGlobalScale, void *valLookup, int64_t valLookupPitchBytes, bool outF16,
+                          void *stream);
+    const float *GetSumWeightLog() const { return SumWeightLog; }
+    int GetSumWeightLogPitch() const { return MaxLen; }
+    tsattn_handle_t GetHandle() const { return Handle; }
+};
+
+// Device-resident KV cache: planar [seq][head][maxLen][dim] 8-bit planes and [seq][head][maxLen] fp32
+// key and value row scales.
+struct TAttentionVecHistory {
+    tsattn_handle_t Handle = nullptr;
+    int DType = TSATTN_I8;
+    int SeqCount = 0, HeadCount = 0, MaxLen = 0, HeadDim = 0;
+    uint8_t *QVState = nullptr;        // keys
+    uint8_t *VState = nullptr;         // values
+    float *QVStateScale = nullptr;
+    float *VStateScale = nullptr;
+    int32_t *Length = nullptr;         // device [seqCount]
+    float *SplitAcc = nullptr;
+
+    TAttentionVecHistory(tsattn_handle_t handle, int dtype, int seqCount, int headCount, int maxLen, int headDim);
+    ~TAttentionVecHistory();
+    TAttentionVecHistory(const TAttentionVecHistory &) = delete;
+    TAttentionVecHistory &operator=(const TAttentionVecHistory &) = delete;
+
+    // qv, v: device [seqCount][headCount*headDim]; scales device [seqCount][headCount]
+    void AddVectors(const void *qv, const float *qvScale, const void *v, const float *vScale, void *stream);
+};
+
+// One new token per sequence; qk: device [seqCount][headCount*headDim] 8-bit with qkScale
+// [seqCount][headCount] (nullptr = qkConstScale).  valLookup: device [seqCount][headCount*headDim] fp32.
+void ComputeValLookup(int width, float alibiSlope, const TAttentionVecHistory &history, const void *qk,
+                      const float *qkScale, float qkConstScale, float *valLookup, void *stream);
+
+} // namespace NTsAttn
