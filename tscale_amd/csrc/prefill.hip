@@ -158,8 +158,11 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
     int wg = blockIdx.x;
     const int n_wg = gridDim.x;
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
-    const int head = wg / n_qtiles;
-    const int tile = n_qtiles - 1 - (wg % n_qtiles); // long rows first
+    // With d = 64 one 128-byte line of K or V holds the rows of two heads: consecutive workgroups then
+    // alternate between the two heads of a pair on the same query tile, so the pair shares the line in L2.
+    const int hg = (D == 64 && (p.n_heads & 1) == 0) ? 2 : 1;
+    const int head = (wg / (hg * n_qtiles)) * hg + wg % hg;
+    const int tile = n_qtiles - 1 - ((wg / hg) % n_qtiles); // long rows first
     const int q0 = tile * PF_BM + wave * 32;
     const int from = q0 + qi;
     const bool row_ok = from < p.n_tokens;
