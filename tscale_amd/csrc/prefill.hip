@@ -24,7 +24,14 @@ namespace tsattn {
 constexpr int PF_THREADS = 256;
 constexpr int PF_WAVES = 4;
 constexpr int PF_BM = 128; // queries per workgroup
-constexpr int PF_BN = 64;  // keys per tile
+#ifndef TSATTN_PF_BN
+#define TSATTN_PF_BN 64
+#endif
+#ifndef TSATTN_PF_OCC
+#define TSATTN_PF_OCC 2
+#endif
+constexpr int PF_BN = TSATTN_PF_BN;  // keys per tile (32 or 64)
+constexpr int PF_KT = PF_BN / 32; // 32-key sub-tiles per tile
 
 template <int D>
 struct PfLayout {
@@ -135,13 +142,14 @@ typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
 constexpr float PF_RESCALE_THRESHOLD = 8.0f;
 
 template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP>
-__global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p, int n_qtiles)
+__global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(PrefillParams p, int n_qtiles)
 {
     typedef PfLayout<D> L;
     typedef QkMma<DTYPE, D> Qk;
     constexpr int DT = D / 32;                               // 32-row tiles of O^T
     constexpr int CHUNKS = D / 16;                           // 16-byte chunks per 8-bit row
-    constexpr int NLD = (PF_BN * CHUNKS) / PF_THREADS;       // 16-byte chunks per thread per tile
+    constexpr int NLD = (PF_BN * CHUNKS + PF_THREADS - 1) / PF_THREADS;
+    constexpr bool LD_ALL = (PF_BN * CHUNKS) % PF_THREADS == 0; // every thread owns NLD chunks       // 16-byte chunks per thread per tile
 
     __shared__ __attribute__((aligned(16))) uint8_t k_lds[2][L::K_BYTES];
     __shared__ __attribute__((aligned(16))) uint8_t v_lds[2][L::V_BYTES];
@@ -240,6 +248,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
         auto load_tile = [&]() { // loads the next tile in sequence
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
+                if (!LD_ALL && tid + i * PF_THREADS >= PF_BN * CHUNKS) break;
                 rk[i] = *(const v4i *)(k_base[i] + (k_off[i] < k_last ? k_off[i] : k_last));
                 rv[i] = *(const v4i *)(v_base[i] + (v_off[i] < v_last ? v_off[i] : v_last));
                 rvs[i] = vs_row ? vs_row[min(s_idx[i], p.n_tokens - 1)] : p.vs_const;
@@ -256,6 +265,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
                 const int ch = tid + i * PF_THREADS;
+                if (!LD_ALL && ch >= PF_BN * CHUNKS) break;
                 const int r = ch / CHUNKS, c = ch % CHUNKS;
                 *(v4i *)(k_lds[buf] + r * L::K_PITCH + c * 16) = rk[i];
                 v8h lo, hi;
@@ -285,21 +295,21 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
         auto compute_tile = [&](auto interior_tag, auto ref_tag, int buf, int kb) {
             constexpr bool INTERIOR = decltype(interior_tag)::value;
             constexpr bool REF = decltype(ref_tag)::value || SLOPE; // general form: logit * qs + base
-            float t[2][16];
+            float t[PF_KT][16];
             float tmax = -INFINITY;
             // keys of register r of sub-tile kt: kb + kt*32 + 8*(r/4) + 4*g + r%4
             const int rel_a = sp_a - kb - 4 * g;            // span start relative to this lane's first key
             const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
             const float dist0 = (float)(from - kb - 4 * g);
             const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
-            typename Qk::acc_t accs[2];
+            typename Qk::acc_t accs[PF_KT];
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt) accs[kt] = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
+            for (int kt = 0; kt < PF_KT; ++kt) accs[kt] = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
             vload(0, 0, buf);
             vload(1, 1, buf);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt) {
+            for (int kt = 0; kt < PF_KT; ++kt) {
                 typename Qk::acc_t acc = accs[kt];
 #pragma unroll
                 for (int c4 = 0; c4 < 4; ++c4) {
@@ -325,8 +335,10 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
                     }
                 }
             }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+            // the two lanes of a query exchange their maxima only if some lane of the wave is over the
+            // threshold: the common path has no cross-lane operation at all
             if (__any(tmax > PF_RESCALE_THRESHOLD)) {
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
                 const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
                 const float alpha = fast_exp2(-shift);
                 have_ref = true;
@@ -336,7 +348,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
 #pragma unroll
                 for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
 #pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
+                for (int kt = 0; kt < PF_KT; ++kt)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) t[kt][r] -= shift;
             }
@@ -344,7 +356,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
             // group are read from LDS two groups ahead (ring of two register sets) so that no MFMA waits
             // for an LDS round trip.
 #pragma unroll
-            for (int grp = 0; grp < 4; ++grp) {
+            for (int grp = 0; grp < 2 * PF_KT; ++grp) {
                 const int kt = grp >> 1, i = grp & 1;
                 v2h pp[4];
 #pragma unroll
@@ -358,7 +370,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_kernel(PrefillParams p,
                 const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[grp & 1][dt], pb, o_acc[dt], 0, 0, 0);
-                if (grp + 2 < 4) vload(grp & 1, grp + 2, buf);
+                if (grp + 2 < 2 * PF_KT) vload(grp & 1, grp + 2, buf);
             }
         };
 
