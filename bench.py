@@ -127,6 +127,116 @@ class DecodeWorkload:
         self.ctx.compute_val_lookup_decode(c, self.q, None, 10 ** 6, 0.0, out=self.out)
 
 
+class GenerationWorkload:
+    """Attention share of the 1.5B-style greedy-decode configuration: 24 layers (InitAlibi's schedule: 4 of
+    width 1, 10 of width 64 with slope 0.5, 10 full), 16 heads x 128, int8 Q/K/V with per-row scales, batch 32,
+    a 2048-token prompt, then 256 generated tokens.  Per layer: prefill over the prompt, the prompt's K/V rows
+    moved into that layer's KV cache, and per generated token one append + one decode launch pair.  The
+    projections, FFN and sampling of the model are not part of this path; the new tokens' Q/K/V are synthetic."""
+
+    def __init__(self, ctx, B=32, prompt=2048, n_new=256, H=16, d=128, depth=24, seed=1313 + 5):
+        import torch
+        from tscale_amd import KVCache, capi
+        from tscale_amd.attention import alibi_layer_schedule
+        self.ctx, self.B, self.prompt, self.n_new, self.H, self.d = ctx, B, prompt, n_new, H, d
+        self.L = prompt + n_new
+        self.i8 = capi.I8
+        self.sched = alibi_layer_schedule(depth, self.L)
+        n = B * prompt
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        self.qkv = [ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g), H, capi.I8) for _ in range(3)]
+        self.off = torch.arange(0, n + 1, prompt, dtype=torch.int32, device="cuda")
+        self.spans = {W: ctx.build_spans(self.off, n, W) for W in {w for w, _ in self.sched}}
+        self.out = torch.empty((n, H * d), dtype=torch.float16, device="cuda")
+        self.caches = [KVCache(ctx, capi.I8, B, H, self.L, d) for _ in range(depth)]
+        new = [ctx.quantize_rows(torch.randn((B, H * d), device="cuda", generator=g), H, capi.I8) for _ in range(3)]
+        self.new = [(x, s.t().contiguous()) for x, s in new]     # scales as [B, H]
+        self.dout = torch.empty((B, H * d), dtype=torch.float32, device="cuda")
+        self.kinds = sorted({w for w, _ in self.sched})
+        torch.cuda.synchronize()
+
+    def prefill_layer(self, i):
+        (q, qs), (k, ks), (v, vs) = self.qkv
+        W, slope = self.sched[i]
+        st, fi = self.spans[W]
+        self.ctx.compute_val_lookup(self.i8, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out)
+
+    def fill_caches(self):
+        (_, _), (k, ks), (v, vs) = self.qkv
+        for c in self.caches:
+            c.cache_len.zero_()
+            c.fill_from_prefill(self.off, k, ks, v, vs)
+
+    def decode_step(self):
+        (q, qs), (k, ks), (v, vs) = self.new
+        for c, (W, slope) in zip(self.caches, self.sched):
+            c.add_vectors(k, ks, v, vs)
+            self.ctx.compute_val_lookup_decode(c, q, qs, W, slope, out=self.dout)
+
+    def prefill_flops(self, i):
+        return prefill_flops(self.B, self.prompt, self.H, self.d, self.sched[i][0])
+
+    def decode_bytes(self):
+        """Cache rows each generated token reads (K + V rows and their two scales), its q and its output."""
+        total = 0
+        for t in range(self.n_new):
+            n = self.prompt + t + 1
+            for W, _ in self.sched:
+                rows = min(n - 1, W)
+                total += self.B * self.H * (rows * (2 * self.d + 8) + self.d + 4 + 4 * self.d)
+        return total
+
+
+def bench_generation(ctx, steps):
+    import torch
+    gw = GenerationWorkload(ctx)
+    res = {"config": "24 layers (4 x W=1, 10 x W=64 slope 0.5, 10 x full), B32, prompt 2048 + 256 generated tokens, "
+                     "H16 d128 int8 Q/K/V + per-row f32 scales; attention launches only"}
+    first = {W: [i for i, (w, _) in enumerate(gw.sched) if w == W][0] for W in gw.kinds}
+    pre_ms = {W: gpu_time_ms(lambda i=i: gw.prefill_layer(i), max(3, steps // 10), 1) for W, i in first.items()}
+    total_ms = sum(pre_ms[w] for w, _ in gw.sched)
+    total_flops = sum(gw.prefill_flops(i) for i in range(len(gw.sched)))
+    wide = max(gw.kinds)
+    res["prefill"] = {"layer_ms": {f"W={w}": round(t, 5) for w, t in pre_ms.items()},
+                      "pass_ms": round(total_ms, 4), "TOP/s": round(total_flops / total_ms / 1e9, 2),
+                      "full_layer_TOP/s": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9, 2),
+                      "full_layer_frac_of_int8_peak": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9 / PEAK_I8_TOPS, 5)}
+    fill_ms = gpu_time_ms(gw.fill_caches, 2, 1)
+    n = gw.B * gw.prompt
+    fill_bytes = len(gw.caches) * 2 * (n * gw.H * gw.d * 2 + n * gw.H * 4 * 2)   # read + write of K, V and both scales
+    res["cache_fill"] = {"ms_24_layers": round(fill_ms, 4), "GB/s": round(fill_bytes / fill_ms / 1e6, 1)}
+    # generation: one captured step (24 x (append + decode pair)) replayed once per generated token
+    gw.fill_caches()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        gw.decode_step()                       # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    gw.fill_caches()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gw.decode_step()
+    gw.fill_caches()                           # capture does not run the step
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(gw.n_new):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    gen_ms = e0.elapsed_time(e1)
+    lens = {int(c.cache_len[0]) for c in gw.caches}
+    assert lens == {gw.L}, lens
+    nbytes = gw.decode_bytes()
+    res["generate"] = {"ms_256_tokens": round(gen_ms, 3), "ms_per_token": round(gen_ms / gw.n_new, 4),
+                       "us_per_layer_step": round(gen_ms / gw.n_new / len(gw.sched) * 1e3, 2),
+                       "GB/s": round(nbytes / gen_ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / gen_ms / 1e6 / PEAK_HBM_GBPS, 4),
+                       "bytes": nbytes, "launch": "HIP graph of one step, replayed per token"}
+    return res
+
+
 def cpu_baseline_prefill(wl, n_seq_sample):
     """The oracle (a port of the reference's CPU attention) on the same quantised inputs: the first
     `n_seq_sample` sequences of every layer of the pass, all host threads; plus one sequence of one
@@ -227,7 +337,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-decode", action="store_true")
-    ap.add_argument("--extra", action="store_true", help="also time the 1.5B-style prefill shapes")
+    ap.add_argument("--extra", action="store_true",
+                    help="also time the 1.5B-style prefill shapes and the attention share of the 1.5B-style generation run")
     ap.add_argument("--only", default=None,
                     choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode"],
                     help="profiling aid: run just this launch --steps times and print its timing")
@@ -308,6 +419,8 @@ def main():
             "layer_tflops": {"window256": round(wl.flops_layer[0] / ms_s / 1e9, 2), "full": round(wl.flops_layer[1] / ms_w / 1e9, 2)},
             "frac_of_fp8_peak_full": round(wl.flops_layer[1] / ms_w / 1e9 / PEAK_FP8_TFLOPS, 5)}
         del wl
+        torch.cuda.empty_cache()
+        result["generation_1p5B_style"] = bench_generation(ctx, args.steps)
     print(json.dumps(result))
 
 

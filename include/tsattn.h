@@ -153,6 +153,30 @@ typedef struct tsattn_append_args {
 
 int tsattn_cache_append(tsattn_handle_t h, const tsattn_append_args *a, void *stream);
 
+/* Append a whole prefill batch to the cache: sequence s owns tokens [seq_offset[s], seq_offset[s+1])
+ * of the [n_tokens][n_heads*head_dim] K and V arrays (the layout tsattn_prefill reads); they are
+ * written to cache rows cache_len[s], cache_len[s]+1, ... and cache_len[s] grows by their count.
+ * Same result as TAttentionVecHistory::AddVectors once per token, which is how the reference feeds a
+ * prompt to its cache (gpt/train/cpu_infer.cpp:403-408, token loop :586-600).  Rows that would land
+ * at or beyond max_len are dropped. */
+typedef struct tsattn_fill_args {
+    int n_seqs, n_heads, head_dim;
+    int64_t n_tokens;
+    const int32_t *seq_offset; /* device [n_seqs+1], ascending, seq_offset[n_seqs] <= n_tokens */
+    const void *k, *v;         /* [n_tokens][n_heads*head_dim] 8-bit */
+    int64_t pitch;             /* bytes per token row */
+    const float *k_scale, *v_scale; /* [n_heads][scale_pitch] planes; NULL = leave the cache's scale planes untouched */
+    int64_t scale_pitch;       /* floats */
+    void *k_cache, *v_cache;
+    int64_t seq_stride, head_stride, tok_stride;
+    float *k_scale_cache, *v_scale_cache;
+    int64_t s_seq_stride, s_head_stride;
+    int32_t *cache_len;        /* device [n_seqs], updated in place */
+    int max_len;
+} tsattn_fill_args;
+
+int tsattn_cache_fill(tsattn_handle_t h, const tsattn_fill_args *a, void *stream);
+
 /* Per-(row, head) absmax quantiser: scale = absmax/127 (int8) or absmax/256 (e4m3), values
  * round-to-nearest-even, int8 clamped to [-127,127].  Replaces NormalizeVecsRowTileMax /
  * TStoreRowTileMaxNormalize (gpt/compute/row_tile_scale.cuh:59-81, lib/cuda/cuda_matmul.cuh:207-260,

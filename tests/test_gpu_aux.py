@@ -87,3 +87,44 @@ def test_error_paths(ctx):
     with pytest.raises(TsattnError) as e:
         ctx.compute_val_lookup(7, 1, q[:, :64], q[:, :64], q[:, :64], 1.0, 1.0, 1.0, sp, sp, 0.0)
     assert e.value.code in (1, 2)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_cache_fill_equals_token_by_token_append(ctx, d):
+    """The bulk append of a prefill batch writes what AddVectors would write one token at a time
+    (cpu_infer.cpp:403-408): ragged sequences, an empty one, caches that already hold rows, one that overflows."""
+    from tscale_amd import KVCache
+    B, H, L = 5, 3, 40
+    lens = [17, 0, 33, 1, 25]
+    start = [0, 3, 5, 39, 30]     # the last sequence would reach 55 rows: rows beyond 40 are dropped
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    n = int(off[-1])
+    g = torch.Generator().manual_seed(d)
+    k = torch.randint(0, 256, (n, H * d), dtype=torch.uint8, generator=g).cuda()
+    v = torch.randint(0, 256, (n, H * d), dtype=torch.uint8, generator=g).cuda()
+    ks = torch.rand((H, n), generator=g).cuda()
+    vs = torch.rand((H, n), generator=g).cuda()
+
+    bulk = KVCache(ctx, capi.I8, B, H, L, d)
+    bulk.cache_len.copy_(torch.tensor(start, dtype=torch.int32))
+    bulk.fill_from_prefill(torch.from_numpy(off).cuda(), k, ks, v, vs)
+
+    single = KVCache(ctx, capi.I8, B, H, L, d)
+    single.cache_len.copy_(torch.tensor(start, dtype=torch.int32))
+    # token-by-token: sequences that have run out of tokens are parked on a full cache_len (= no-op)
+    for t in range(max(lens)):
+        rows = [int(off[b]) + min(t, max(lens[b] - 1, 0)) for b in range(B)]
+        kk = k[rows].contiguous(); vv = v[rows].contiguous()
+        kss = ks[:, rows].t().contiguous(); vss = vs[:, rows].t().contiguous()
+        active = torch.tensor([t < lens[b] for b in range(B)]).cuda()
+        saved = single.cache_len.clone()
+        single.cache_len.copy_(torch.where(active, saved, torch.full_like(saved, L)))
+        single.add_vectors(kk, kss, vv, vss)
+        single.cache_len.copy_(torch.where(active, single.cache_len, saved))
+    torch.cuda.synchronize()
+    want_len = [min(L, s + n_) for s, n_ in zip(start, lens)]
+    assert bulk.cache_len.tolist() == want_len == single.cache_len.tolist()
+    for a, b in ((bulk.k, single.k), (bulk.v, single.v), (bulk.k_scale, single.k_scale), (bulk.v_scale, single.v_scale)):
+        assert torch.equal(a, b)
+    assert torch.equal(bulk.k[0, 1, 16], k[16, d:2 * d]) and torch.equal(bulk.v[2, 2, 5], v[17, 2 * d:3 * d])
+    assert not bulk.k[1].any()

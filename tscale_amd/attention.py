@@ -30,6 +30,22 @@ def _scale_arg(s):
     return None, float(s)
 
 
+def alibi_layer_schedule(depth, wide_window):
+    """Per-layer (attention width, ALiBi slope) of a TScale model of `depth` layers: the ALIBI_V3 rule of
+    InitAlibi (gpt/model_params/model_dim.cpp:55-97): max(1, groups/6) leading pairs of width-1 layers,
+    then pairs of (64, slope 0.5) and (wide, slope 0); a one-layer model is (wide, 0.1)."""
+    if depth == 1:
+        return [(wide_window, 0.1)]
+    groups = (depth + 1) // 2
+    w1 = max(1, groups // 6)
+    out = []
+    for _ in range(w1):
+        out += [(1, 0.0), (1, 0.0)]
+    for _ in range(w1, groups):
+        out += [(64, 0.5), (wide_window, 0.0)]
+    return out
+
+
 class AttentionContext:
     """One per device, like the reference's per-device compute context (gpt_cuda.cu:1478-1573)."""
 
@@ -168,3 +184,24 @@ class KVCache:
             a.s_seq_stride, a.s_head_stride = self.k_scale.stride(0), self.k_scale.stride(1)
         a.cache_len, a.max_len = _ptr(self.cache_len), self.max_len
         capi.check(self.ctx.lib.tsattn_cache_append(self.ctx.handle, ctypes.byref(a), _stream_ptr()))
+
+    def fill_from_prefill(self, seq_offset, k, k_scale, v, v_scale=None):
+        """Append a prefill batch: k, v uint8 [n_tokens, n_heads*d]; scales f32 [n_heads, n_tokens] planes (None
+        with constant scales); seq_offset int32 [n_seqs+1] on the device.  Equals add_vectors once per token."""
+        a = capi.FillArgs()
+        a.n_seqs, a.n_heads, a.head_dim = self.n_seqs, self.n_heads, self.head_dim
+        a.n_tokens = k.shape[0]
+        a.seq_offset = _ptr(seq_offset)
+        a.k, a.v, a.pitch = _ptr(k), _ptr(v), k.stride(0)
+        assert v.stride(0) == k.stride(0)
+        a.k_scale, a.v_scale = _ptr(k_scale), _ptr(v_scale)
+        pitches = [s.stride(0) for s in (k_scale, v_scale) if s is not None]
+        assert len(set(pitches)) <= 1
+        a.scale_pitch = pitches[0] if pitches else a.n_tokens
+        a.k_cache, a.v_cache = _ptr(self.k), _ptr(self.v)
+        a.seq_stride, a.head_stride, a.tok_stride = self.k.stride(0), self.k.stride(1), self.k.stride(2)
+        if isinstance(self.k_scale, torch.Tensor):
+            a.k_scale_cache, a.v_scale_cache = _ptr(self.k_scale), _ptr(self.v_scale)
+            a.s_seq_stride, a.s_head_stride = self.k_scale.stride(0), self.k_scale.stride(1)
+        a.cache_len, a.max_len = _ptr(self.cache_len), self.max_len
+        capi.check(self.ctx.lib.tsattn_cache_fill(self.ctx.handle, ctypes.byref(a), _stream_ptr()))

@@ -68,8 +68,20 @@ class AppendArgs(_c.Structure):
     ]
 
 
+class FillArgs(_c.Structure):
+    _fields_ = [
+        ("n_seqs", _c.c_int), ("n_heads", _c.c_int), ("head_dim", _c.c_int), ("n_tokens", _c.c_int64),
+        ("seq_offset", _c.c_void_p), ("k", _c.c_void_p), ("v", _c.c_void_p), ("pitch", _c.c_int64),
+        ("k_scale", _c.c_void_p), ("v_scale", _c.c_void_p), ("scale_pitch", _c.c_int64),
+        ("k_cache", _c.c_void_p), ("v_cache", _c.c_void_p), ("seq_stride", _c.c_int64),
+        ("head_stride", _c.c_int64), ("tok_stride", _c.c_int64), ("k_scale_cache", _c.c_void_p),
+        ("v_scale_cache", _c.c_void_p), ("s_seq_stride", _c.c_int64), ("s_head_stride", _c.c_int64),
+        ("cache_len", _c.c_void_p), ("max_len", _c.c_int),
+    ]
+
+
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_cache_append", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
+           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
 
 _lib = None
 
@@ -97,6 +109,8 @@ def load():
         L.tsattn_decode.argtypes = [_c.c_void_p, _c.POINTER(DecodeArgs), _c.c_void_p]
         L.tsattn_cache_append.restype = _c.c_int
         L.tsattn_cache_append.argtypes = [_c.c_void_p, _c.POINTER(AppendArgs), _c.c_void_p]
+        L.tsattn_cache_fill.restype = _c.c_int
+        L.tsattn_cache_fill.argtypes = [_c.c_void_p, _c.POINTER(FillArgs), _c.c_void_p]
         L.tsattn_quantize_rows.restype = _c.c_int
         L.tsattn_quantize_rows.argtypes = [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64,
                                            _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64,

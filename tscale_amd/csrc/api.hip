@@ -162,7 +162,9 @@ int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
         // enough workgroups to fill 256 CUs several times over, but at least 512 cache rows per split
         const int64_t pairs = (int64_t)a->n_seqs * a->n_heads;
         int64_t want = (4096 + pairs - 1) / pairs;
-        int64_t by_len = ((int64_t)a->max_len + 511) / 512;
+        int64_t rows = a->max_len;   // rows one query can see
+        if (a->window < rows) rows = a->window > 0 ? a->window : 1;
+        int64_t by_len = (rows + 511) / 512;
         if (want > by_len) want = by_len;
         if (want < 1) want = 1;
         if (want > h->max_splits) want = h->max_splits;
@@ -204,6 +206,34 @@ int tsattn_cache_append(tsattn_handle_t h, const tsattn_append_args *a, void *st
     p.cache_len = a->cache_len; p.max_len = a->max_len; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
     hipError_t e = tsattn::launch_cache_append(p, a->n_seqs, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "cache append launch");
+    return TSATTN_OK;
+}
+
+int tsattn_cache_fill(tsattn_handle_t h, const tsattn_fill_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: null argument");
+    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_cache_fill: head_dim %d (64 or 128 supported)", a->head_dim);
+    if (a->n_seqs < 0 || a->n_heads <= 0 || a->max_len < 0 || a->n_tokens < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: negative size");
+    if (a->n_heads > 65535) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: too many heads");
+    if (a->n_seqs == 0 || a->n_tokens == 0) return TSATTN_OK;
+    if (!a->seq_offset || !a->k || !a->v || !a->k_cache || !a->v_cache || !a->cache_len) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: null data pointer");
+    if ((a->k_scale && !a->k_scale_cache) || (a->v_scale && !a->v_scale_cache)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: scales given without scale planes");
+    if (a->pitch % 16 || a->tok_stride % 16 || a->head_stride % 16 || a->seq_stride % 16 || a->tok_stride < a->head_dim ||
+        a->pitch < (int64_t)a->n_heads * a->head_dim)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: pitches and strides must be multiples of 16 bytes and cover a row");
+    if (!aligned16(a->k) || !aligned16(a->v) || !aligned16(a->k_cache) || !aligned16(a->v_cache))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: pointers must be 16-byte aligned");
+    if ((a->k_scale || a->v_scale) && a->scale_pitch < a->n_tokens) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: scale_pitch below n_tokens");
+    tsattn::FillParams p;
+    p.seq_offset = a->seq_offset; p.k_src = (const uint8_t *)a->k; p.v_src = (const uint8_t *)a->v; p.pitch = a->pitch;
+    p.ks_src = a->k_scale; p.vs_src = a->v_scale; p.scale_pitch = a->scale_pitch;
+    p.k = (uint8_t *)a->k_cache; p.v = (uint8_t *)a->v_cache;
+    p.seq_stride = a->seq_stride; p.head_stride = a->head_stride; p.tok_stride = a->tok_stride;
+    p.ks = a->k_scale_cache; p.vs = a->v_scale_cache; p.s_seq_stride = a->s_seq_stride; p.s_head_stride = a->s_head_stride;
+    p.cache_len = a->cache_len; p.max_len = a->max_len; p.n_seqs = a->n_seqs; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
+    p.n_tokens = a->n_tokens;
+    hipError_t e = tsattn::launch_cache_fill(p, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "cache fill launch");
     return TSATTN_OK;
 }
 

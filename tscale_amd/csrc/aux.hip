@@ -144,4 +144,60 @@ hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st
     return hipGetLastError();
 }
 
+// Bulk form of the append: the K/V rows of a prefill batch ([token][head*d]) go to the planar cache.
+// A workgroup handles 64 consecutive tokens of one head: reads are 16 bytes per lane with the lanes of a
+// row adjacent, writes cover whole cache rows back to back.
+__global__ __launch_bounds__(256) void cache_fill_kernel(FillParams p)
+{
+    const int chunks = p.head_dim / 16;
+    const int rows_per_block = 256 / chunks;
+    const int head = blockIdx.y;
+    const int c = threadIdx.x % chunks;
+    const int64_t tok = (int64_t)blockIdx.x * rows_per_block + threadIdx.x / chunks;
+    if (tok >= p.n_tokens) return;
+    // sequence of this token: last s with seq_offset[s] <= tok
+    int lo = 0, hi = p.n_seqs;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (p.seq_offset[mid] <= tok) lo = mid; else hi = mid;
+    }
+    const int seq = lo;
+    const int64_t first = p.seq_offset[seq];
+    if (tok < first || tok >= p.seq_offset[seq + 1]) return;
+    const int64_t pos = (int64_t)p.cache_len[seq] + (tok - first);
+    if (pos < 0 || pos >= p.max_len) return;
+    const int64_t src = tok * p.pitch + head * p.head_dim + c * 16;
+    const int64_t dst = (int64_t)seq * p.seq_stride + (int64_t)head * p.head_stride + pos * p.tok_stride + c * 16;
+    *(v4i *)(p.k + dst) = *(const v4i *)(p.k_src + src);
+    *(v4i *)(p.v + dst) = *(const v4i *)(p.v_src + src);
+    if (c == 0) {
+        const int64_t sd = (int64_t)seq * p.s_seq_stride + (int64_t)head * p.s_head_stride + pos;
+        if (p.ks_src) p.ks[sd] = p.ks_src[(int64_t)head * p.scale_pitch + tok];
+        if (p.vs_src) p.vs[sd] = p.vs_src[(int64_t)head * p.scale_pitch + tok];
+    }
+}
+
+__global__ void cache_len_add_kernel(int32_t *cache_len, const int32_t *seq_offset, int n_seqs, int max_len)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_seqs) return;
+    const int len = cache_len[i];
+    if (len < 0) return;
+    const int64_t grown = (int64_t)len + (seq_offset[i + 1] - seq_offset[i]);
+    cache_len[i] = (int32_t)(grown < max_len ? grown : max_len);
+}
+
+hipError_t launch_cache_fill(const FillParams &p, hipStream_t st)
+{
+    if (p.n_seqs == 0 || p.n_tokens == 0) return hipSuccess;
+    const int rows_per_block = 256 / (p.head_dim / 16);
+    hipLaunchKernelGGL(cache_fill_kernel, dim3((unsigned)((p.n_tokens + rows_per_block - 1) / rows_per_block), (unsigned)p.n_heads),
+                       dim3(256), 0, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(cache_len_add_kernel, dim3((unsigned)((p.n_seqs + 255) / 256)), dim3(256), 0, st, p.cache_len, p.seq_offset,
+                       p.n_seqs, p.max_len);
+    return hipGetLastError();
+}
+
 } // namespace tsattn

@@ -72,4 +72,24 @@ struct AppendParams {
 
 hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st);
 
+struct FillParams {
+    const int32_t *seq_offset;
+    const uint8_t *k_src, *v_src;
+    int64_t pitch;
+    const float *ks_src, *vs_src;
+    int64_t scale_pitch;
+    uint8_t *k, *v;
+    int64_t seq_stride, head_stride, tok_stride;
+    float *ks, *vs;
+    int64_t s_seq_stride, s_head_stride;
+    int32_t *cache_len;
+    int max_len;
+    int n_seqs;
+    int n_heads;
+    int head_dim;
+    int64_t n_tokens;
+};
+
+hipError_t launch_cache_fill(const FillParams &p, hipStream_t st);
+
 } // namespace tsattn
