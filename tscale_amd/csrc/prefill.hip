@@ -219,46 +219,70 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     float l = 0.0f, l2 = 0.0f; // this lane's share of the weight sum (its 32 of every 64 keys), in two chains
 
     if (b_max_b >= b_min_a) {
-        const int kb_first = (b_min_a / PF_BN) * PF_BN;
-        const int n_tiles = (b_max_b - kb_first) / PF_BN + 1;
+        // the same in every lane; said explicitly so that everything derived from them stays in scalar registers
+        const int kb_first = __builtin_amdgcn_readfirstlane((b_min_a / PF_BN) * PF_BN);
+        const int n_tiles = __builtin_amdgcn_readfirstlane((b_max_b - kb_first) / PF_BN + 1);
 
         // ---- staging: global -> registers -> LDS (K as is; V widened to f16 * row scale) -----------------
+        // Loads go through buffer descriptors whose base (a scalar) advances by one tile per load, so the
+        // per-lane offsets are loop constants and no vector address arithmetic is left in the loop.  A
+        // descriptor ends at the last token's row: rows past it read as zeros (their logits are masked).
         v4i rk[NLD], rv[NLD];
         float rvs[NLD], rks = 0.0f;
-        // Row offsets advance by one tile per load; rows past the last token re-read the last row
-        // (their logits are masked), so no multiply is needed inside the loop.
-        const int64_t k_last = (int64_t)(p.n_tokens - 1) * p.k_pitch, v_last = (int64_t)(p.n_tokens - 1) * p.v_pitch;
-        int64_t k_off[NLD], v_off[NLD];
-        int s_idx[NLD];
-        const uint8_t *k_base[NLD], *v_base[NLD];
+        int k_voff[NLD], v_voff[NLD];
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const int ch = tid + i * PF_THREADS;
             const int r = ch / CHUNKS, c = ch % CHUNKS;
-            k_off[i] = (int64_t)(kb_first + r) * p.k_pitch;
-            v_off[i] = (int64_t)(kb_first + r) * p.v_pitch;
-            s_idx[i] = kb_first + r;
-            k_base[i] = p.k + hoff + c * 16;
-            v_base[i] = p.v + hoff + c * 16;
+            k_voff[i] = r * (int)p.k_pitch + c * 16;
+            v_voff[i] = r * (int)p.v_pitch + c * 16;
         }
-        int ks_idx = kb_first + tid;
-        const float *vs_row = p.vs ? p.vs + (int64_t)head * p.scale_pitch : nullptr;
-        const float *ks_row = p.ks ? p.ks + (int64_t)head * p.scale_pitch : nullptr;
         const int64_t k_step = (int64_t)PF_BN * p.k_pitch, v_step = (int64_t)PF_BN * p.v_pitch;
+        const uint8_t *k_ptr = p.k + hoff + (int64_t)kb_first * p.k_pitch;
+        const uint8_t *v_ptr = p.v + hoff + (int64_t)kb_first * p.v_pitch;
+        // bytes from the tile's first row to the end of this head's part of the last row
+        int64_t k_left = (int64_t)(p.n_tokens - 1 - kb_first) * p.k_pitch + D;
+        int64_t v_left = (int64_t)(p.n_tokens - 1 - kb_first) * p.v_pitch + D;
+        const float *vs_ptr = p.vs ? p.vs + (int64_t)head * p.scale_pitch + kb_first : nullptr;
+        const float *ks_ptr = p.ks ? p.ks + (int64_t)head * p.scale_pitch + kb_first : nullptr;
+        const int64_t s_left = (int64_t)(p.n_tokens - kb_first) * 4;
+        auto rsrc = [](const void *base, int64_t bytes) {
+            const uint32_t n = bytes <= 0 ? 0u : (bytes > 0xffffffffll ? 0xffffffffu : (uint32_t)bytes);
+            return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+        };
+        __amdgpu_buffer_rsrc_t kr = rsrc(k_ptr, k_left), vr = rsrc(v_ptr, v_left);
+        const __amdgpu_buffer_rsrc_t ksr = rsrc(ks_ptr, s_left), vsr = rsrc(vs_ptr, s_left);
+        // scalar byte offsets of the next tile to load, relative to the descriptors' bases
+        uint32_t k_soff = 0, v_soff = 0, s_soff = 0;
         auto load_tile = [&]() { // loads the next tile in sequence
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
                 if (!LD_ALL && tid + i * PF_THREADS >= PF_BN * CHUNKS) break;
-                rk[i] = *(const v4i *)(k_base[i] + (k_off[i] < k_last ? k_off[i] : k_last));
-                rv[i] = *(const v4i *)(v_base[i] + (v_off[i] < v_last ? v_off[i] : v_last));
-                rvs[i] = vs_row ? vs_row[min(s_idx[i], p.n_tokens - 1)] : p.vs_const;
-                k_off[i] += k_step;
-                v_off[i] += v_step;
-                s_idx[i] += PF_BN;
+                rk[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(kr, k_voff[i], (int)k_soff, 0));
+                rv[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(vr, v_voff[i], (int)v_soff, 0));
             }
-            if (tid < PF_BN) {
-                rks = ks_row ? ks_row[min(ks_idx, p.n_tokens - 1)] : p.ks_const;
-                ks_idx += PF_BN;
+            if (vs_ptr) {
+#pragma unroll
+                for (int i = 0; i < NLD; ++i) {
+                    const int r = (tid + i * PF_THREADS) / CHUNKS;
+                    rvs[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(vsr, r * 4, (int)s_soff, 0));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NLD; ++i) rvs[i] = p.vs_const;
+            }
+            // lanes beyond the tile's 64 keys read past it harmlessly (zeros past the end)
+            if (ks_ptr) rks = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ksr, (tid & (PF_BN - 1)) * 4, (int)s_soff, 0));
+            else rks = p.ks_const;
+            k_soff += (uint32_t)k_step;
+            v_soff += (uint32_t)v_step;
+            s_soff += PF_BN * 4;
+            // far into a very long key range the 32-bit offsets are folded back into the bases
+            if ((k_soff | v_soff) >= 0x40000000u) {
+                k_ptr += k_soff; k_left -= k_soff; k_soff = 0;
+                v_ptr += v_soff; v_left -= v_soff; v_soff = 0;
+                kr = rsrc(k_ptr, k_left);
+                vr = rsrc(v_ptr, v_left);
             }
         };
         auto store_tile = [&](int buf) {
