@@ -398,23 +398,157 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             }
         };
 
+        // ---- the common tile: every key inside every span of the wave, no ALiBi ------------------------
+        // Written so that matrix and vector instructions alternate in the instruction stream (a wave issues
+        // in order: vector work placed between two MFMAs runs while the first one executes):
+        //   block 1: K.Q^T of both 32-key sub-tiles; the weights of sub-tile 0 overlap the MFMAs of sub-tile 1
+        //   block 2: V^T.P^T of sub-tile 0 overlaps the weights of sub-tile 1
+        //   block 3: V^T.P^T of sub-tile 1 overlaps the staging (widening, LDS stores) of the next tile
+        // Weights are computed against the reference maximum without looking at the logits' maximum; if a
+        // sub-tile's weight sum shows that a logit was more than the threshold above it, the sub-tile is redone
+        // on the slow path with a raised reference.
+        constexpr float PF_SUM_LIMIT = 256.0f; // = 2^PF_RESCALE_THRESHOLD: one weight above it is enough to exceed it
+        auto weights_sub = [&](const typename Qk::acc_t &acc, const float *ksp, float nbase, v8h &pa, v8h &pb, float &s0, float &s1) {
+            v2h pp[8];
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+                const v4f ksv = *(const v4f *)(ksp + 8 * c4);
+#pragma unroll
+                for (int j2 = 0; j2 < 2; ++j2) {
+                    const int r = c4 * 4 + 2 * j2;
+                    const float x0 = Qk::to_float(acc, r) * ksv[2 * j2];
+                    const float x1 = Qk::to_float(acc, r + 1) * ksv[2 * j2 + 1];
+                    const float p0 = fast_exp2(fmaf(x0, qs, nbase));
+                    const float p1 = fast_exp2(fmaf(x1, qs, nbase));
+                    s0 += p0;
+                    s1 += p1;
+                    pp[r / 2] = v2h{(_Float16)p0, (_Float16)p1};
+                }
+            }
+            pa = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
+            pb = v8h{pp[4][0], pp[4][1], pp[5][0], pp[5][1], pp[6][0], pp[6][1], pp[7][0], pp[7][1]};
+        };
+        // slow path of one sub-tile: exact maximum, raise the reference, rescale the accumulators, redo the weights
+        auto weights_sub_rescale = [&](const typename Qk::acc_t &acc, const float *ksp, v8h &pa, v8h &pb, float &s0, float &s1) {
+            float xs[16];
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                xs[r] = fmaf(Qk::to_float(acc, r) * ksp[8 * (r / 4) + (r & 3)], qs, -m_ref);
+                tmax = fmaxf(tmax, xs[r]);
+            }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+            const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
+            const float alpha = fast_exp2(-shift);
+            have_ref = true;
+            m_ref += shift;
+            l *= alpha;
+            l2 *= alpha;
+#pragma unroll
+            for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
+            s0 = 0.0f;
+            s1 = 0.0f;
+            v2h pp[8];
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = fast_exp2(xs[r] - shift), p1 = fast_exp2(xs[r + 1] - shift);
+                s0 += p0;
+                s1 += p1;
+                pp[r / 2] = v2h{(_Float16)p0, (_Float16)p1};
+            }
+            pa = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
+            pb = v8h{pp[4][0], pp[4][1], pp[5][0], pp[5][1], pp[6][0], pp[6][1], pp[7][0], pp[7][1]};
+        };
+        auto fast_tile = [&](auto stage_tag, int buf) {
+            constexpr bool STAGE = decltype(stage_tag)::value;
+            static_assert(PF_KT == 2, "the common-tile path is written for 64-key tiles");
+            // ---- block 1 ----
+            const typename Qk::acc_t acc0 = qk.mma(k_lds[buf] + qi * L::K_PITCH, g);
+            const typename Qk::acc_t acc1 = qk.mma(k_lds[buf] + (32 + qi) * L::K_PITCH, g);
+            vload(0, 0, buf);
+            vload(1, 1, buf);
+            v8h p0a, p0b, p1a, p1b;
+            float s0 = 0.0f, s1 = 0.0f;
+            weights_sub(acc0, ks_lds[buf] + 4 * g, -m_ref, p0a, p0b, s0, s1);
+            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc0, ks_lds[buf] + 4 * g, p0a, p0b, s0, s1);
+            l += s0;
+            l2 += s1;
+            // ---- block 2 ----
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[0][dt], p0a, o_acc[dt], 0, 0, 0);
+            vload(0, 2, buf);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[1][dt], p0b, o_acc[dt], 0, 0, 0);
+            vload(1, 3, buf);
+            s0 = 0.0f;
+            s1 = 0.0f;
+            weights_sub(acc1, ks_lds[buf] + 32 + 4 * g, -m_ref, p1a, p1b, s0, s1);
+#pragma unroll
+            for (int i = 0; i < 2 * DT; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+                __builtin_amdgcn_sched_group_barrier(0x002, 10, 0); // vector work of the other sub-tile behind it
+            }
+            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc1, ks_lds[buf] + 32 + 4 * g, p1a, p1b, s0, s1);
+            l += s0;
+            l2 += s1;
+            // ---- block 3 ----
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[0][dt], p1a, o_acc[dt], 0, 0, 0);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[1][dt], p1b, o_acc[dt], 0, 0, 0);
+            if (STAGE) {
+                store_tile(buf ^ 1);
+#pragma unroll
+                for (int i = 0; i < 2 * DT; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                }
+            }
+        };
+
         load_tile();
         store_tile(0);
         if (n_tiles > 1) load_tile();
         __syncthreads();
-        for (int it = 0; it < n_tiles; ++it) {
-            const int buf = it & 1;
-            const int kb = kb_first + it * PF_BN;
-            // does this wave need the tile at all, and does it need the per-element mask?
-            if (!(kb + PF_BN - 1 < w_min_a || kb > w_max_b)) {
-                const bool interior = w_all_have_keys && (kb >= w_max_a) && (kb + PF_BN - 1 <= w_min_b);
-                if (interior && !have_ref) compute_tile(std::true_type{}, std::false_type{}, buf, kb);
-                else if (interior) compute_tile(std::true_type{}, std::true_type{}, buf, kb);
-                else compute_tile(std::false_type{}, std::true_type{}, buf, kb);
+        // Tiles in key order are: not needed by this wave, partly inside its spans, fully inside, partly
+        // inside (the diagonal), not needed.  The fully-inside run [f0, f1) takes the common-tile path (never
+        // the last tile of the workgroup, which has no successor to stage); everything else the general one.
+        int f0 = n_tiles, f1 = n_tiles;
+        if (!SLOPE && !DUMP && w_all_have_keys) {
+            f0 = max(0, (w_max_a - kb_first + PF_BN - 1) / PF_BN);
+            f1 = min(n_tiles - 1, (w_min_b + 1 - kb_first) / PF_BN); // tiles [.., f1) end at or before the smallest span end
+            if (f1 < f0) f1 = f0;
+            f0 = min(f0, n_tiles);
+            f1 = max(f1, f0);
+        }
+        f0 = __builtin_amdgcn_readfirstlane(f0);
+        f1 = __builtin_amdgcn_readfirstlane(f1);
+        int it = 0;
+        for (int pass = 0; pass < 2; ++pass) {
+            const int end = pass == 0 ? f0 : n_tiles;
+            for (; it < end; ++it) {
+                const int buf = it & 1;
+                const int kb = kb_first + it * PF_BN;
+                // does this wave need the tile at all, and does it need the per-element mask?
+                if (!(kb + PF_BN - 1 < w_min_a || kb > w_max_b)) {
+                    const bool interior = w_all_have_keys && (kb >= w_max_a) && (kb + PF_BN - 1 <= w_min_b);
+                    if (interior) compute_tile(std::true_type{}, std::true_type{}, buf, kb);
+                    else compute_tile(std::false_type{}, std::true_type{}, buf, kb);
+                }
+                if (it + 1 < n_tiles) store_tile(buf ^ 1);
+                if (it + 2 < n_tiles) load_tile();
+                __syncthreads();
             }
-            if (it + 1 < n_tiles) store_tile(buf ^ 1);
-            if (it + 2 < n_tiles) load_tile();
-            __syncthreads();
+            if constexpr (!SLOPE && !DUMP) {
+                if (pass == 0) {
+                    for (; it < f1; ++it) {
+                        fast_tile(std::true_type{}, it & 1);
+                        if (it + 2 < n_tiles) load_tile();
+                        __syncthreads();
+                    }
+                }
+            }
         }
     }
 
