@@ -89,7 +89,9 @@ class PrefillWorkload:
         (q, qs), (k, ks), (v, vs) = self.inputs[i]
         W, slope = self.layers[i]
         st, fi = self.spans[W]
-        self.ctx.compute_val_lookup(self.dtype, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out)
+        # equal-length sequences: tell the library the causal period of the wide layers (a launch-order hint)
+        self.ctx.compute_val_lookup(self.dtype, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
+                                    causal_period=self.S if W >= self.S else 0)
 
     def step(self):
         for i in range(len(self.layers)):
@@ -159,7 +161,8 @@ class GenerationWorkload:
         (q, qs), (k, ks), (v, vs) = self.qkv
         W, slope = self.sched[i]
         st, fi = self.spans[W]
-        self.ctx.compute_val_lookup(self.i8, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out)
+        self.ctx.compute_val_lookup(self.i8, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
+                                    causal_period=self.prompt if W >= self.prompt else 0)
 
     def fill_caches(self):
         (_, _), (k, ks), (v, vs) = self.qkv

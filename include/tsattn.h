@@ -94,6 +94,11 @@ typedef struct tsattn_prefill_args {
     void *debug_qk_acc;          /* optional raw QK^T accumulators, [n_heads][n_tokens][debug_pitch]
                                     int32 (int8 inputs) or f32 (e4m3); only in-span pairs are written */
     int64_t debug_pitch;         /* elements per (head, from) row of debug_qk_acc */
+    int64_t causal_period;       /* scheduling hint, 0 = none: rows t and t + causal_period have spans of equal
+                                    length and spans grow with t inside a period (a batch of equal-length
+                                    sequences under a wide causal window, as the reference's fixed-length
+                                    fragments are).  Only the order in which work is launched depends on it,
+                                    never the result; a value the kernel cannot use is ignored. */
 } tsattn_prefill_args;
 
 int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream);

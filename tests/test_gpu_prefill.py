@@ -150,3 +150,41 @@ def test_prefill_full_size_properties(ctx):
     want = 1 - torch.exp2(-swl).t()
     assert (o - want[:, :, None]).abs().max().item() < 2e-3
     assert (o.max(dim=2).values - o.min(dim=2).values).max().item() < 1e-6
+
+
+@pytest.mark.parametrize("dtype,d", [(capi.E4M3, 64), (capi.I8, 128)])
+def test_prefill_launch_order_hint_never_changes_results(ctx, dtype, d):
+    """causal_period only permutes the order in which query tiles are launched: with a usable value, a value the
+    kernel cannot use (not a multiple of the tile, not dividing the batch) and a wrong one, the output is
+    bit-identical to the one without a hint."""
+    B, S, H = 8, 512, 4     # 32 query tiles x 4 heads = 128 workgroups: the reordering applies
+    n = B * S
+    q, qs, k, ks, v, vs = make_qkv(77, n, H, d, dtype)
+    st, fi = orc.make_spans([S] * B, S)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    args = (dtype, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), 0.0)
+    base = ctx.compute_val_lookup(*args).cpu().numpy()
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, 0.0)
+    assert_within_tolerance(base, want, "no hint")
+    for period in (S, 2 * S, 256, 100, 384, n, 10 ** 9):
+        got = ctx.compute_val_lookup(*args, causal_period=period).cpu().numpy()
+        assert np.array_equal(got, base), f"causal_period={period}"
+
+
+def test_prefill_logits_far_above_the_zero_vector(ctx):
+    """Large query scales push logits tens of log2 units above the zero vector's 0: the reference maximum has to
+    be raised several times, on interior tiles (the common-tile path's weight-sum check) and on the diagonal."""
+    H, d = 2, 128
+    seq_lens = [700, 330]
+    n = sum(seq_lens)
+    for dtype in (capi.E4M3, capi.I8):
+        q, qs, k, ks, v, vs = make_qkv(31, n, H, d, dtype)
+        for boost in (8.0, 40.0):
+            qb = (qs * np.float32(boost)).astype(np.float32)
+            st, fi = orc.make_spans(seq_lens, 10 ** 6)
+            want, want_swl = orc.prefill_q8(dtype, q, k, v, H, qb, ks, vs, st, fi, 0.0, want_swl=True)
+            out, swl = run_gpu(ctx, dtype, H, q, qb, k, ks, v, vs, st, fi, 0.0, want_swl=True)
+            assert np.isfinite(out).all()
+            assert want_swl.max() > 20.0 if boost > 10 else want_swl.max() > 4.0
+            assert_within_tolerance(out, want, f"boost {boost}")
+            assert np.abs(swl - want_swl).max() < 2e-3 * max(1.0, np.abs(want_swl).max() / 16)

@@ -95,8 +95,10 @@ class AttentionContext:
     # ---- prefill --------------------------------------------------------------------------------
     def compute_val_lookup(self, dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, span_start, span_finish,
                            alibi_slope, out=None, out_f16=False, sum_weight_log=None, k_global_scale=None,
-                           debug_qk_acc=None):
-        """q,k,v: uint8 [n_tokens, n_heads*d] (row pitch = stride(0)); scales f32 [n_heads, n_tokens] or numbers."""
+                           debug_qk_acc=None, causal_period=0):
+        """q,k,v: uint8 [n_tokens, n_heads*d] (row pitch = stride(0)); scales f32 [n_heads, n_tokens] or numbers.
+        causal_period: launch-order hint for batches of equal-length sequences under a wide causal window (the
+        common sequence length); never changes the result."""
         n_tokens, hd = q.shape
         d = hd // n_heads
         if out is None:
@@ -120,6 +122,7 @@ class AttentionContext:
         a.sum_weight_log = _ptr(sum_weight_log)
         if debug_qk_acc is not None:
             a.debug_qk_acc, a.debug_pitch = _ptr(debug_qk_acc), debug_qk_acc.stride(1)
+        a.causal_period = int(causal_period)
         capi.check(self.lib.tsattn_prefill(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
 

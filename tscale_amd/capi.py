@@ -39,7 +39,7 @@ class PrefillArgs(_c.Structure):
         ("v_scale_const", _c.c_float), ("k_global_scale", _c.c_void_p), ("span_start", _c.c_void_p),
         ("span_finish", _c.c_void_p), ("alibi_slope", _c.c_float), ("out", _c.c_void_p),
         ("out_pitch", _c.c_int64), ("sum_weight_log", _c.c_void_p), ("debug_qk_acc", _c.c_void_p),
-        ("debug_pitch", _c.c_int64),
+        ("debug_pitch", _c.c_int64), ("causal_period", _c.c_int64),
     ]
 
 

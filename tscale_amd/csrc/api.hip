@@ -133,6 +133,7 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     p.sum_weight_log = a->sum_weight_log;
     p.dbg = a->debug_qk_acc; p.dbg_pitch = a->debug_pitch;
     p.n_tokens = (int)a->n_tokens; p.n_heads = a->n_heads;
+    p.period_tiles = (a->causal_period > 0 && a->causal_period % 128 == 0 && a->n_tokens % a->causal_period == 0) ? (int)(a->causal_period / 128) : 0;
     hipError_t e = tsattn::launch_prefill(p, a->dtype, a->head_dim, a->out_dtype, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "prefill launch");
     return TSATTN_OK;

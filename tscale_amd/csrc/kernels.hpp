@@ -45,6 +45,7 @@ struct PrefillParams {
     int64_t dbg_pitch;
     int n_tokens;
     int n_heads;
+    int period_tiles; // query tiles per period of equal span structure, 0 = unknown (launch order only)
 };
 
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int head_dim, int out_dtype, hipStream_t st);

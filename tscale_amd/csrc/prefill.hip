@@ -23,7 +23,7 @@ namespace tsattn {
 
 constexpr int PF_THREADS = 256;
 constexpr int PF_WAVES = 4;
-constexpr int PF_BM = 128; // queries per workgroup
+constexpr int PF_BM = 128; // queries per workgroup (the C ABI's causal_period hint is counted in these)
 #ifndef TSATTN_PF_BN
 #define TSATTN_PF_BN 64
 #endif
@@ -74,6 +74,15 @@ struct QkMma<TSATTN_E4M3, D> {
         }
         return acc;
     }
+    // the same in single steps, for code that places each LDS read and MFMA itself
+    typedef v8i kop_t;
+    __device__ static kop_t load_k(const uint8_t *krow, int g, int s)
+    {
+        const v4i *p = (const v4i *)(krow + 64 * s + 32 * g);
+        v4i a = p[0], b = p[1];
+        return v8i{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    }
+    __device__ acc_t step(kop_t kk, int s, acc_t acc) const { return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kk, q[s], acc, 0, 0, 0, 0, 0, 0); }
     __device__ static float to_float(const acc_t &a, int r) { return a[r]; }
     __device__ static float bits(const acc_t &a, int r) { return a[r]; }
 };
@@ -101,6 +110,9 @@ struct QkMma<TSATTN_I8, D> {
         }
         return acc;
     }
+    typedef v4i kop_t;
+    __device__ static kop_t load_k(const uint8_t *krow, int g, int s) { return *(const v4i *)(krow + 32 * s + 16 * g); }
+    __device__ acc_t step(kop_t kk, int s, acc_t acc) const { return __builtin_amdgcn_mfma_i32_32x32x32_i8(kk, q[s], acc, 0, 0, 0); }
     __device__ static float to_float(const acc_t &a, int r) { return (float)a[r]; }
     __device__ static float bits(const acc_t &a, int r) { return __int_as_float(a[r]); }
 };
@@ -132,6 +144,23 @@ __device__ inline void widen_v(v4i raw, float vs, v8h &lo, v8h &hi)
     }
     lo = v8h{h[0][0], h[0][1], h[1][0], h[1][1], h[2][0], h[2][1], h[3][0], h[3][1]};
     hi = v8h{h[4][0], h[4][1], h[5][0], h[5][1], h[6][0], h[6][1], h[7][0], h[7][1]};
+}
+
+// one 32-bit word (4 values) of the same: two packed pairs
+template <int DTYPE>
+__device__ inline void widen_v_word(int w, v2h vs2, v2h &h0, v2h &h1)
+{
+    if (DTYPE == TSATTN_I8) {
+        const unsigned u = (unsigned)w ^ 0x80808080u;
+        const unsigned a = __builtin_amdgcn_perm(u, 0x64646464u, 0x00050004u);
+        const unsigned b = __builtin_amdgcn_perm(u, 0x64646464u, 0x00070006u);
+        const v2h off = v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
+        h0 = (__builtin_bit_cast(v2h, a) + off) * vs2;
+        h1 = (__builtin_bit_cast(v2h, b) + off) * vs2;
+    } else {
+        h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false) * vs2;
+        h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true) * vs2;
+    }
 }
 
 typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
@@ -169,8 +198,25 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     // With d = 64 one 128-byte line of K or V holds the rows of two heads: consecutive workgroups then
     // alternate between the two heads of a pair on the same query tile, so the pair shares the line in L2.
     const int hg = (D == 64 && (p.n_heads & 1) == 0) ? 2 : 1;
-    const int head = (wg / (hg * n_qtiles)) * hg + wg % hg;
-    const int tile = n_qtiles - 1 - ((wg / hg) % n_qtiles); // long rows first
+    int head = (wg / (hg * n_qtiles)) * hg + wg % hg;
+    int tile = n_qtiles - 1 - ((wg / hg) % n_qtiles); // long rows first
+    // When the caller has said that the batch repeats the same span structure every T query tiles (equal-length
+    // sequences, causal), each XCD still gets a contiguous run of (head, sequence) units, but walks it position by
+    // position from the end of the sequences to their start: the longest rows of every unit first, the shortest
+    // last, so the launch does not end on a few long-running workgroups.
+    {
+        const int T = p.period_tiles;
+        const int per_xcd = n_wg >> 3;
+        if (T > 1 && (n_wg & 7) == 0 && per_xcd % (T * hg) == 0 && n_qtiles % T == 0) {
+            const int x = wg / per_xcd, i = wg % per_xcd;
+            const int R = per_xcd / (T * hg);
+            const int pos_rank = i / (R * hg), rem = i % (R * hg);
+            const int U = x * R + rem / hg, hsel = rem % hg;
+            const int n_seq = n_qtiles / T;
+            head = (U / n_seq) * hg + hsel;
+            tile = (U % n_seq) * T + (T - 1 - pos_rank);
+        }
+    }
     const int q0 = tile * PF_BM + wave * 32;
     const int from = q0 + qi;
     const bool row_ok = from < p.n_tokens;
@@ -408,27 +454,20 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         // sub-tile's weight sum shows that a logit was more than the threshold above it, the sub-tile is redone
         // on the slow path with a raised reference.
         constexpr float PF_SUM_LIMIT = 256.0f; // = 2^PF_RESCALE_THRESHOLD: one weight above it is enough to exceed it
-        auto weights_sub = [&](const typename Qk::acc_t &acc, const float *ksp, float nbase, v8h &pa, v8h &pb, float &s0, float &s1) {
-            v2h pp[8];
-#pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
-                const v4f ksv = *(const v4f *)(ksp + 8 * c4);
-#pragma unroll
-                for (int j2 = 0; j2 < 2; ++j2) {
-                    const int r = c4 * 4 + 2 * j2;
-                    const float x0 = Qk::to_float(acc, r) * ksv[2 * j2];
-                    const float x1 = Qk::to_float(acc, r + 1) * ksv[2 * j2 + 1];
-                    const float p0 = fast_exp2(fmaf(x0, qs, nbase));
-                    const float p1 = fast_exp2(fmaf(x1, qs, nbase));
-                    s0 += p0;
-                    s1 += p1;
-                    pp[r / 2] = v2h{(_Float16)p0, (_Float16)p1};
-                }
-            }
-            pa = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
-            pb = v8h{pp[4][0], pp[4][1], pp[5][0], pp[5][1], pp[6][0], pp[6][1], pp[7][0], pp[7][1]};
+        // weights of four keys (accumulator registers 4*c4 .. 4*c4+3)
+        auto weights_quarter = [&](const typename Qk::acc_t &acc, int c4, v4f ksv, float nbase, v2h &pa, v2h &pb, float &s0, float &s1) {
+            const int r = 4 * c4;
+            const float p0 = fast_exp2(fmaf(Qk::to_float(acc, r) * ksv[0], qs, nbase));
+            const float p1 = fast_exp2(fmaf(Qk::to_float(acc, r + 1) * ksv[1], qs, nbase));
+            const float p2 = fast_exp2(fmaf(Qk::to_float(acc, r + 2) * ksv[2], qs, nbase));
+            const float p3 = fast_exp2(fmaf(Qk::to_float(acc, r + 3) * ksv[3], qs, nbase));
+            s0 += p0;
+            s1 += p1;
+            s0 += p2;
+            s1 += p3;
+            pa = v2h{(_Float16)p0, (_Float16)p1};
+            pb = v2h{(_Float16)p2, (_Float16)p3};
         };
-        // slow path of one sub-tile: exact maximum, raise the reference, rescale the accumulators, redo the weights
         auto weights_sub_rescale = [&](const typename Qk::acc_t &acc, const float *ksp, v8h &pa, v8h &pb, float &s0, float &s1) {
             float xs[16];
             float tmax = -INFINITY;
@@ -459,53 +498,95 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             pa = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
             pb = v8h{pp[4][0], pp[4][1], pp[5][0], pp[5][1], pp[6][0], pp[6][1], pp[7][0], pp[7][1]};
         };
-        auto fast_tile = [&](auto stage_tag, int buf) {
-            constexpr bool STAGE = decltype(stage_tag)::value;
+#define PF_FENCE __builtin_amdgcn_sched_barrier(0)
+        auto fast_tile = [&](int buf) {
             static_assert(PF_KT == 2, "the common-tile path is written for 64-key tiles");
-            // ---- block 1 ----
-            const typename Qk::acc_t acc0 = qk.mma(k_lds[buf] + qi * L::K_PITCH, g);
-            const typename Qk::acc_t acc1 = qk.mma(k_lds[buf] + (32 + qi) * L::K_PITCH, g);
+            constexpr int QS = Qk::STEPS;
+            const uint8_t *kr0 = k_lds[buf] + qi * L::K_PITCH, *kr1 = kr0 + 32 * L::K_PITCH;
+            const float *ksp = ks_lds[buf] + 4 * g;
+            // ---- block 1: K.Q^T; sub-tile 0's weights between sub-tile 1's MFMAs ----
+            typename Qk::kop_t k0[QS], k1[QS];
+#pragma unroll
+            for (int st = 0; st < QS; ++st) k0[st] = Qk::load_k(kr0, g, st);
+#pragma unroll
+            for (int st = 0; st < QS; ++st) k1[st] = Qk::load_k(kr1, g, st);
+            PF_FENCE;
+            typename Qk::acc_t acc0 = {0}, acc1 = {0};
+#pragma unroll
+            for (int st = 0; st < QS; ++st) acc0 = qk.step(k0[st], st, acc0);
+            acc1 = qk.step(k1[0], 0, acc1);
+            v4f ksv[4];
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) ksv[c4] = *(const v4f *)(ksp + 8 * c4);
             vload(0, 0, buf);
             vload(1, 1, buf);
-            v8h p0a, p0b, p1a, p1b;
+            PF_FENCE;
+            v2h pp0[8], pp1[8];
             float s0 = 0.0f, s1 = 0.0f;
-            weights_sub(acc0, ks_lds[buf] + 4 * g, -m_ref, p0a, p0b, s0, s1);
-            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc0, ks_lds[buf] + 4 * g, p0a, p0b, s0, s1);
-            l += s0;
-            l2 += s1;
-            // ---- block 2 ----
+            const float nbase = -m_ref;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[0][dt], p0a, o_acc[dt], 0, 0, 0);
-            vload(0, 2, buf);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[1][dt], p0b, o_acc[dt], 0, 0, 0);
-            vload(1, 3, buf);
-            s0 = 0.0f;
-            s1 = 0.0f;
-            weights_sub(acc1, ks_lds[buf] + 32 + 4 * g, -m_ref, p1a, p1b, s0, s1);
-#pragma unroll
-            for (int i = 0; i < 2 * DT; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
-                __builtin_amdgcn_sched_group_barrier(0x002, 10, 0); // vector work of the other sub-tile behind it
-            }
-            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc1, ks_lds[buf] + 32 + 4 * g, p1a, p1b, s0, s1);
-            l += s0;
-            l2 += s1;
-            // ---- block 3 ----
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[0][dt], p1a, o_acc[dt], 0, 0, 0);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[1][dt], p1b, o_acc[dt], 0, 0, 0);
-            if (STAGE) {
-                store_tile(buf ^ 1);
-#pragma unroll
-                for (int i = 0; i < 2 * DT; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            for (int c4 = 0; c4 < 4; ++c4) {
+                weights_quarter(acc0, c4, ksv[c4], nbase, pp0[2 * c4], pp0[2 * c4 + 1], s0, s1);
+                PF_FENCE;
+                if (c4 + 1 < QS) {
+                    acc1 = qk.step(k1[c4 + 1], c4 + 1, acc1);
+                    PF_FENCE;
                 }
             }
+            v8h p0a = v8h{pp0[0][0], pp0[0][1], pp0[1][0], pp0[1][1], pp0[2][0], pp0[2][1], pp0[3][0], pp0[3][1]};
+            v8h p0b = v8h{pp0[4][0], pp0[4][1], pp0[5][0], pp0[5][1], pp0[6][0], pp0[6][1], pp0[7][0], pp0[7][1]};
+            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc0, ksp, p0a, p0b, s0, s1);
+            l += s0;
+            l2 += s1;
+            // ---- block 2: V^T.P^T of sub-tile 0; sub-tile 1's weights between the MFMAs ----
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) ksv[c4] = *(const v4f *)(ksp + 32 + 8 * c4);
+            s0 = 0.0f;
+            s1 = 0.0f;
+            const float nbase1 = -m_ref;
+            PF_FENCE;
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+                // MFMAs c4*DT/2 .. of the 2*DT of this block: group 0 (operand p0a) first, then group 1 (p0b)
+#pragma unroll
+                for (int j = 0; j < DT / 2; ++j) {
+                    const int m = c4 * (DT / 2) + j, grp = m / DT, dt = m % DT;
+                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[grp][dt], grp == 0 ? p0a : p0b, o_acc[dt], 0, 0, 0);
+                }
+                weights_quarter(acc1, c4, ksv[c4], nbase1, pp1[2 * c4], pp1[2 * c4 + 1], s0, s1);
+                if (c4 == 1) vload(0, 2, buf); // group 0's operands have been consumed
+                PF_FENCE;
+            }
+            vload(1, 3, buf);
+            v8h p1a = v8h{pp1[0][0], pp1[0][1], pp1[1][0], pp1[1][1], pp1[2][0], pp1[2][1], pp1[3][0], pp1[3][1]};
+            v8h p1b = v8h{pp1[4][0], pp1[4][1], pp1[5][0], pp1[5][1], pp1[6][0], pp1[6][1], pp1[7][0], pp1[7][1]};
+            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc1, ksp + 32, p1a, p1b, s0, s1);
+            l += s0;
+            l2 += s1;
+            // ---- block 3: V^T.P^T of sub-tile 1; the next tile's staging between the MFMAs ----
+            static_assert(LD_ALL && 4 * NLD == 2 * DT, "one 32-bit word of V per MFMA");
+            v2h hh[NLD][8];
+            PF_FENCE;
+#pragma unroll
+            for (int m = 0; m < 2 * DT; ++m) {
+                const int grp = m / DT, dt = m % DT;
+                o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[grp][dt], grp == 0 ? p1a : p1b, o_acc[dt], 0, 0, 0);
+                const int i = m / 4, w = m % 4;
+                const _Float16 vsh = (_Float16)rvs[i];
+                widen_v_word<DTYPE>(rv[i][w], v2h{vsh, vsh}, hh[i][2 * w], hh[i][2 * w + 1]);
+                if (w == 3) {
+                    const int ch = tid + i * PF_THREADS;
+                    const int r = ch / CHUNKS, c = ch % CHUNKS;
+                    uint8_t *vdst = v_lds[buf ^ 1] + r * L::V_PITCH + c * 32;
+                    *(v4i *)(k_lds[buf ^ 1] + r * L::K_PITCH + c * 16) = rk[i];
+                    *(v8h *)(vdst) = v8h{hh[i][0][0], hh[i][0][1], hh[i][1][0], hh[i][1][1], hh[i][2][0], hh[i][2][1], hh[i][3][0], hh[i][3][1]};
+                    *(v8h *)(vdst + 16) = v8h{hh[i][4][0], hh[i][4][1], hh[i][5][0], hh[i][5][1], hh[i][6][0], hh[i][6][1], hh[i][7][0], hh[i][7][1]};
+                }
+                PF_FENCE;
+            }
+            if (tid < PF_BN) ks_lds[buf ^ 1][tid] = rks * ads;
         };
+#undef PF_FENCE
 
         load_tile();
         store_tile(0);
@@ -543,7 +624,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             if constexpr (!SLOPE && !DUMP) {
                 if (pass == 0) {
                     for (; it < f1; ++it) {
-                        fast_tile(std::true_type{}, it & 1);
+                        fast_tile(it & 1);
                         if (it + 2 < n_tiles) load_tile();
                         __syncthreads();
                     }

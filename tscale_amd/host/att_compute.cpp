@@ -90,6 +90,27 @@ void TAttentionComputer::SetAttention(const TAttentionInfo &attInfo, void *strea
         }
     }
     Len = len;
+    // Launch-order hint: rows without keys mark sequence starts; if they are equally spaced, cover the batch and
+    // the window is wide (the last row of a sequence sees at least half of it), the batch has a causal period.
+    CausalPeriod = 0;
+    {
+        int period = 0, last = -1;
+        bool regular = len > 0 && fi[0] < st[0];
+        for (int t = 0; t < len && regular; ++t) {
+            if (fi[t] < st[t]) {
+                if (last >= 0) {
+                    if (period == 0) period = t - last;
+                    else if (t - last != period) regular = false;
+                }
+                last = t;
+            }
+        }
+        if (regular && period == 0) period = len; // a single sequence
+        if (regular && period > 0 && len % period == 0 && last == len - period) {
+            const int tail = len - 1;
+            if (fi[tail] - st[tail] + 1 >= period / 2) CausalPeriod = period;
+        }
+    }
     // pageable source: the copy has returned from the host's point of view when the call returns
     CheckHip(hipMemcpyAsync(SpanStart, st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
     CheckHip(hipMemcpyAsync(SpanFinish, fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
@@ -117,6 +138,7 @@ void TAttentionComputer::ComputeValLookup(int len, int dtype, const TQuantRows &
     a.alibi_slope = AlibiSlope;
     a.out = valLookup; a.out_pitch = valLookupPitchBytes;
     a.sum_weight_log = SumWeightLog;
+    a.causal_period = CausalPeriod;
     Check(tsattn_prefill(Handle, &a, stream), "tsattn_prefill");
 }
 

@@ -75,6 +75,7 @@ class TAttentionComputer
     float AlibiSlope = 0;
     int MaxLen = 0;
     int Len = 0;
+    int CausalPeriod = 0; // launch-order hint derived from the spans by SetAttention
     int32_t *SpanStart = nullptr; // device
     int32_t *SpanFinish = nullptr;
     float *SumWeightLog = nullptr; // device [headCount][MaxLen]
