@@ -362,25 +362,24 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         };
 
         // ---- one 64-key tile for this wave's 32 queries ---------------------------------------------------
+        // General form: any mix of rows, one 32-key sub-tile at a time (few live registers; a sub-tile outside
+        // every span of the wave is skipped, which for a short window is one in four).
         auto compute_tile = [&](auto interior_tag, auto ref_tag, int buf, int kb) {
             constexpr bool INTERIOR = decltype(interior_tag)::value;
             constexpr bool REF = decltype(ref_tag)::value || SLOPE; // general form: logit * qs + base
-            float t[PF_KT][16];
-            float tmax = -INFINITY;
             // keys of register r of sub-tile kt: kb + kt*32 + 8*(r/4) + 4*g + r%4
             const int rel_a = sp_a - kb - 4 * g;            // span start relative to this lane's first key
             const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
             const float dist0 = (float)(from - kb - 4 * g);
-            const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
-            typename Qk::acc_t accs[PF_KT];
-#pragma unroll
-            for (int kt = 0; kt < PF_KT; ++kt) accs[kt] = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
-            vload(0, 0, buf);
-            vload(1, 1, buf);
-            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kt = 0; kt < PF_KT; ++kt) {
-                typename Qk::acc_t acc = accs[kt];
+                if (!INTERIOR && (kb + kt * 32 + 31 < w_min_a || kb + kt * 32 > w_max_b)) continue;
+                float t[16];
+                float tmax = -INFINITY;
+                const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
+                const typename Qk::acc_t acc = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
+                vload(0, 2 * kt, buf);
+                vload(1, 2 * kt + 1, buf);
 #pragma unroll
                 for (int c4 = 0; c4 < 4; ++c4) {
                     const int off0 = kt * 32 + 8 * c4;
@@ -395,52 +394,45 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                                 ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + kb + off + 4 * g] = Qk::bits(acc, r);
                             }
                         }
-                        // while the reference maximum is still 0 (no slope): two 2-operand multiplies
                         float x = Qk::to_float(acc, r) * ksv[j];
                         float tv = REF ? fmaf(x, qs, base) : x * qs;
                         if (SLOPE) tv += p.slope * (float)off;
                         if (!INTERIOR) tv = in_span ? tv : -INFINITY;
-                        t[kt][r] = tv;
-                        tmax = max2(tmax, tv);
+                        t[r] = tv;
+                        tmax = fmaxf(tmax, tv);
                     }
                 }
-            }
-            // the two lanes of a query exchange their maxima only if some lane of the wave is over the
-            // threshold: the common path has no cross-lane operation at all
-            if (__any(tmax > PF_RESCALE_THRESHOLD)) {
-                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-                const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
-                const float alpha = fast_exp2(-shift);
-                have_ref = true;
-                m_ref += shift;
-                l *= alpha;
-                l2 *= alpha;
+                // the two lanes of a query exchange their maxima only if some lane of the wave is over the
+                // threshold: the common case has no cross-lane operation at all
+                if (__any(tmax > PF_RESCALE_THRESHOLD)) {
+                    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+                    const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
+                    const float alpha = fast_exp2(-shift);
+                    have_ref = true;
+                    m_ref += shift;
+                    l *= alpha;
+                    l2 *= alpha;
 #pragma unroll
-                for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
+                    for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
 #pragma unroll
-                for (int kt = 0; kt < PF_KT; ++kt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) t[kt][r] -= shift;
-            }
-            // P = 2^t ; O^T += V^T . P^T in four groups of DT MFMAs (16 keys each).  The V^T operands of a
-            // group are read from LDS two groups ahead (ring of two register sets) so that no MFMA waits
-            // for an LDS round trip.
-#pragma unroll
-            for (int grp = 0; grp < 2 * PF_KT; ++grp) {
-                const int kt = grp >> 1, i = grp & 1;
-                v2h pp[4];
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const float p0 = fast_exp2(t[kt][8 * i + 2 * x]);
-                    const float p1 = fast_exp2(t[kt][8 * i + 2 * x + 1]);
-                    pp[x] = v2h{(_Float16)p0, (_Float16)p1};
-                    l += p0;
-                    l2 += p1;
+                    for (int r = 0; r < 16; ++r) t[r] -= shift;
                 }
-                const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
+                // P = 2^t ; O^T += V^T . P^T in two groups of DT MFMAs (16 keys each)
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[grp & 1][dt], pb, o_acc[dt], 0, 0, 0);
-                if (grp + 2 < 2 * PF_KT) vload(grp & 1, grp + 2, buf);
+                for (int i = 0; i < 2; ++i) {
+                    v2h pp[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const float p0 = fast_exp2(t[8 * i + 2 * x]);
+                        const float p1 = fast_exp2(t[8 * i + 2 * x + 1]);
+                        pp[x] = v2h{(_Float16)p0, (_Float16)p1};
+                        l += p0;
+                        l2 += p1;
+                    }
+                    const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[i][dt], pb, o_acc[dt], 0, 0, 0);
+                }
             }
         };
 
