@@ -228,6 +228,12 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         sp_a = p.span_start[from];
         sp_b = p.span_finish[from];
     }
+    // ---- query operand and per-row constants (issued before the span reductions so that their latency
+    //      runs under them) ---------------------------------------------------------------------------
+    Qk qk;
+    if (row_ok) qk.load_q(p.q + (int64_t)from * p.q_pitch + hoff, g);
+    else qk.clear_q();
+    const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
     const bool has_keys = sp_b >= sp_a;
     const bool w_all_have_keys = __all(has_keys);
     int w_min_a = has_keys ? sp_a : 0x7fffffff, w_max_a = has_keys ? sp_a : -1;
@@ -249,11 +255,6 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         b_max_b = max(b_max_b, red_lds[PF_WAVES + w]);
     }
 
-    // ---- query operand and per-row constants -------------------------------------------------------
-    Qk qk;
-    if (row_ok) qk.load_q(p.q + (int64_t)from * p.q_pitch + hoff, g);
-    else qk.clear_q();
-    const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
     float ads = att_dot_scale(D);
     if (p.k_global_scale) ads *= *p.k_global_scale;
 
