@@ -46,6 +46,7 @@ struct PrefillParams {
     int n_tokens;
     int n_heads;
     int period_tiles; // query tiles per period of equal span structure, 0 = unknown (launch order only)
+    int period_group; // set by the launcher: units per group of the period-aware launch order, 0 = not used
 };
 
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int head_dim, int out_dtype, hipStream_t st);

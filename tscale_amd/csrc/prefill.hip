@@ -201,17 +201,19 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     int head = (wg / (hg * n_qtiles)) * hg + wg % hg;
     int tile = n_qtiles - 1 - ((wg / hg) % n_qtiles); // long rows first
     // When the caller has said that the batch repeats the same span structure every T query tiles (equal-length
-    // sequences, causal), each XCD still gets a contiguous run of (head, sequence) units, but walks it position by
-    // position from the end of the sequences to their start: the longest rows of every unit first, the shortest
-    // last, so the launch does not end on a few long-running workgroups.
+    // sequences, causal), each XCD still gets a contiguous run of (head, sequence) units, but walks groups of G
+    // units position by position from the end of the sequences to their start: the longest rows of every unit
+    // first, the shortest last, so the launch does not end on a few long-running workgroups.  G is chosen by
+    // the host so that the K/V rows of a group fit in the XCD's L2.
     {
-        const int T = p.period_tiles;
+        const int T = p.period_tiles, G = p.period_group;
         const int per_xcd = n_wg >> 3;
-        if (T > 1 && (n_wg & 7) == 0 && per_xcd % (T * hg) == 0 && n_qtiles % T == 0) {
+        if (T > 1 && G > 0) {
             const int x = wg / per_xcd, i = wg % per_xcd;
             const int R = per_xcd / (T * hg);
-            const int pos_rank = i / (R * hg), rem = i % (R * hg);
-            const int U = x * R + rem / hg, hsel = rem % hg;
+            const int grp = i / (G * T * hg), j = i % (G * T * hg);
+            const int pos_rank = j / (G * hg), rem = j % (G * hg);
+            const int U = x * R + grp * G + rem / hg, hsel = rem % hg;
             const int n_seq = n_qtiles / T;
             head = (U / n_seq) * hg + hsel;
             tile = (U % n_seq) * T + (T - 1 - pos_rank);
@@ -654,10 +656,28 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
 }
 
 template <int DTYPE, int D, bool OUT_F16>
-static void launch_prefill_do(const PrefillParams &p, dim3 grid2, hipStream_t st)
+static void launch_prefill_do(const PrefillParams &p_in, dim3 grid2, hipStream_t st)
 {
     const int n_qtiles = (int)grid2.x;
     dim3 grid(grid2.x * grid2.y);
+    // Launch-order hint: usable only if every XCD's share of the grid is a whole number of (head group, sequence)
+    // units; units are then walked in groups whose K and V rows (2 * period * d bytes per head) stay within
+    // about the size of the XCD's 4 MB L2 (the rows are streamed, so slightly more than it still pays).
+    PrefillParams p = p_in;
+    p.period_group = 0;
+    {
+        const int T = p.period_tiles;
+        const int hg = (D == 64 && (p.n_heads & 1) == 0) ? 2 : 1;
+        const int n_wg = (int)grid.x, per_xcd = n_wg / 8;
+        if (T > 1 && n_wg % 8 == 0 && per_xcd % (T * hg) == 0 && n_qtiles % T == 0) {
+            const int R = per_xcd / (T * hg);
+            const int64_t unit_bytes = (int64_t)2 * T * PF_BM * D * hg;
+            int G = 1;
+            for (int c = 1; c <= R; ++c)
+                if (R % c == 0 && c * unit_bytes <= (5 << 20)) G = c;
+            p.period_group = G;
+        }
+    }
     const bool dump = p.dbg != nullptr;
     const bool slope = p.slope != 0.0f;
     dim3 block(PF_THREADS);
