@@ -80,6 +80,7 @@ class PrefillWorkload:
             self.inputs.append(qkv)
         off = torch.arange(0, n + 1, S, dtype=torch.int32, device="cuda")
         self.spans = {W: ctx.build_spans(off, n, W) for W in {w for w, _ in self.layers}}
+        self.span_tiles = {W: ctx.build_span_tiles(*sp) for W, sp in self.spans.items()}   # once per batch and mask
         self.out = torch.empty((n, H * d), dtype=torch.float16, device="cuda")
         self.flops_layer = [prefill_flops(B, S, H, d, W) for W, _ in self.layers]
         self.flops = sum(self.flops_layer)
@@ -91,7 +92,7 @@ class PrefillWorkload:
         st, fi = self.spans[W]
         # equal-length sequences: tell the library the causal period of the wide layers (a launch-order hint)
         self.ctx.compute_val_lookup(self.dtype, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
-                                    causal_period=self.S if W >= self.S else 0)
+                                    causal_period=self.S if W >= self.S else 0, span_tiles=self.span_tiles[W])
 
     def step(self):
         for i in range(len(self.layers)):
@@ -149,6 +150,7 @@ class GenerationWorkload:
         self.qkv = [ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g), H, capi.I8) for _ in range(3)]
         self.off = torch.arange(0, n + 1, prompt, dtype=torch.int32, device="cuda")
         self.spans = {W: ctx.build_spans(self.off, n, W) for W in {w for w, _ in self.sched}}
+        self.span_tiles = {W: ctx.build_span_tiles(*sp) for W, sp in self.spans.items()}
         self.out = torch.empty((n, H * d), dtype=torch.float16, device="cuda")
         self.caches = [KVCache(ctx, capi.I8, B, H, self.L, d) for _ in range(depth)]
         new = [ctx.quantize_rows(torch.randn((B, H * d), device="cuda", generator=g), H, capi.I8) for _ in range(3)]
@@ -162,7 +164,7 @@ class GenerationWorkload:
         W, slope = self.sched[i]
         st, fi = self.spans[W]
         self.ctx.compute_val_lookup(self.i8, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
-                                    causal_period=self.prompt if W >= self.prompt else 0)
+                                    causal_period=self.prompt if W >= self.prompt else 0, span_tiles=self.span_tiles[W])
 
     def fill_caches(self):
         (_, _), (k, ks), (v, vs) = self.qkv

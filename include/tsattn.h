@@ -94,6 +94,10 @@ typedef struct tsattn_prefill_args {
     void *debug_qk_acc;          /* optional raw QK^T accumulators, [n_heads][n_tokens][debug_pitch]
                                     int32 (int8 inputs) or f32 (e4m3); only in-span pairs are written */
     int64_t debug_pitch;         /* elements per (head, from) row of debug_qk_acc */
+    const int32_t *span_tiles;   /* optional: what tsattn_build_span_tiles made from THESE span arrays (per 128 query
+                                    rows the key range the rows need, per 32 rows the extremes of their spans); the
+                                    kernel then starts loading K and V without first reducing the spans itself.
+                                    NULL = derive it in the kernel.  Same result either way. */
     int64_t causal_period;       /* scheduling hint, 0 = none: rows t and t + causal_period have spans of equal
                                     length and spans grow with t inside a period (a batch of equal-length
                                     sequences under a wide causal window, as the reference's fixed-length
@@ -181,6 +185,16 @@ typedef struct tsattn_fill_args {
 } tsattn_fill_args;
 
 int tsattn_cache_fill(tsattn_handle_t h, const tsattn_fill_args *a, void *stream);
+
+/* Summary of a span list for tsattn_prefill (its span_tiles argument), built once per batch and mask and shared
+ * by every layer and head that uses the same spans: TSATTN_SPAN_TILE_INTS int32 per 128 query rows.
+ * The reference builds its per-64-row tile-skip list on the host for the same purpose
+ * (TAttentionSpanGroup / GroupAttention, gpt/att/att.h:56-64,95-181).  tiles: device array of
+ * tsattn_span_tiles_count(n_tokens) * TSATTN_SPAN_TILE_INTS int32. */
+#define TSATTN_SPAN_TILE_INTS 32
+int64_t tsattn_span_tiles_count(int64_t n_tokens);
+int tsattn_build_span_tiles(tsattn_handle_t h, int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish,
+                            int32_t *tiles, void *stream);
 
 /* Per-(row, head) absmax quantiser: scale = absmax/127 (int8) or absmax/256 (e4m3), values
  * round-to-nearest-even, int8 clamped to [-127,127].  Replaces NormalizeVecsRowTileMax /

@@ -188,3 +188,42 @@ def test_prefill_logits_far_above_the_zero_vector(ctx):
             assert want_swl.max() > 20.0 if boost > 10 else want_swl.max() > 4.0
             assert_within_tolerance(out, want, f"boost {boost}")
             assert np.abs(swl - want_swl).max() < 2e-3 * max(1.0, np.abs(want_swl).max() / 16)
+
+
+@pytest.mark.parametrize("window,slope", [(10 ** 6, 0.0), (64, 0.5), (0, 0.0), (5, 0.2)])
+def test_prefill_span_summary_gives_identical_results(ctx, window, slope):
+    """With the per-128-row span summary (tsattn_build_span_tiles) the kernel skips its own span reduction; the
+    summary equals a numpy reduction of the spans and the output is bit-identical to the run without it.  Ragged
+    sequences, document starts, rows without keys, a last partial tile."""
+    H, d, dtype = 2, 64, capi.E4M3
+    seq_lens = [300, 1, 129, 70, 513]
+    n = sum(seq_lens)
+    rng = np.random.default_rng(3)
+    flags = (rng.random(n) < 0.01).astype(np.uint8)
+    q, qs, k, ks, v, vs = make_qkv(8, n, H, d, dtype)
+    st, fi = orc.make_spans(seq_lens, window, flags)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    tiles = ctx.build_span_tiles(t(st), t(fi))
+    got_tiles = tiles.cpu().numpy()
+    n_tiles = (n + 127) // 128
+    assert got_tiles.shape == (n_tiles, capi.SPAN_TILE_INTS)
+    for i in range(n_tiles):
+        a, b = st[i * 128:(i + 1) * 128], fi[i * 128:(i + 1) * 128]
+        has = b >= a
+        want_min = a[has].min() if has.any() else 0x7fffffff
+        want_max = b[has].max() if has.any() else -1
+        assert got_tiles[i, 0] == want_min and got_tiles[i, 1] == want_max
+        for w in range(4):
+            aw, bw = a[32 * w:32 * w + 32], b[32 * w:32 * w + 32]
+            hw = bw >= aw
+            e = got_tiles[i, 4 + 5 * w: 9 + 5 * w]
+            if hw.any():
+                assert e.tolist()[:4] == [aw[hw].min(), aw[hw].max(), bw[hw].min(), bw[hw].max()]
+            else:
+                assert e[0] > e[3]
+            assert e[4] == int(len(aw) == 32 and hw.all())
+    args = (dtype, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), slope)
+    base = ctx.compute_val_lookup(*args).cpu().numpy()
+    with_tiles = ctx.compute_val_lookup(*args, span_tiles=tiles).cpu().numpy()
+    assert np.array_equal(base, with_tiles)
+    assert_within_tolerance(base, orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, slope), "span summary")

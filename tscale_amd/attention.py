@@ -92,13 +92,21 @@ class AttentionContext:
                                                _ptr(doc_start_flag), int(window), _ptr(st), _ptr(fi), _stream_ptr()))
         return st, fi
 
+    def build_span_tiles(self, span_start, span_finish):
+        """Per-128-row summary of a span list for compute_val_lookup(span_tiles=...); build once per batch and mask."""
+        n = span_start.numel()
+        tiles = torch.empty((self.lib.tsattn_span_tiles_count(n), capi.SPAN_TILE_INTS), dtype=torch.int32, device=self.device)
+        capi.check(self.lib.tsattn_build_span_tiles(self.handle, n, _ptr(span_start), _ptr(span_finish), _ptr(tiles),
+                                                    _stream_ptr()))
+        return tiles
+
     # ---- prefill --------------------------------------------------------------------------------
     def compute_val_lookup(self, dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, span_start, span_finish,
                            alibi_slope, out=None, out_f16=False, sum_weight_log=None, k_global_scale=None,
-                           debug_qk_acc=None, causal_period=0):
+                           debug_qk_acc=None, causal_period=0, span_tiles=None):
         """q,k,v: uint8 [n_tokens, n_heads*d] (row pitch = stride(0)); scales f32 [n_heads, n_tokens] or numbers.
         causal_period: launch-order hint for batches of equal-length sequences under a wide causal window (the
-        common sequence length); never changes the result."""
+        common sequence length); never changes the result.  span_tiles: what build_span_tiles made of these spans."""
         n_tokens, hd = q.shape
         d = hd // n_heads
         if out is None:
@@ -123,6 +131,7 @@ class AttentionContext:
         if debug_qk_acc is not None:
             a.debug_qk_acc, a.debug_pitch = _ptr(debug_qk_acc), debug_qk_acc.stride(1)
         a.causal_period = int(causal_period)
+        a.span_tiles = _ptr(span_tiles)
         capi.check(self.lib.tsattn_prefill(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
 

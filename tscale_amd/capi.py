@@ -14,6 +14,7 @@ I8, E4M3 = 0, 1
 OUT_F32, OUT_F16 = 0, 1
 SRC_F32, SRC_BF16 = 0, 1
 Q_8BIT, Q_BF16 = 0, 1
+SPAN_TILE_INTS = 32
 
 STATUS_NAMES = {0: "OK", 1: "BAD_ARG", 2: "UNSUPPORTED", 3: "HIP", 4: "SCRATCH"}
 
@@ -39,7 +40,7 @@ class PrefillArgs(_c.Structure):
         ("v_scale_const", _c.c_float), ("k_global_scale", _c.c_void_p), ("span_start", _c.c_void_p),
         ("span_finish", _c.c_void_p), ("alibi_slope", _c.c_float), ("out", _c.c_void_p),
         ("out_pitch", _c.c_int64), ("sum_weight_log", _c.c_void_p), ("debug_qk_acc", _c.c_void_p),
-        ("debug_pitch", _c.c_int64), ("causal_period", _c.c_int64),
+        ("debug_pitch", _c.c_int64), ("span_tiles", _c.c_void_p), ("causal_period", _c.c_int64),
     ]
 
 
@@ -81,7 +82,7 @@ class FillArgs(_c.Structure):
 
 
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
+           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
 
 _lib = None
 
@@ -111,6 +112,10 @@ def load():
         L.tsattn_cache_append.argtypes = [_c.c_void_p, _c.POINTER(AppendArgs), _c.c_void_p]
         L.tsattn_cache_fill.restype = _c.c_int
         L.tsattn_cache_fill.argtypes = [_c.c_void_p, _c.POINTER(FillArgs), _c.c_void_p]
+        L.tsattn_span_tiles_count.restype = _c.c_int64
+        L.tsattn_span_tiles_count.argtypes = [_c.c_int64]
+        L.tsattn_build_span_tiles.restype = _c.c_int
+        L.tsattn_build_span_tiles.argtypes = [_c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]
         L.tsattn_quantize_rows.restype = _c.c_int
         L.tsattn_quantize_rows.argtypes = [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64,
                                            _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64,

@@ -128,6 +128,7 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     p.qs_const = a->q_scale_const; p.ks_const = a->k_scale_const; p.vs_const = a->v_scale_const;
     p.k_global_scale = a->k_global_scale;
     p.span_start = a->span_start; p.span_finish = a->span_finish;
+    p.span_tiles = a->span_tiles;
     p.slope = a->alibi_slope;
     p.out = a->out; p.out_pitch = a->out_pitch;
     p.sum_weight_log = a->sum_weight_log;
@@ -207,6 +208,24 @@ int tsattn_cache_append(tsattn_handle_t h, const tsattn_append_args *a, void *st
     p.cache_len = a->cache_len; p.max_len = a->max_len; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
     hipError_t e = tsattn::launch_cache_append(p, a->n_seqs, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "cache append launch");
+    return TSATTN_OK;
+}
+
+int64_t tsattn_span_tiles_count(int64_t n_tokens)
+{
+    return n_tokens <= 0 ? 0 : (n_tokens + 127) / 128;
+}
+
+int tsattn_build_span_tiles(tsattn_handle_t h, int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish,
+                            int32_t *tiles, void *stream)
+{
+    if (!h) return fail(TSATTN_ERR_BAD_ARG, "tsattn_build_span_tiles: null handle");
+    if (n_tokens < 0 || n_tokens > 0x7fffffff) return fail(TSATTN_ERR_BAD_ARG, "tsattn_build_span_tiles: n_tokens %lld", (long long)n_tokens);
+    if (n_tokens == 0) return TSATTN_OK;
+    if (!span_start || !span_finish || !tiles) return fail(TSATTN_ERR_BAD_ARG, "tsattn_build_span_tiles: null data pointer");
+    if ((uintptr_t)tiles % 16) return fail(TSATTN_ERR_BAD_ARG, "tsattn_build_span_tiles: tiles must be 16-byte aligned");
+    hipError_t e = tsattn::launch_build_span_tiles(n_tokens, span_start, span_finish, tiles, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "span tiles launch");
     return TSATTN_OK;
 }
 

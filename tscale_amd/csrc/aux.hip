@@ -103,6 +103,52 @@ hipError_t launch_build_spans(int n_seqs, const int32_t *seq_offset, int64_t n_t
     return hipGetLastError();
 }
 
+// Span summary for the prefill kernel: one workgroup of 128 threads per 128 query rows, one wave half (32 lanes)
+// per 32-row group.  Rows without keys (span_finish < span_start) and rows past the end do not count.
+__global__ __launch_bounds__(128) void span_tiles_kernel(int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish, int32_t *tiles)
+{
+    __shared__ int red[8];
+    const int tid = threadIdx.x;
+    const int64_t row = (int64_t)blockIdx.x * 128 + tid;
+    int a = 1, b = 0;
+    if (row < n_tokens) {
+        a = span_start[row];
+        b = span_finish[row];
+    }
+    const bool has = b >= a;
+    int min_a = has ? a : 0x7fffffff, max_a = has ? a : -1, min_b = has ? b : 0x7fffffff, max_b = has ? b : -1;
+    int all = has ? 1 : 0;
+    for (int o = 16; o > 0; o >>= 1) { // within each 32-lane half
+        min_a = min(min_a, __shfl_xor(min_a, o, WAVE));
+        max_a = max(max_a, __shfl_xor(max_a, o, WAVE));
+        min_b = min(min_b, __shfl_xor(min_b, o, WAVE));
+        max_b = max(max_b, __shfl_xor(max_b, o, WAVE));
+        all &= __shfl_xor(all, o, WAVE);
+    }
+    int32_t *out = tiles + (int64_t)blockIdx.x * SPAN_TILE_INTS;
+    const int grp = tid >> 5;
+    if ((tid & 31) == 0) {
+        int32_t *w = out + SPAN_TILE_WAVE0 + grp * SPAN_TILE_WAVE_INTS;
+        w[0] = min_a; w[1] = max_a; w[2] = min_b; w[3] = max_b; w[4] = all;
+        red[grp] = min_a;
+        red[4 + grp] = max_b;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        out[SPAN_TILE_MIN_A] = min(min(red[0], red[1]), min(red[2], red[3]));
+        out[SPAN_TILE_MAX_B] = max(max(red[4], red[5]), max(red[6], red[7]));
+        out[2] = 0; out[3] = 0;
+        for (int i = SPAN_TILE_WAVE0 + 4 * SPAN_TILE_WAVE_INTS; i < SPAN_TILE_INTS; ++i) out[i] = 0;
+    }
+}
+
+hipError_t launch_build_span_tiles(int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish, int32_t *tiles, hipStream_t st)
+{
+    if (n_tokens <= 0) return hipSuccess;
+    hipLaunchKernelGGL(span_tiles_kernel, dim3((unsigned)((n_tokens + 127) / 128)), dim3(128), 0, st, n_tokens, span_start, span_finish, tiles);
+    return hipGetLastError();
+}
+
 // TAttentionVecHistory::AddVectors (gpt/train/cpu_infer.cpp:403-408) for a planar cache: one thread
 // copies 16 bytes of the new K and V rows to row cache_len[seq]; a second kernel bumps the lengths.
 __global__ __launch_bounds__(256) void cache_append_kernel(AppendParams p, int n_seqs)

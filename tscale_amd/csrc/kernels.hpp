@@ -37,6 +37,7 @@ struct PrefillParams {
     float qs_const, ks_const, vs_const;
     const float *k_global_scale;
     const int32_t *span_start, *span_finish;
+    const int32_t *span_tiles; // optional per-128-row summary (SPAN_TILE_* layout below)
     float slope;
     void *out;
     int64_t out_pitch;
@@ -54,6 +55,13 @@ hipError_t launch_prefill(const PrefillParams &p, int dtype, int head_dim, int o
 hipError_t launch_quantize_rows(int src_dtype, int dst_dtype, const void *src, int64_t src_pitch, int64_t n_rows,
                                 int n_heads, int head_dim, void *dst, int64_t dst_pitch, float *scale,
                                 int64_t scale_pitch, hipStream_t st);
+
+// Layout of one entry of the span summary (32 int32 per 128 query rows): the workgroup's key range, then for each
+// of its four 32-row waves the extremes of the rows' spans and whether every row has keys.
+constexpr int SPAN_TILE_INTS = 32;
+constexpr int SPAN_TILE_MIN_A = 0, SPAN_TILE_MAX_B = 1; // over rows that have keys; MIN_A > MAX_B if none has
+constexpr int SPAN_TILE_WAVE0 = 4, SPAN_TILE_WAVE_INTS = 5; // per wave: min_a, max_a, min_b, max_b, all_have_keys
+hipError_t launch_build_span_tiles(int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish, int32_t *tiles, hipStream_t st);
 
 hipError_t launch_build_spans(int n_seqs, const int32_t *seq_offset, int64_t n_tokens, const uint8_t *doc_start_flag,
                               int64_t window, int32_t *span_start, int32_t *span_finish, hipStream_t st);

@@ -237,24 +237,42 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     else qk.clear_q();
     const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
     const bool has_keys = sp_b >= sp_a;
-    const bool w_all_have_keys = __all(has_keys);
-    int w_min_a = has_keys ? sp_a : 0x7fffffff, w_max_a = has_keys ? sp_a : -1;
-    int w_min_b = has_keys ? sp_b : 0x7fffffff, w_max_b = has_keys ? sp_b : -1;
-    for (int o = 16; o > 0; o >>= 1) {
-        w_min_a = min(w_min_a, __shfl_xor(w_min_a, o, WAVE));
-        w_max_a = max(w_max_a, __shfl_xor(w_max_a, o, WAVE));
-        w_min_b = min(w_min_b, __shfl_xor(w_min_b, o, WAVE));
-        w_max_b = max(w_max_b, __shfl_xor(w_max_b, o, WAVE));
-    }
-    if (lane == 0) {
-        red_lds[wave] = w_min_a;
-        red_lds[PF_WAVES + wave] = w_max_b;
-    }
-    __syncthreads();
-    int b_min_a = red_lds[0], b_max_b = red_lds[PF_WAVES];
-    for (int w = 1; w < PF_WAVES; ++w) {
-        b_min_a = min(b_min_a, red_lds[w]);
-        b_max_b = max(b_max_b, red_lds[PF_WAVES + w]);
+    // What the loop needs to know about the spans: the workgroup's key range and the extremes of this wave's 32
+    // spans.  Either read from the caller's summary (scalar loads, so K and V can be requested at once) or
+    // reduced here from the rows' spans (shuffles, LDS, a barrier).
+    bool w_all_have_keys;
+    int w_min_a, w_max_a, w_min_b, w_max_b, b_min_a, b_max_b;
+    if (p.span_tiles) {
+        typedef __attribute__((address_space(4))) const int32_t *const_i32_ptr;
+        const const_i32_ptr t = (const_i32_ptr)(p.span_tiles + (int64_t)tile * SPAN_TILE_INTS);
+        const const_i32_ptr w = t + SPAN_TILE_WAVE0 + __builtin_amdgcn_readfirstlane(wave) * SPAN_TILE_WAVE_INTS;
+        b_min_a = t[SPAN_TILE_MIN_A];
+        b_max_b = t[SPAN_TILE_MAX_B];
+        w_min_a = w[0];
+        w_max_a = w[1];
+        w_min_b = w[2];
+        w_max_b = w[3];
+        w_all_have_keys = w[4] != 0;
+    } else {
+        w_all_have_keys = __all(has_keys);
+        w_min_a = has_keys ? sp_a : 0x7fffffff, w_max_a = has_keys ? sp_a : -1;
+        w_min_b = has_keys ? sp_b : 0x7fffffff, w_max_b = has_keys ? sp_b : -1;
+        for (int o = 16; o > 0; o >>= 1) {
+            w_min_a = min(w_min_a, __shfl_xor(w_min_a, o, WAVE));
+            w_max_a = max(w_max_a, __shfl_xor(w_max_a, o, WAVE));
+            w_min_b = min(w_min_b, __shfl_xor(w_min_b, o, WAVE));
+            w_max_b = max(w_max_b, __shfl_xor(w_max_b, o, WAVE));
+        }
+        if (lane == 0) {
+            red_lds[wave] = w_min_a;
+            red_lds[PF_WAVES + wave] = w_max_b;
+        }
+        __syncthreads();
+        b_min_a = red_lds[0], b_max_b = red_lds[PF_WAVES];
+        for (int w = 1; w < PF_WAVES; ++w) {
+            b_min_a = min(b_min_a, red_lds[w]);
+            b_max_b = max(b_max_b, red_lds[PF_WAVES + w]);
+        }
     }
 
     float ads = att_dot_scale(D);
@@ -264,7 +282,6 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
 #pragma unroll
     for (int i = 0; i < DT; ++i) o_acc[i] = v16f{0};
     float m_ref = 0.0f; // reference maximum: starts at the zero vector's logit
-    bool have_ref = false; // wave-uniform: some lane of this wave has m_ref != 0
     float l = 0.0f, l2 = 0.0f; // this lane's share of the weight sum (its 32 of every 64 keys), in two chains
 
     if (b_max_b >= b_min_a) {
@@ -411,7 +428,6 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
                     const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
                     const float alpha = fast_exp2(-shift);
-                    have_ref = true;
                     m_ref += shift;
                     l *= alpha;
                     l2 *= alpha;
@@ -474,7 +490,6 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
             const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
             const float alpha = fast_exp2(-shift);
-            have_ref = true;
             m_ref += shift;
             l *= alpha;
             l2 *= alpha;

@@ -62,6 +62,7 @@ TAttentionComputer::TAttentionComputer(const TModelDims &dims, float alibiSlope,
     Check(tsattn_create(&cfg, &Handle), "tsattn_create");
     CheckHip(hipMalloc((void **)&SpanStart, sizeof(int32_t) * (size_t)maxLen), "hipMalloc(spans)");
     CheckHip(hipMalloc((void **)&SpanFinish, sizeof(int32_t) * (size_t)maxLen), "hipMalloc(spans)");
+    CheckHip(hipMalloc((void **)&SpanTiles, sizeof(int32_t) * TSATTN_SPAN_TILE_INTS * (size_t)tsattn_span_tiles_count(maxLen)), "hipMalloc(span tiles)");
     CheckHip(hipMalloc((void **)&SumWeightLog, sizeof(float) * (size_t)maxLen * dims.HeadCount), "hipMalloc(sumWeightLog)");
 }
 
@@ -69,6 +70,7 @@ TAttentionComputer::~TAttentionComputer()
 {
     (void)hipFree(SpanStart);
     (void)hipFree(SpanFinish);
+    (void)hipFree(SpanTiles);
     (void)hipFree(SumWeightLog);
     tsattn_destroy(Handle);
 }
@@ -114,6 +116,7 @@ void TAttentionComputer::SetAttention(const TAttentionInfo &attInfo, void *strea
     // pageable source: the copy has returned from the host's point of view when the call returns
     CheckHip(hipMemcpyAsync(SpanStart, st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
     CheckHip(hipMemcpyAsync(SpanFinish, fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
+    Check(tsattn_build_span_tiles(Handle, len, SpanStart, SpanFinish, SpanTiles, stream), "tsattn_build_span_tiles");
     CheckHip(hipStreamSynchronize((hipStream_t)stream), "span copy");
 }
 
@@ -135,6 +138,7 @@ void TAttentionComputer::ComputeValLookup(int len, int dtype, const TQuantRows &
     a.q_scale_const = qk.ConstScale; a.k_scale_const = qv.ConstScale; a.v_scale_const = v.ConstScale;
     a.k_global_scale = qvGlobalScale;
     a.span_start = SpanStart; a.span_finish = SpanFinish;
+    a.span_tiles = SpanTiles;
     a.alibi_slope = AlibiSlope;
     a.out = valLookup; a.out_pitch = valLookupPitchBytes;
     a.sum_weight_log = SumWeightLog;

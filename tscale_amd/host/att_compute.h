@@ -78,6 +78,7 @@ class TAttentionComputer
     int CausalPeriod = 0; // launch-order hint derived from the spans by SetAttention
     int32_t *SpanStart = nullptr; // device
     int32_t *SpanFinish = nullptr;
+    int32_t *SpanTiles = nullptr; // per-128-row summary of the spans (tsattn_build_span_tiles)
     float *SumWeightLog = nullptr; // device [headCount][MaxLen]
 
   public:
