@@ -242,6 +242,22 @@ def bench_generation(ctx, steps):
     return res
 
 
+def bench_producer(ctx, steps):
+    """RoPE + per-head RMS normalisation + int8 conversion of one projection result of the 1.5B-style prompt
+    (B32 x 2048 rows, 16 heads x 128, f32 in): bytes = 4 in + 1 out per element, the rope row, the scales."""
+    import torch
+    from tscale_amd import capi
+    n, H, d = 32 * 2048, 16, 128
+    x = torch.randn((n, H * d), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1313 + 6))
+    pos = (torch.arange(n, device="cuda", dtype=torch.int32) % 2048).contiguous()
+    rope = ctx.fill_rope_table(d, 2048)
+    ms = gpu_time_ms(lambda: ctx.rope_normalize_rows(x, H, capi.I8, pos=pos, rope=rope), max(5, steps // 5), 2)
+    nbytes = n * H * d * 5 + n * H * 4 + n * 4 + n * d * 4
+    return {"config": "rope_normalize_rows: 65536 rows x 16 heads x 128, f32 -> int8 + f32 scale per (row, head), with RoPE",
+            "ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4),
+            "bytes": nbytes}
+
+
 def cpu_baseline_prefill(wl, n_seq_sample):
     """The oracle (a port of the reference's CPU attention) on the same quantised inputs: the first
     `n_seq_sample` sequences of every layer of the pass, all host threads; plus one sequence of one
@@ -426,6 +442,8 @@ def main():
         del wl
         torch.cuda.empty_cache()
         result["generation_1p5B_style"] = bench_generation(ctx, args.steps)
+        torch.cuda.empty_cache()
+        result["producer"] = bench_producer(ctx, args.steps)
     print(json.dumps(result))
 
 

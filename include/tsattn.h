@@ -40,7 +40,7 @@ enum tsattn_status {
 
 enum tsattn_dtype { TSATTN_I8 = 0, TSATTN_E4M3 = 1 };               /* Q/K/V element type */
 enum tsattn_out_dtype { TSATTN_OUT_F32 = 0, TSATTN_OUT_F16 = 1 };   /* prefill output type */
-enum tsattn_src_dtype { TSATTN_SRC_F32 = 0, TSATTN_SRC_BF16 = 1 };  /* quantiser input type */
+enum tsattn_src_dtype { TSATTN_SRC_F32 = 0, TSATTN_SRC_BF16 = 1, TSATTN_SRC_I32 = 2 };  /* producer input types */
 enum tsattn_q_dtype { TSATTN_Q_8BIT = 0, TSATTN_Q_BF16 = 1 };       /* decode query type */
 
 /* Sizes the handle's one-time scratch is provisioned for (decode split partials). */
@@ -195,6 +195,39 @@ int tsattn_cache_fill(tsattn_handle_t h, const tsattn_fill_args *a, void *stream
 int64_t tsattn_span_tiles_count(int64_t n_tokens);
 int tsattn_build_span_tiles(tsattn_handle_t h, int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish,
                             int32_t *tiles, void *stream);
+
+/* Producer of Q, K or V for the calls above from a projection result: optional RoPE at each row's position, then per
+ * head sko = sqrt(mean x^2), scale = sko * vec_scale, values / scale converted to int8 (round to nearest even,
+ * clamped to +-127) or e4m3, and scale * scale_mult written to scale[head * scale_pitch + row].  Replaces
+ * ApplyRope + NormalizeState of the reference's inference path (gpt/train/cpu_infer.cpp:486-499, :358-391,
+ * gpt/att/rope.cpp:28-46; the GPU epilogue TStoreRowTileNormalizeRope, gpt/compute/gpt_rope.cuh:4-66, computes the
+ * same per 128-wide head), in the CPU path's operation order: results are identical to it bit for bit.
+ * scale_mult is how the reference folds QVScale * VEC_SCALE * CalcDotScale(dim) into the cached key scale
+ * (cpu_infer.cpp:502-504). */
+typedef struct tsattn_produce_args {
+    int src_dtype;             /* TSATTN_SRC_F32 or TSATTN_SRC_I32 */
+    int dst_dtype;             /* tsattn_dtype */
+    int64_t n_rows;
+    int n_heads, head_dim;
+    const void *src;           /* [n_rows][n_heads*head_dim], 16-byte aligned */
+    int64_t src_pitch;         /* elements per row, multiple of 4 */
+    const int32_t *pos;        /* device [n_rows]: position of each row in its sequence; NULL = no rotation */
+    const float *rope;         /* device [rope_len][head_dim] table, see tsattn_fill_rope_table; NULL only with pos == NULL */
+    int64_t rope_len;          /* positions are clamped into [0, rope_len) */
+    float rotate_dir;          /* +1 (the forward direction) or -1 */
+    float vec_scale;           /* the reference's VEC_SCALE = 1/24 */
+    float scale_mult;
+    void *dst;                 /* [n_rows][n_heads*head_dim] 8-bit */
+    int64_t dst_pitch;         /* bytes per row, multiple of 16 */
+    float *scale;              /* [n_heads][scale_pitch] or NULL */
+    int64_t scale_pitch;
+} tsattn_produce_args;
+
+int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, void *stream);
+
+/* The table ApplyRope reads: FillRopeBuf, gpt/att/rope.cpp:4-24.  Host function, host memory:
+ * table[t * head_dim + x], t < max_len; copy it to the device once. */
+void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table);
 
 /* Per-(row, head) absmax quantiser: scale = absmax/127 (int8) or absmax/256 (e4m3), values
  * round-to-nearest-even, int8 clamped to [-127,127].  Replaces NormalizeVecsRowTileMax /

@@ -1,6 +1,6 @@
 #!/bin/bash
 # Builds oracle/_ref/libtsref.so from the reference's own sources where they lie under
-# /root/reference (nothing is copied): the mask / layer-schedule / e4m3 code that compiles with
+# /root/reference (nothing is copied): the mask / layer-schedule / RoPE / e4m3 code that compiles with
 # stock g++.  The attention arithmetic itself (gpt_cpu.cpp, cpu_infer.cpp) needs the CUDA SDK
 # headers and is not buildable here.  Output only into oracle/_ref/.
 set -e
@@ -11,7 +11,7 @@ OUT="$HERE/_ref"
 mkdir -p "$OUT/obj"
 CXX="g++ -std=c++17 -O1 -mavx2 -mfma -mf16c -fPIC -w -I$R"
 $CXX -c "$HERE/ref_wrap.cpp" -o "$OUT/obj/ref_wrap.o"
-for f in gpt/att/att.cpp gpt/att/sliding_window.cpp gpt/att/nodes_batch.cpp gpt/model_params/model_dim.cpp lib/config/config.cpp; do
+for f in gpt/att/att.cpp gpt/att/rope.cpp gpt/att/sliding_window.cpp gpt/att/nodes_batch.cpp gpt/model_params/model_dim.cpp lib/config/config.cpp; do
   $CXX -I"$R/$(dirname $f)" -c "$R/$f" -o "$OUT/obj/$(basename $f .cpp).o"
 done
 # util/ has a string.h of its own: keep it off the <...> search path

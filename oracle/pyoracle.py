@@ -149,6 +149,38 @@ def bf16_bits_to_float(b):
 
 
 # ---- masks -----------------------------------------------------------------------------------
+def fill_rope(width, max_len):
+    L = lib()
+    rope = np.empty((max_len, width), dtype=np.float32)
+    L.tso_fill_rope(int(width), ctypes.c_int64(max_len), _p(rope))
+    return rope
+
+
+def apply_rope(rope_row, rotate_dir, vec, head_size):
+    L = lib()
+    v = np.array(vec, dtype=np.float32, copy=True)
+    r = _c_arr(rope_row, np.float32)
+    L.tso_apply_rope(_p(r), ctypes.c_float(rotate_dir), int(v.size), int(head_size), _p(v))
+    return v
+
+
+def rope_normalize_rows(dtype, x, n_heads, pos=None, rope=None, rotate_dir=1.0, vec_scale=1.0 / 24, scale_mult=1.0):
+    """x: [n_rows, H*d] float32 or int32 -> (q uint8 [n_rows, H*d], scale f32 [H, n_rows])."""
+    L = lib()
+    is_i32 = x.dtype == np.int32
+    x = _c_arr(x, np.int32 if is_i32 else np.float32)
+    n_rows, hd = x.shape
+    d = hd // n_heads
+    q = np.empty((n_rows, hd), dtype=np.uint8)
+    scale = np.empty((n_heads, n_rows), dtype=np.float32)
+    ps = None if pos is None else _c_arr(pos, np.int32)
+    rp = None if rope is None else _c_arr(rope, np.float32)
+    L.tso_rope_normalize_rows(int(dtype), _p(x), int(is_i32), ctypes.c_int64(hd), ctypes.c_int64(n_rows), _p(ps), _p(rp),
+                              ctypes.c_float(rotate_dir), int(n_heads), int(d), ctypes.c_float(vec_scale),
+                              ctypes.c_float(scale_mult), _p(q), ctypes.c_int64(hd), _p(scale), ctypes.c_int64(n_rows))
+    return q, scale
+
+
 def make_spans(seq_lens, window, doc_start_flag=None):
     L = lib()
     off = np.zeros(len(seq_lens) + 1, dtype=np.int64)

@@ -9,6 +9,7 @@
 #include <gpt/att/att.h>
 #include <gpt/data/data.h>
 #include <gpt/model_params/model_dim.h>
+#include <gpt/att/rope.h>
 
 extern "C" {
 
@@ -103,4 +104,31 @@ float ref_e4m3_to_float(int code) { return ConvertE4toFloat((i8)code); }
 float ref_att_dot_scale(int dim) { return CalcDotScale(dim) * CalcAttentionMult(); }
 float ref_attention_decay(int dist, float slope) { return GetAttentionDecay(dist, slope); }
 
+
+// FillRopeBuf (gpt/att/rope.cpp:4-24): rope[t][x], row-major [max_len][width]
+void ref_fill_rope(int width, long long max_len, float *rope)
+{
+    TArray2D<float> buf;
+    FillRopeBuf(&buf, width, max_len);
+    for (long long t = 0; t < max_len; ++t) {
+        for (int x = 0; x < width; ++x) {
+            rope[t * width + x] = buf[t][x];
+        }
+    }
+}
+
+// ApplyRope (gpt/att/rope.cpp:48-53) on one vector of `dim` floats at position t
+void ref_apply_rope(int width, long long max_len, float rotate_dir, long long t, int dim, float *vec)
+{
+    TArray2D<float> buf;
+    FillRopeBuf(&buf, width, max_len);
+    TVector<float> v;
+    for (int i = 0; i < dim; ++i) {
+        v.push_back(vec[i]);
+    }
+    ApplyRope(buf, rotate_dir, t, &v);
+    for (int i = 0; i < dim; ++i) {
+        vec[i] = v[i];
+    }
+}
 }

@@ -31,6 +31,14 @@
  *                                                         inputs; scale-shift invariance
  *   tso_decode             train/cpu_infer.cpp:413-460   pinned: equals prefill row t on cache [0..t]
  *   tso_softmax_buf        train/cpu_infer.cpp:220-281   pinned: against exp2 in double, |rel| < 1e-5
+ *   tso_fill_rope, tso_apply_rope   att/rope.cpp:4-46     pinned: the reference's own FillRopeBuf / ApplyRope built
+ *                                                         into oracle/_ref (bit-identical tables and rotations);
+ *                                                         rotation preserves each pair's norm
+ *   tso_normalize_heads    train/cpu_infer.cpp:358-391 (e4m3 target: compute/gpt_rope.cuh:41-46,61)
+ *                                                         pinned: constant vector -> 24, zero vector, scale
+ *                                                         invariance, numpy restatement with the same
+ *                                                         sequential float sum
+ *   tso_rope_normalize_rows  train/cpu_infer.cpp:486-499  composition of the two above
  *
  * The reference holds no golden vectors or known-answer tests for this path, and the two files
  * that contain it (gpt_cpu.cpp, cpu_infer.cpp) cannot be compiled without the CUDA SDK, so the
@@ -189,6 +197,112 @@ void tso_quantize_rows_bf16(int dtype, const uint16_t *x, int64_t x_pitch, int64
         }
     }
     free(tmp);
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* producer of the attention operands: RoPE, per-head RMS normalisation, 8-bit conversion       */
+
+/* FillRopeBuf, att/rope.cpp:4-24: rope[t][base + k] = cos(t * f), rope[t][base + k + 32] = sin(t * f),
+ * f = theta^-(2 * (base/2 + k) / width), theta = 500000; blocks of 64 columns. */
+void tso_fill_rope(int width, int64_t max_len, float *rope)
+{
+    float theta = 500000;
+    float *freq = (float *)malloc(sizeof(float) * (size_t)(width / 2 + 1));
+    for (int k = 0; k < width / 2; ++k) {
+        /* C++ overload resolution in the reference: log(float) is the float function, its product with the
+         * double (k * 2. / width) and exp of it are double; cos(float) and sin(float) below are float */
+        freq[k] = (float)exp((double)(-logf(theta)) * (k * 2. / width));
+    }
+    for (int64_t t = 0; t < max_len; ++t) {
+        for (int base = 0; base < width; base += 2 * 32) {
+            for (int k = 0; k < 32; ++k) {
+                float angle = t * freq[base / 2 + k];
+                rope[t * width + base + k] = cosf(angle);
+                rope[t * width + base + k + 32] = sinf(angle);
+            }
+        }
+    }
+    free(freq);
+}
+
+/* ReferenceApplyRope, att/rope.cpp:28-46, on one vector of dim/head_size heads; rope_row = ropeBuf[t]. */
+void tso_apply_rope(const float *rope_row, float rotate_dir, int dim, int head_size, float *vec)
+{
+    for (int offset = 0; offset < dim; offset += head_size) {
+        for (int blk = 0; blk < head_size; blk += 64) {
+            for (int k = 0; k < 32; ++k) {
+                float v0 = vec[offset + blk + k];
+                float v1 = vec[offset + blk + k + 32];
+                float cos_value = rope_row[blk + k];
+                float sin_value = rope_row[blk + k + 32] * rotate_dir;
+                float r0 = v0 * cos_value - v1 * sin_value;
+                float r1 = v0 * sin_value + v1 * cos_value;
+                vec[offset + blk + k] = r0;
+                vec[offset + blk + k + 32] = r1;
+            }
+        }
+    }
+}
+
+/* NormalizeState, train/cpu_infer.cpp:358-391: per head sko = sqrt(sum x^2 / headDim) (float, summed in index
+ * order), discrScale = sko * vec_scale, values multiplied by 1/discrScale and converted (int8: cpu_infer.cpp:88-92;
+ * e4m3: the conversion of the GPU epilogue, gpt_rope.cuh:41-46,61).  A zero head gives zeros and scale 0. */
+void tso_normalize_heads(int dtype, const float *state, int dim, int n_heads, float vec_scale, uint8_t *res,
+                         float *head_scale)
+{
+    int head_dim = dim / n_heads;
+    for (int h = 0; h < n_heads; ++h) {
+        int offset = h * head_dim;
+        float sum2 = 0;
+        for (int x = 0; x < head_dim; ++x) {
+            sum2 += state[offset + x] * state[offset + x];
+        }
+        if (sum2 == 0) {
+            for (int x = 0; x < head_dim; ++x) {
+                res[offset + x] = 0;
+            }
+            if (head_scale) head_scale[h] = 0;
+        } else {
+            float sko = sqrtf(sum2 / head_dim);
+            float discr_scale = sko * vec_scale;
+            float mult = 1 / discr_scale;
+            for (int x = 0; x < head_dim; ++x) {
+                float y = state[offset + x] * mult;
+                res[offset + x] = (dtype == TSO_I8) ? (uint8_t)tso_float_to_i8(y) : tso_float_to_e4m3(y);
+            }
+            if (head_scale) head_scale[h] = discr_scale;
+        }
+    }
+}
+
+/* AddLookupProduct's operand preparation, train/cpu_infer.cpp:486-499: ApplyRope(ropeBuf, dir, t, &src) then
+ * NormalizeState(&dst, src, headCount, &headScale), per row; the written scale is headScale * scale_mult
+ * (cpu_infer.cpp:502-504 folds the matrix scale into the key scale that way).  pos == NULL: no rotation
+ * (the K and V projections, :496-499).  src_is_i32: the projection results that are int32 (:479-482). */
+void tso_rope_normalize_rows(int dtype, const void *src, int src_is_i32, int64_t src_pitch, int64_t n_rows,
+                             const int32_t *pos, const float *rope, float rotate_dir, int n_heads, int head_dim,
+                             float vec_scale, float scale_mult, uint8_t *q, int64_t q_pitch, float *scale,
+                             int64_t scale_pitch)
+{
+    int dim = n_heads * head_dim;
+    float *tmp = (float *)malloc(sizeof(float) * (size_t)dim);
+    float *hs = (float *)malloc(sizeof(float) * (size_t)n_heads);
+    for (int64_t t = 0; t < n_rows; ++t) {
+        for (int i = 0; i < dim; ++i) {
+            tmp[i] = src_is_i32 ? (float)((const int32_t *)src)[t * src_pitch + i] : ((const float *)src)[t * src_pitch + i];
+        }
+        if (pos) {
+            tso_apply_rope(rope + (int64_t)pos[t] * head_dim, rotate_dir, dim, head_dim, tmp);
+        }
+        tso_normalize_heads(dtype, tmp, dim, n_heads, vec_scale, q + t * q_pitch, hs);
+        if (scale) {
+            for (int h = 0; h < n_heads; ++h) {
+                scale[h * scale_pitch + t] = hs[h] * scale_mult;
+            }
+        }
+    }
+    free(tmp);
+    free(hs);
 }
 
 /* ------------------------------------------------------------------------------------------ */

@@ -36,6 +36,14 @@ float   tso_att_dot_scale(int head_dim);       /* sqrtf(1/d) * (0.5f/0.693147f),
 void tso_quantize_rows(int dtype, const float *x, int64_t x_pitch, int64_t n_rows, int n_heads,
                        int head_dim, uint8_t *q, int64_t q_pitch, float *scale, int64_t scale_pitch);
 /* same for bf16 source rows (decode query prologue) */
+void tso_fill_rope(int width, int64_t max_len, float *rope);
+void tso_apply_rope(const float *rope_row, float rotate_dir, int dim, int head_size, float *vec);
+void tso_normalize_heads(int dtype, const float *state, int dim, int n_heads, float vec_scale, uint8_t *res,
+                         float *head_scale);
+void tso_rope_normalize_rows(int dtype, const void *src, int src_is_i32, int64_t src_pitch, int64_t n_rows,
+                             const int32_t *pos, const float *rope, float rotate_dir, int n_heads, int head_dim,
+                             float vec_scale, float scale_mult, uint8_t *q, int64_t q_pitch, float *scale,
+                             int64_t scale_pitch);
 void tso_quantize_rows_bf16(int dtype, const uint16_t *x, int64_t x_pitch, int64_t n_rows,
                             int n_heads, int head_dim, uint8_t *q, int64_t q_pitch, float *scale,
                             int64_t scale_pitch);

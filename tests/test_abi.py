@@ -18,6 +18,7 @@ STRUCTS = {
     "tsattn_decode_args": capi.DecodeArgs,
     "tsattn_append_args": capi.AppendArgs,
     "tsattn_fill_args": capi.FillArgs,
+    "tsattn_produce_args": capi.ProduceArgs,
 }
 
 

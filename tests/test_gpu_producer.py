@@ -1,0 +1,85 @@
+"""GPU: the producer kernel (RoPE + per-head RMS normalisation + 8-bit conversion, tsattn_rope_normalize_rows)
+through the C ABI against its oracle (gpt/att/rope.cpp:28-46, gpt/train/cpu_infer.cpp:358-391,486-499).
+The kernel keeps the CPU path's operation order, so bytes and scales must be identical, not merely close."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import pyoracle as orc
+from tests.common import assert_within_tolerance
+from tscale_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from tscale_amd import AttentionContext
+    c = AttentionContext(0, max_seqs=64, max_heads=16, max_head_dim=128, max_splits=32)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("dtype", [capi.I8, capi.E4M3])
+@pytest.mark.parametrize("d,H", [(64, 12), (128, 5)])
+@pytest.mark.parametrize("with_rope", [True, False])
+def test_producer_bit_exact(ctx, dtype, d, H, with_rope):
+    n = 333                                     # (row, head) pairs not a multiple of the kernel's 64
+    rng = np.random.default_rng(d + H)
+    x = (rng.standard_normal((n, H * d)) * rng.uniform(0.05, 20, (n, 1))).astype(np.float32)
+    x[7] = 0                                    # a zero row: zeros and scale 0
+    x[9, d:2 * d] = 0                           # a zero head
+    pos = rng.integers(0, 900, n).astype(np.int32) if with_rope else None
+    rope_dev = ctx.fill_rope_table(d, 900)
+    rope = orc.fill_rope(d, 900)
+    assert np.array_equal(rope_dev.cpu().numpy(), rope)
+    want_q, want_s = orc.rope_normalize_rows(dtype, x, H, pos=pos, rope=rope if with_rope else None, scale_mult=0.4)
+    q, s = ctx.rope_normalize_rows(torch.from_numpy(x).cuda(), H, dtype,
+                                   pos=None if pos is None else torch.from_numpy(pos).cuda(),
+                                   rope=rope_dev if with_rope else None, scale_mult=0.4)
+    torch.cuda.synchronize()
+    assert np.array_equal(s.cpu().numpy(), want_s)
+    assert np.array_equal(q.cpu().numpy(), want_q)
+    assert not q.cpu().numpy()[7].any() and s.cpu().numpy()[1, 9] == 0
+
+
+def test_producer_int32_source_reverse_direction_and_clamped_positions(ctx):
+    H, d, n = 4, 128, 70
+    rng = np.random.default_rng(1)
+    xi = rng.integers(-30000, 30000, (n, H * d)).astype(np.int32)
+    rope = orc.fill_rope(d, 50)
+    pos = rng.integers(-5, 80, n).astype(np.int32)              # out of range on both sides: clamped
+    want_q, want_s = orc.rope_normalize_rows(orc.I8, xi, H, pos=np.clip(pos, 0, 49), rope=rope, rotate_dir=-1.0)
+    q, s = ctx.rope_normalize_rows(torch.from_numpy(xi).cuda(), H, capi.I8, pos=torch.from_numpy(pos).cuda(),
+                                   rope=torch.from_numpy(rope).cuda(), rotate_dir=-1.0)
+    assert np.array_equal(q.cpu().numpy(), want_q) and np.array_equal(s.cpu().numpy(), want_s)
+
+
+def test_producer_feeds_prefill(ctx):
+    """Projection results -> producer -> prefill, all on the GPU, against the oracle's producer -> oracle's prefill:
+    the reference's order of operations in AddLookupProduct (cpu_infer.cpp:479-509) for a whole sequence."""
+    H, d = 4, 128
+    seq_lens = [200, 120]
+    n = sum(seq_lens)
+    rng = np.random.default_rng(2)
+    src = [rng.standard_normal((n, H * d)).astype(np.float32) * 3 for _ in range(3)]
+    pos = np.concatenate([np.arange(L) for L in seq_lens]).astype(np.int32)
+    rope = orc.fill_rope(d, 256)
+    key_mult = 0.8 / 24 * np.float32(1.0 / np.sqrt(H * d))     # QVScale * VEC_SCALE * CalcDotScale(dim)
+    oq, _ = orc.rope_normalize_rows(orc.I8, src[0], H, pos=pos, rope=rope)
+    ok, oks = orc.rope_normalize_rows(orc.I8, src[1], H, pos=pos, rope=rope, scale_mult=key_mult)
+    ov, _ = orc.rope_normalize_rows(orc.I8, src[2], H)
+    st, fi = orc.make_spans(seq_lens, 10 ** 6)
+    VEC = 1.0 / 24
+    want = orc.prefill_q8(orc.I8, oq, ok, ov, H, VEC, oks, VEC, st, fi, 0.0)
+
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    rope_dev = ctx.fill_rope_table(d, 256)
+    gq, _ = ctx.rope_normalize_rows(dev(src[0]), H, capi.I8, pos=dev(pos), rope=rope_dev)
+    gk, gks = ctx.rope_normalize_rows(dev(src[1]), H, capi.I8, pos=dev(pos), rope=rope_dev, scale_mult=key_mult)
+    gv, _ = ctx.rope_normalize_rows(dev(src[2]), H, capi.I8)
+    assert np.array_equal(gk.cpu().numpy(), ok) and np.array_equal(gks.cpu().numpy(), oks)
+    off = dev(np.concatenate([[0], np.cumsum(seq_lens)]).astype(np.int32))
+    gst, gfi = ctx.build_spans(off, n, 10 ** 6)
+    out = ctx.compute_val_lookup(capi.I8, H, gq, gk, gv, VEC, gks, VEC, gst, gfi, 0.0).cpu().numpy()
+    assert_within_tolerance(out, want, "producer -> prefill")

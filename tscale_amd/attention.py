@@ -84,6 +84,33 @@ class AttentionContext:
                                                  _stream_ptr()))
         return q, scale
 
+    def fill_rope_table(self, head_dim, max_len):
+        """The table of FillRopeBuf (gpt/att/rope.cpp:4-24), computed on the host by the library, on the device."""
+        host = torch.empty((max_len, head_dim), dtype=torch.float32)
+        self.lib.tsattn_fill_rope_table(head_dim, max_len, ctypes.c_void_p(host.data_ptr()))
+        return host.to(self.device)
+
+    def rope_normalize_rows(self, x, n_heads, dtype, pos=None, rope=None, rotate_dir=1.0, vec_scale=1.0 / 24,
+                            scale_mult=1.0):
+        """ApplyRope + NormalizeState of the reference's inference path (cpu_infer.cpp:486-499): x [n_rows, H*d]
+        float32 or int32 -> (uint8 [n_rows, H*d], f32 scale [H, n_rows]); pos int32 [n_rows] or None (no rotation)."""
+        assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.dtype in (torch.float32, torch.int32)
+        n_rows, hd = x.shape
+        q = torch.empty((n_rows, hd), dtype=torch.uint8, device=x.device)
+        scale = torch.empty((n_heads, n_rows), dtype=torch.float32, device=x.device)
+        a = capi.ProduceArgs()
+        a.src_dtype = capi.SRC_F32 if x.dtype == torch.float32 else capi.SRC_I32
+        a.dst_dtype = dtype
+        a.n_rows, a.n_heads, a.head_dim = n_rows, n_heads, hd // n_heads
+        a.src, a.src_pitch = _ptr(x), hd
+        a.pos, a.rope = _ptr(pos), _ptr(rope)
+        a.rope_len = 0 if rope is None else rope.shape[0]
+        a.rotate_dir, a.vec_scale, a.scale_mult = float(rotate_dir), float(vec_scale), float(scale_mult)
+        a.dst, a.dst_pitch = _ptr(q), hd
+        a.scale, a.scale_pitch = _ptr(scale), n_rows
+        capi.check(self.lib.tsattn_rope_normalize_rows(self.handle, ctypes.byref(a), _stream_ptr()))
+        return q, scale
+
     def build_spans(self, seq_offset, n_tokens, window, doc_start_flag=None):
         """seq_offset: int32 [n_seqs+1] on the device.  Returns (span_start, span_finish) int32 [n_tokens]."""
         st = torch.empty(n_tokens, dtype=torch.int32, device=self.device)

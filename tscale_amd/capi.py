@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libtsattn.so")
 
 I8, E4M3 = 0, 1
 OUT_F32, OUT_F16 = 0, 1
-SRC_F32, SRC_BF16 = 0, 1
+SRC_F32, SRC_BF16, SRC_I32 = 0, 1, 2
 Q_8BIT, Q_BF16 = 0, 1
 SPAN_TILE_INTS = 32
 
@@ -69,6 +69,16 @@ class AppendArgs(_c.Structure):
     ]
 
 
+class ProduceArgs(_c.Structure):
+    _fields_ = [
+        ("src_dtype", _c.c_int), ("dst_dtype", _c.c_int), ("n_rows", _c.c_int64), ("n_heads", _c.c_int),
+        ("head_dim", _c.c_int), ("src", _c.c_void_p), ("src_pitch", _c.c_int64), ("pos", _c.c_void_p),
+        ("rope", _c.c_void_p), ("rope_len", _c.c_int64), ("rotate_dir", _c.c_float), ("vec_scale", _c.c_float),
+        ("scale_mult", _c.c_float), ("dst", _c.c_void_p), ("dst_pitch", _c.c_int64), ("scale", _c.c_void_p),
+        ("scale_pitch", _c.c_int64),
+    ]
+
+
 class FillArgs(_c.Structure):
     _fields_ = [
         ("n_seqs", _c.c_int), ("n_heads", _c.c_int), ("head_dim", _c.c_int), ("n_tokens", _c.c_int64),
@@ -82,7 +92,7 @@ class FillArgs(_c.Structure):
 
 
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
+           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
 
 _lib = None
 
@@ -116,6 +126,10 @@ def load():
         L.tsattn_span_tiles_count.argtypes = [_c.c_int64]
         L.tsattn_build_span_tiles.restype = _c.c_int
         L.tsattn_build_span_tiles.argtypes = [_c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p]
+        L.tsattn_rope_normalize_rows.restype = _c.c_int
+        L.tsattn_rope_normalize_rows.argtypes = [_c.c_void_p, _c.POINTER(ProduceArgs), _c.c_void_p]
+        L.tsattn_fill_rope_table.restype = None
+        L.tsattn_fill_rope_table.argtypes = [_c.c_int, _c.c_int64, _c.c_void_p]
         L.tsattn_quantize_rows.restype = _c.c_int
         L.tsattn_quantize_rows.argtypes = [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64,
                                            _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64,

@@ -257,6 +257,37 @@ int tsattn_cache_fill(tsattn_handle_t h, const tsattn_fill_args *a, void *stream
     return TSATTN_OK;
 }
 
+int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: null argument");
+    if (!dtype_ok(a->dst_dtype) || (a->src_dtype != TSATTN_SRC_F32 && a->src_dtype != TSATTN_SRC_I32))
+        return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_rope_normalize_rows: dtypes %d -> %d", a->src_dtype, a->dst_dtype);
+    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_rope_normalize_rows: head_dim %d (64 or 128 supported)", a->head_dim);
+    if (a->n_rows < 0 || a->n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: negative size");
+    if (a->n_rows == 0) return TSATTN_OK;
+    if (!a->src || !a->dst) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: null data pointer");
+    if (a->pos && (!a->rope || a->rope_len <= 0)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: positions given without a rope table");
+    const int64_t row = (int64_t)a->n_heads * a->head_dim;
+    if (a->src_pitch < row || a->dst_pitch < row || a->dst_pitch % 16 || a->src_pitch % 4 || !aligned16(a->dst) || !aligned16(a->src) ||
+        (a->rope && !aligned16(a->rope)))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: pitches must cover a row; src, dst and rope 16-byte aligned, pitches multiples of 16 bytes");
+    if (a->scale && a->scale_pitch < a->n_rows) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale_pitch below n_rows");
+    tsattn::ProduceParams p;
+    p.src = a->src; p.src_pitch = a->src_pitch; p.n_rows = a->n_rows; p.n_heads = a->n_heads;
+    p.pos = a->pos; p.rope = a->rope; p.rope_len = a->rope_len;
+    p.rotate_dir = a->rotate_dir; p.vec_scale = a->vec_scale; p.scale_mult = a->scale_mult;
+    p.dst = (uint8_t *)a->dst; p.dst_pitch = a->dst_pitch; p.scale = a->scale; p.scale_pitch = a->scale_pitch;
+    hipError_t e = tsattn::launch_rope_normalize(p, a->dst_dtype, a->head_dim, a->src_dtype == TSATTN_SRC_I32, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "rope normalize launch");
+    return TSATTN_OK;
+}
+
+void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table)
+{
+    if (!table || head_dim <= 0 || head_dim % 64 || max_len <= 0) return;
+    tsattn::fill_rope_table(head_dim, max_len, table);
+}
+
 int tsattn_quantize_rows(tsattn_handle_t h, int src_dtype, int dst_dtype, const void *src, int64_t src_pitch, int64_t n_rows,
                          int n_heads, int head_dim, void *dst, int64_t dst_pitch, float *scale, int64_t scale_pitch, void *stream)
 {

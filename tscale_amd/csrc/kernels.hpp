@@ -82,6 +82,24 @@ struct AppendParams {
 
 hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st);
 
+struct ProduceParams {
+    const void *src;
+    int64_t src_pitch; // elements per row
+    int64_t n_rows;
+    int n_heads;
+    const int32_t *pos;
+    const float *rope;
+    int64_t rope_len;
+    float rotate_dir, vec_scale, scale_mult;
+    uint8_t *dst;
+    int64_t dst_pitch;
+    float *scale;
+    int64_t scale_pitch;
+};
+
+hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head_dim, bool src_i32, hipStream_t st);
+void fill_rope_table(int width, int64_t max_len, float *table);
+
 struct FillParams {
     const int32_t *seq_offset;
     const uint8_t *k_src, *v_src;

@@ -1,0 +1,158 @@
+// Producer of the attention operands: RoPE, per-head RMS normalisation and 8-bit conversion of a projection
+// result, with the per-(row, head) scale the attention kernels consume.  Follows the reference's CPU inference
+// (ApplyRope + NormalizeState, gpt/train/cpu_infer.cpp:486-499, :358-391; gpt/att/rope.cpp:28-46) operation by
+// operation: the same float products, the sum of squares taken in index order, no fused multiply-adds, so the
+// bytes and scales are identical to a CPU evaluation in that order.
+//
+// A workgroup takes 64 consecutive (row, head) pairs.  The rotated values go to LDS (row pitch d+1 floats, so
+// that 64 lanes walking 64 different pairs in step hit 64 different banks); then lane j of the first wave sums
+// pair j's squares one after the other, which keeps the summation order while 64 sums advance together; then
+// all threads convert and write the bytes out, four per thread, consecutively.
+#include <math.h>
+
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace tsattn {
+
+constexpr int PR_PAIRS = 64;
+
+// every float operation below is meant as written: no fused multiply-adds
+#pragma clang fp contract(off)
+
+template <int D, int DST, bool SRC_I32>
+__global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
+{
+    constexpr int PITCH = D + 1;
+    __shared__ float vals[PR_PAIRS * PITCH];
+    __shared__ float mults[PR_PAIRS];
+    __shared__ int64_t s_row[PR_PAIRS];
+    __shared__ int s_head[PR_PAIRS], s_pos[PR_PAIRS];
+    const int tid = threadIdx.x;
+    const int64_t pair0 = (int64_t)blockIdx.x * PR_PAIRS;
+    const int64_t n_pairs = p.n_rows * p.n_heads;
+    const int n_here = (int)(n_pairs - pair0 < PR_PAIRS ? n_pairs - pair0 : PR_PAIRS);
+
+    if (tid < n_here) {
+        const int64_t pair = pair0 + tid;
+        const int64_t row = pair / p.n_heads;
+        s_row[tid] = row;
+        s_head[tid] = (int)(pair - row * p.n_heads);
+        int t = p.pos ? p.pos[row] : 0;
+        s_pos[tid] = t < 0 ? 0 : (t >= p.rope_len ? (int)p.rope_len - 1 : t);
+    }
+    __syncthreads();
+
+    // ---- load + rotate: four (k, k+32) couples per thread and step, 16-byte loads ----------------------------
+    constexpr int PER_PAIR = D / 8;
+    for (int j = tid; j < n_here * PER_PAIR; j += 256) {
+        const int pr = j / PER_PAIR, c = j % PER_PAIR;
+        const int x0 = (c / 8) * 64 + (c % 8) * 4, x1 = x0 + 32;
+        const int64_t e = s_row[pr] * p.src_pitch + (int64_t)s_head[pr] * D;
+        v4f v0, v1;
+        if (SRC_I32) {
+            const v4i a = *(const v4i *)((const int32_t *)p.src + e + x0), b = *(const v4i *)((const int32_t *)p.src + e + x1);
+            v0 = v4f{(float)a.x, (float)a.y, (float)a.z, (float)a.w};
+            v1 = v4f{(float)b.x, (float)b.y, (float)b.z, (float)b.w};
+        } else {
+            v0 = *(const v4f *)((const float *)p.src + e + x0);
+            v1 = *(const v4f *)((const float *)p.src + e + x1);
+        }
+        if (p.pos) {
+            const float *rr = p.rope + (int64_t)s_pos[pr] * D;
+            const v4f cs = *(const v4f *)(rr + x0), sn = *(const v4f *)(rr + x1);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float cos_value = cs[i];
+                const float sin_value = sn[i] * p.rotate_dir;
+                const float r0 = v0[i] * cos_value - v1[i] * sin_value;
+                const float r1 = v0[i] * sin_value + v1[i] * cos_value;
+                v0[i] = r0;
+                v1[i] = r1;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            vals[pr * PITCH + x0 + i] = v0[i];
+            vals[pr * PITCH + x1 + i] = v1[i];
+        }
+    }
+    __syncthreads();
+
+    // ---- per pair: sum of squares in index order, scale -----------------------------------------------------
+    if (tid < n_here) {
+        const float *v = vals + tid * PITCH;
+        float sum2 = 0.0f;
+#pragma unroll 8
+        for (int x = 0; x < D; ++x) sum2 = sum2 + v[x] * v[x];
+        float discr = 0.0f, mult = 0.0f;
+        if (sum2 != 0.0f) {
+            // the single-precision square root instruction is one ulp off now and then; the double-precision routine
+            // is exact to well below a float ulp, and rounding its result to float gives the correctly rounded root
+            const float sko = (float)sqrt((double)(sum2 / (float)D));
+            discr = sko * p.vec_scale;
+            mult = 1.0f / discr;
+        }
+        mults[tid] = mult;
+        if (p.scale) p.scale[s_head[tid] * p.scale_pitch + s_row[tid]] = discr * p.scale_mult;
+    }
+    __syncthreads();
+
+    // ---- convert and store, 16 bytes per thread and step ------------------------------------------------------
+    constexpr int OUT_PER_PAIR = D / 16;
+    for (int j = tid; j < n_here * OUT_PER_PAIR; j += 256) {
+        const int pr = j / OUT_PER_PAIR, x = (j % OUT_PER_PAIR) * 16;
+        const float mult = mults[pr];
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            w[k] = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float y = vals[pr * PITCH + x + 4 * k + i] * mult;
+                // a head of zeros is written as zero bytes whatever the signs of its (rotated) zeros
+                const uint32_t b = mult == 0.0f ? 0u : ((DST == TSATTN_I8) ? (uint8_t)float_to_i8(y) : float_to_e4m3(y));
+                w[k] |= b << (8 * i);
+            }
+        }
+        *(v4i *)(p.dst + s_row[pr] * p.dst_pitch + (int64_t)s_head[pr] * D + x) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    }
+}
+
+hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head_dim, bool src_i32, hipStream_t st)
+{
+    const int64_t n_pairs = p.n_rows * p.n_heads;
+    if (n_pairs == 0) return hipSuccess;
+    dim3 grid((unsigned)((n_pairs + PR_PAIRS - 1) / PR_PAIRS)), block(256);
+#define TSATTN_PR(D_, DST_, I32_) hipLaunchKernelGGL((rope_normalize_kernel<D_, DST_, I32_>), grid, block, 0, st, p)
+    if (head_dim == 128 && dst_dtype == TSATTN_I8 && !src_i32) TSATTN_PR(128, TSATTN_I8, false);
+    else if (head_dim == 128 && dst_dtype == TSATTN_I8 && src_i32) TSATTN_PR(128, TSATTN_I8, true);
+    else if (head_dim == 128 && dst_dtype == TSATTN_E4M3 && !src_i32) TSATTN_PR(128, TSATTN_E4M3, false);
+    else if (head_dim == 128 && dst_dtype == TSATTN_E4M3 && src_i32) TSATTN_PR(128, TSATTN_E4M3, true);
+    else if (head_dim == 64 && dst_dtype == TSATTN_I8 && !src_i32) TSATTN_PR(64, TSATTN_I8, false);
+    else if (head_dim == 64 && dst_dtype == TSATTN_I8 && src_i32) TSATTN_PR(64, TSATTN_I8, true);
+    else if (head_dim == 64 && dst_dtype == TSATTN_E4M3 && !src_i32) TSATTN_PR(64, TSATTN_E4M3, false);
+    else if (head_dim == 64 && dst_dtype == TSATTN_E4M3 && src_i32) TSATTN_PR(64, TSATTN_E4M3, true);
+    else return hipErrorInvalidValue;
+#undef TSATTN_PR
+    return hipGetLastError();
+}
+
+// FillRopeBuf, gpt/att/rope.cpp:4-24 (host): table[t][base + k] = cos(t f), table[t][base + k + 32] = sin(t f),
+// f = theta^-(2 (base/2 + k) / width), theta = 500000.  The float/double mix follows the reference's C++ overloads.
+void fill_rope_table(int width, int64_t max_len, float *table)
+{
+    const float theta = 500000;
+    for (int64_t t = 0; t < max_len; ++t) {
+        for (int base = 0; base < width; base += 64) {
+            for (int k = 0; k < 32; ++k) {
+                const float freq = (float)exp((double)(-logf(theta)) * ((base / 2 + k) * 2. / width));
+                const float angle = t * freq;
+                table[t * width + base + k] = cosf(angle);
+                table[t * width + base + k + 32] = sinf(angle);
+            }
+        }
+    }
+}
+
+} // namespace tsattn
