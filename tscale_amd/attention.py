@@ -164,8 +164,9 @@ class AttentionContext:
 
     # ---- decode ---------------------------------------------------------------------------------
     def compute_val_lookup_decode(self, cache, q, q_scale, window, alibi_slope, out=None, n_splits=0,
-                                  debug_qk_acc=None, max_len=None):
-        """q: uint8 [B, H*d] with q_scale f32 [B, H] (or a number), or bfloat16 [B, H*d] (quantised in the kernel)."""
+                                  debug_qk_acc=None, max_len=None, append=None):
+        """q: uint8 [B, H*d] with q_scale f32 [B, H] (or a number), or bfloat16 [B, H*d] (quantised in the kernel).
+        append = (k_new, k_scale_new, v_new, v_scale_new): KVCache.add_vectors fused into the same launches."""
         B, H, d = cache.n_seqs, cache.n_heads, cache.head_dim
         if out is None:
             out = torch.empty((B, H * d), dtype=torch.float32, device=q.device)
@@ -189,6 +190,10 @@ class AttentionContext:
         a.n_splits = int(n_splits)
         if debug_qk_acc is not None:
             a.debug_qk_acc, a.debug_pitch = _ptr(debug_qk_acc), debug_qk_acc.stride(1)
+        if append is not None:
+            k_new, ks_new, v_new, vs_new = append
+            a.k_new, a.v_new, a.new_pitch = _ptr(k_new), _ptr(v_new), k_new.stride(0)
+            a.k_scale_new, a.v_scale_new = _ptr(ks_new), _ptr(vs_new)
         capi.check(self.lib.tsattn_decode(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
 

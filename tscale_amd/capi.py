@@ -54,7 +54,8 @@ class DecodeArgs(_c.Structure):
         ("s_head_stride", _c.c_int64), ("k_scale_const", _c.c_float), ("v_scale_const", _c.c_float),
         ("cache_len", _c.c_void_p), ("max_len", _c.c_int), ("window", _c.c_int64),
         ("alibi_slope", _c.c_float), ("out", _c.c_void_p), ("n_splits", _c.c_int),
-        ("debug_qk_acc", _c.c_void_p), ("debug_pitch", _c.c_int64),
+        ("debug_qk_acc", _c.c_void_p), ("debug_pitch", _c.c_int64), ("k_new", _c.c_void_p), ("v_new", _c.c_void_p),
+        ("new_pitch", _c.c_int64), ("k_scale_new", _c.c_void_p), ("v_scale_new", _c.c_void_p),
     ]
 
 

@@ -182,6 +182,17 @@ int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
     p.n_heads = a->n_heads; p.n_splits = splits;
     p.part_acc = h->part_acc; p.part_ml = h->part_ml;
     p.dbg = a->debug_qk_acc; p.dbg_pitch = a->debug_pitch;
+    p.out = a->out;
+    p.k_new = (const uint8_t *)a->k_new; p.v_new = (const uint8_t *)a->v_new; p.new_pitch = a->new_pitch;
+    p.ks_new = a->k_scale_new; p.vs_new = a->v_scale_new;
+    p.cache_len_rw = const_cast<int32_t *>(a->cache_len); p.max_len = a->max_len;
+    if (a->k_new || a->v_new) {
+        if (!a->k_new || !a->v_new) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: fused append needs both k_new and v_new");
+        if (a->window == 0) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: fused append is not available with window 0; call tsattn_cache_append first");
+        if (a->new_pitch % 16 || a->new_pitch < (int64_t)a->n_heads * a->head_dim || !aligned16(a->k_new) || !aligned16(a->v_new))
+            return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: k_new/v_new must be 16-byte aligned with a pitch that covers a row");
+        if ((a->k_scale_new && !a->k_scale) || (a->v_scale_new && !a->v_scale)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: new scales given without scale planes");
+    }
     hipError_t e = tsattn::launch_decode(p, a->dtype, a->head_dim, a->q_dtype == TSATTN_Q_BF16, a->n_seqs, a->out, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "decode launch");
     return TSATTN_OK;

@@ -142,7 +142,25 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
     __shared__ float sm_acc[DEC_WAVES][D];
 
     // ---- key range of this block --------------------------------------------------------------
-    const int cur = p.cache_len[seq] - 1;
+    // With a fused append the cache holds cache_len rows and the new token's row is being added as row cache_len
+    // by the first split's workgroup of each head (a full cache drops it, as the separate append does).
+    int cur = p.cache_len[seq] - 1;
+    if (p.k_new && cur + 1 < p.max_len) {
+        cur += 1;
+        if (split == 0 && tid < 2 * LPK) {
+            const int pl = tid / LPK, ch = tid % LPK; // plane (K or V), 16-byte chunk
+            const int64_t src = (int64_t)seq * p.new_pitch + head * D + ch * 16;
+            const int64_t dst = (int64_t)seq * p.seq_stride + (int64_t)head * p.head_stride + (int64_t)cur * p.tok_stride + ch * 16;
+            if (pl == 0) *(v4i *)(const_cast<uint8_t *>(p.k) + dst) = *(const v4i *)(p.k_new + src);
+            else *(v4i *)(const_cast<uint8_t *>(p.v) + dst) = *(const v4i *)(p.v_new + src);
+            if (ch == 0) {
+                const int64_t sd = (int64_t)seq * p.s_seq_stride + (int64_t)head * p.s_head_stride + cur;
+                if (pl == 0 && p.ks_new) const_cast<float *>(p.ks)[sd] = p.ks_new[seq * p.n_heads + head];
+                if (pl == 1 && p.vs_new) const_cast<float *>(p.vs)[sd] = p.vs_new[seq * p.n_heads + head];
+            }
+        }
+    }
+    const bool direct = p.n_splits == 1 && !p.k_new; // no merge kernel follows: this workgroup writes the output
     int lo, n;
     if (cur < 0) {
         lo = 0; n = 0;
@@ -160,6 +178,10 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
 
     const int64_t part = ((int64_t)seq * p.n_heads + head) * p.n_splits + split;
     if (s0 >= s1) { // nothing to do: neutral partial (max 0, sum 0, zeros)
+        if (direct) {
+            if (tid < D) p.out[((int64_t)seq * p.n_heads + head) * D + tid] = 0.0f;
+            return;
+        }
         if (tid < D) p.part_acc[part * D + tid] = 0.0f;
         if (tid == 0) { p.part_ml[part * 2] = 0.0f; p.part_ml[part * 2 + 1] = 0.0f; }
         return;
@@ -287,17 +309,29 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
             o += sm_acc[w][tid] * f;
             L += sm_l[w] * f;
         }
-        p.part_acc[part * D + tid] = o;
-        if (tid == 0) { p.part_ml[part * 2] = M; p.part_ml[part * 2 + 1] = L; }
+        if (direct) {
+            // the only split: add the zero vector's weight 2^-M (M >= 0 by construction) and normalise here
+            p.out[((int64_t)seq * p.n_heads + head) * D + tid] = o / (L + fast_exp2(-M));
+        } else {
+            p.part_acc[part * D + tid] = o;
+            if (tid == 0) { p.part_ml[part * 2] = M; p.part_ml[part * 2 + 1] = L; }
+        }
     }
 }
 
 // out = sum_s acc_s 2^(m_s - M) / (2^-M + sum_s l_s 2^(m_s - M)),  M = max(0, max_s m_s)
 template <int D>
-__global__ __launch_bounds__(D) void decode_merge_kernel(const float *part_acc, const float *part_ml, int n_splits, float *out)
+__global__ __launch_bounds__(D) void decode_merge_kernel(const float *part_acc, const float *part_ml, int n_splits, float *out,
+                                                         int32_t *bump_len, int n_heads, int max_len)
 {
     const int64_t sh = blockIdx.x; // seq * n_heads + head
     const int x = threadIdx.x;
+    // after a fused append: every split kernel has finished with the old length, count the new row
+    if (bump_len && x == 0 && sh % n_heads == 0) {
+        const int64_t seq = sh / n_heads;
+        const int len = bump_len[seq];
+        if (len >= 0 && len < max_len) bump_len[seq] = len + 1;
+    }
     float M = 0.0f;
     for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[(sh * n_splits + s) * 2]);
     float L = fast_exp2(-M); // the zero vector of weight 1 (cpu_infer.cpp:444)
@@ -333,9 +367,11 @@ hipError_t launch_decode(const DecodeParams &p, int dtype, int head_dim, bool qb
     else return hipErrorInvalidValue;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
+    if (p.n_splits == 1 && !p.k_new) return hipSuccess; // the split kernel wrote the output itself
     dim3 mgrid((unsigned)(n_seqs * p.n_heads));
-    if (head_dim == 128) hipLaunchKernelGGL((decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p.part_acc, p.part_ml, p.n_splits, out);
-    else hipLaunchKernelGGL((decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p.part_acc, p.part_ml, p.n_splits, out);
+    int32_t *bump = p.k_new ? p.cache_len_rw : nullptr;
+    if (head_dim == 128) hipLaunchKernelGGL((decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p.part_acc, p.part_ml, p.n_splits, out, bump, p.n_heads, p.max_len);
+    else hipLaunchKernelGGL((decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p.part_acc, p.part_ml, p.n_splits, out, bump, p.n_heads, p.max_len);
     return hipGetLastError();
 }
 

@@ -25,6 +25,14 @@ struct DecodeParams {
     float *part_ml;  // [seq][head][split][2] = running max, sum
     void *dbg;
     int64_t dbg_pitch;
+    float *out;           // final output; written by the split kernel itself when there is one split and no append
+    // fused append (all null/0 when not used): the new token's row goes to row cache_len[seq] of the cache, the
+    // token attends as if cache_len were one more, and the merge kernel bumps cache_len afterwards
+    const uint8_t *k_new, *v_new;
+    int64_t new_pitch;
+    const float *ks_new, *vs_new;
+    int32_t *cache_len_rw;
+    int max_len;
 };
 
 hipError_t launch_decode(const DecodeParams &p, int dtype, int head_dim, bool qbf16, int n_seqs, float *out, hipStream_t st);
