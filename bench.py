@@ -333,6 +333,9 @@ def run_only(ctx, args):
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
+    if name == "producer":
+        print(json.dumps({"only": name, **bench_producer(ctx, args.steps * 5)}))
+        return
     if name == "decode":
         dw = DecodeWorkload(ctx, 64, 4096, 16, 128, n_caches=4, seed=1313 + 3)
         ms = gpu_time_ms(dw.step, args.steps, args.warmup)
@@ -361,7 +364,7 @@ def main():
     ap.add_argument("--extra", action="store_true",
                     help="also time the 1.5B-style prefill shapes and the attention share of the 1.5B-style generation run")
     ap.add_argument("--only", default=None,
-                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode"],
+                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer"],
                     help="profiling aid: run just this launch --steps times and print its timing")
     ap.add_argument("--calibrate", action="store_true",
                     help="with --only: first run three 256 MiB device copies (counter calibration)")

@@ -4,9 +4,9 @@
 // operation: the same float products, the sum of squares taken in index order, no fused multiply-adds, so the
 // bytes and scales are identical to a CPU evaluation in that order.
 //
-// A workgroup takes 64 consecutive (row, head) pairs.  The rotated values go to LDS (row pitch d+1 floats, so
-// that 64 lanes walking 64 different pairs in step hit 64 different banks); then lane j of the first wave sums
-// pair j's squares one after the other, which keeps the summation order while 64 sums advance together; then
+// A workgroup takes 32 consecutive (row, head) pairs.  The rotated values go to LDS (row pitch d+1 floats, so
+// that 32 lanes walking 32 different pairs in step hit 32 different banks); then lane j of the first wave sums
+// pair j's squares one after the other, which keeps the summation order while 32 sums advance together; then
 // all threads convert and write the bytes out, four per thread, consecutively.
 #include <math.h>
 
@@ -15,7 +15,7 @@
 
 namespace tsattn {
 
-constexpr int PR_PAIRS = 64;
+constexpr int PR_PAIRS = 32;
 
 // every float operation below is meant as written: no fused multiply-adds
 #pragma clang fp contract(off)
@@ -43,38 +43,53 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
     }
     __syncthreads();
 
-    // ---- load + rotate: four (k, k+32) couples per thread and step, 16-byte loads ----------------------------
+    // ---- load + rotate: four (k, k+32) couples per thread and step, 16-byte loads; all loads of a thread are
+    //      issued before the first is used ------------------------------------------------------------------
     constexpr int PER_PAIR = D / 8;
-    for (int j = tid; j < n_here * PER_PAIR; j += 256) {
+    constexpr int STEPS = PR_PAIRS * PER_PAIR / 256;
+    v4f v0[STEPS], v1[STEPS], cs[STEPS], sn[STEPS];
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+        const int j = tid + st * 256;
         const int pr = j / PER_PAIR, c = j % PER_PAIR;
+        if (pr >= n_here) continue;
         const int x0 = (c / 8) * 64 + (c % 8) * 4, x1 = x0 + 32;
         const int64_t e = s_row[pr] * p.src_pitch + (int64_t)s_head[pr] * D;
-        v4f v0, v1;
         if (SRC_I32) {
             const v4i a = *(const v4i *)((const int32_t *)p.src + e + x0), b = *(const v4i *)((const int32_t *)p.src + e + x1);
-            v0 = v4f{(float)a.x, (float)a.y, (float)a.z, (float)a.w};
-            v1 = v4f{(float)b.x, (float)b.y, (float)b.z, (float)b.w};
+            v0[st] = v4f{(float)a.x, (float)a.y, (float)a.z, (float)a.w};
+            v1[st] = v4f{(float)b.x, (float)b.y, (float)b.z, (float)b.w};
         } else {
-            v0 = *(const v4f *)((const float *)p.src + e + x0);
-            v1 = *(const v4f *)((const float *)p.src + e + x1);
+            v0[st] = *(const v4f *)((const float *)p.src + e + x0);
+            v1[st] = *(const v4f *)((const float *)p.src + e + x1);
         }
         if (p.pos) {
             const float *rr = p.rope + (int64_t)s_pos[pr] * D;
-            const v4f cs = *(const v4f *)(rr + x0), sn = *(const v4f *)(rr + x1);
+            cs[st] = *(const v4f *)(rr + x0);
+            sn[st] = *(const v4f *)(rr + x1);
+        }
+    }
+#pragma unroll
+    for (int st = 0; st < STEPS; ++st) {
+        const int j = tid + st * 256;
+        const int pr = j / PER_PAIR, c = j % PER_PAIR;
+        if (pr >= n_here) continue;
+        const int x0 = (c / 8) * 64 + (c % 8) * 4, x1 = x0 + 32;
+        if (p.pos) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float cos_value = cs[i];
-                const float sin_value = sn[i] * p.rotate_dir;
-                const float r0 = v0[i] * cos_value - v1[i] * sin_value;
-                const float r1 = v0[i] * sin_value + v1[i] * cos_value;
-                v0[i] = r0;
-                v1[i] = r1;
+                const float cos_value = cs[st][i];
+                const float sin_value = sn[st][i] * p.rotate_dir;
+                const float r0 = v0[st][i] * cos_value - v1[st][i] * sin_value;
+                const float r1 = v0[st][i] * sin_value + v1[st][i] * cos_value;
+                v0[st][i] = r0;
+                v1[st][i] = r1;
             }
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            vals[pr * PITCH + x0 + i] = v0[i];
-            vals[pr * PITCH + x1 + i] = v1[i];
+            vals[pr * PITCH + x0 + i] = v0[st][i];
+            vals[pr * PITCH + x1 + i] = v1[st][i];
         }
     }
     __syncthreads();
