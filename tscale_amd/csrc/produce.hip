@@ -7,7 +7,7 @@
 // A workgroup takes 32 consecutive (row, head) pairs.  The rotated values go to LDS (row pitch d+1 floats, so
 // that 32 lanes walking 32 different pairs in step hit 32 different banks); then lane j of the first wave sums
 // pair j's squares one after the other, which keeps the summation order while 32 sums advance together; then
-// all threads convert and write the bytes out, four per thread, consecutively.
+// all threads convert and write the bytes out, sixteen per thread, consecutively.
 #include <math.h>
 
 #include "common.hpp"
