@@ -258,6 +258,19 @@ def bench_producer(ctx, steps):
             "bytes": nbytes}
 
 
+def bench_kv_product(ctx, steps):
+    """KVProduct on the decode output of the 1.5B-style prompt batch: int8 k + f32 attention output -> 4 x int8."""
+    import torch
+    n, H, d = 32 * 2048, 16, 128
+    g = torch.Generator(device="cuda").manual_seed(1313 + 7)
+    k = torch.randint(0, 256, (n, H * d), dtype=torch.uint8, device="cuda", generator=g)
+    val = torch.randn((n, H * d), device="cuda", generator=g) * 0.3
+    ms = gpu_time_ms(lambda: ctx.kv_product(k, val, H), max(5, steps // 5), 2)
+    nbytes = n * H * d * (1 + 4 + 4)
+    return {"config": "kv_product: 65536 rows x 16 heads x 128, int8 k x f32 value -> 4 x int8", "ms": round(ms, 4),
+            "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4), "bytes": nbytes}
+
+
 def cpu_baseline_prefill(wl, n_seq_sample):
     """The oracle (a port of the reference's CPU attention) on the same quantised inputs: the first
     `n_seq_sample` sequences of every layer of the pass, all host threads; plus one sequence of one
@@ -447,6 +460,8 @@ def main():
         result["generation_1p5B_style"] = bench_generation(ctx, args.steps)
         torch.cuda.empty_cache()
         result["producer"] = bench_producer(ctx, args.steps)
+        torch.cuda.empty_cache()
+        result["kv_product"] = bench_kv_product(ctx, args.steps)
     print(json.dumps(result))
 
 

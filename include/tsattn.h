@@ -233,6 +233,16 @@ typedef struct tsattn_produce_args {
 
 int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, void *stream);
 
+/* Consumer of the attention output: kv[row][(head*rep + blk)*head_dim + z] = int8(k[row][head*head_dim + (z ^ blk)] *
+ * value[row][head*head_dim + z] * mult), blk < rep (the reference's COMBINER_REP = 4), int8 = round to nearest even
+ * clamped to +-127.  Replaces KVProduct, gpt/train/cpu_infer.cpp:320-337 (call :511; GPU form
+ * gpt/compute/gpt_combiner.cuh:13-37, whose kvMult is `mult`).  k: int8 [n_rows][n_heads*head_dim]; value: the
+ * attention output, f32 or f16 (tsattn_out_dtype); pitches of k and kv in bytes, of value in elements; all 16-byte
+ * aligned. */
+int tsattn_kv_product(tsattn_handle_t h, int64_t n_rows, int n_heads, int head_dim, int rep, const void *k, int64_t k_pitch,
+                      int value_dtype, const void *value, int64_t value_pitch, float mult, void *kv, int64_t kv_pitch,
+                      void *stream);
+
 /* The table ApplyRope reads: FillRopeBuf, gpt/att/rope.cpp:4-24.  Host function, host memory:
  * table[t * head_dim + x], t < max_len; copy it to the device once. */
 void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table);

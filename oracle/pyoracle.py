@@ -181,6 +181,18 @@ def rope_normalize_rows(dtype, x, n_heads, pos=None, rope=None, rotate_dir=1.0, 
     return q, scale
 
 
+def kv_product(k, val, n_heads, rep=4, mult=1.0):
+    """k: int8 (as uint8 or int8) [n_rows, H*d]; val: float32 [n_rows, H*d] -> int8 [n_rows, H*d*rep]."""
+    L = lib()
+    k = _c_arr(np.asarray(k).view(np.int8), np.int8)
+    val = _c_arr(val, np.float32)
+    n, hd = k.shape
+    kv = np.empty((n, hd * rep), dtype=np.int8)
+    L.tso_kv_product(_p(k), ctypes.c_int64(hd), _p(val), ctypes.c_int64(hd), ctypes.c_int64(n), int(n_heads), int(hd // n_heads),
+                     int(rep), ctypes.c_float(mult), _p(kv), ctypes.c_int64(hd * rep))
+    return kv
+
+
 def make_spans(seq_lens, window, doc_start_flag=None):
     L = lib()
     off = np.zeros(len(seq_lens) + 1, dtype=np.int64)

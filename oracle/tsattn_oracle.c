@@ -39,6 +39,9 @@
  *                                                         invariance, numpy restatement with the same
  *                                                         sequential float sum
  *   tso_rope_normalize_rows  train/cpu_infer.cpp:486-499  composition of the two above
+ *   tso_kv_product         train/cpu_infer.cpp:320-337   pinned: numpy restatement (index shuffle z ^ blk, products,
+ *                                                         rounding), blk 0 = plain product, the four blocks are
+ *                                                         permutations of each other when value is constant
  *
  * The reference holds no golden vectors or known-answer tests for this path, and the two files
  * that contain it (gpt_cpu.cpp, cpu_infer.cpp) cannot be compiled without the CUDA SDK, so the
@@ -303,6 +306,28 @@ void tso_rope_normalize_rows(int dtype, const void *src, int src_is_i32, int64_t
     }
     free(tmp);
     free(hs);
+}
+
+/* KVProduct, train/cpu_infer.cpp:320-337: the step after attention.  Per head and block blk < rep (COMBINER_REP = 4,
+ * model_params/model_dim.h:12): kv[head*d*rep + blk*d + z] = int8(k[head*d + (z ^ blk)] * valLookup[head*d + z]),
+ * int8 = round to nearest even clamped to +-127 (:88-92).  mult multiplies the product before the conversion (1 in
+ * the CPU path; the GPU kernel's kvMult, compute/gpt_combiner.cuh:13-37). */
+void tso_kv_product(const int8_t *k, int64_t k_pitch, const float *val, int64_t val_pitch, int64_t n_rows, int n_heads,
+                    int head_dim, int rep, float mult, int8_t *kv, int64_t kv_pitch)
+{
+    for (int64_t t = 0; t < n_rows; ++t) {
+        for (int head = 0; head < n_heads; ++head) {
+            int head_offset = head * head_dim;
+            for (int blk = 0; blk < rep; ++blk) {
+                int64_t base = (int64_t)head * head_dim * rep + (int64_t)blk * head_dim;
+                for (int z = 0; z < head_dim; ++z) {
+                    int8_t key_shfl = k[t * k_pitch + head_offset + (z ^ blk)];
+                    float value = val[t * val_pitch + head_offset + z];
+                    kv[t * kv_pitch + base + z] = tso_float_to_i8((key_shfl * value) * mult);
+                }
+            }
+        }
+    }
 }
 
 /* ------------------------------------------------------------------------------------------ */

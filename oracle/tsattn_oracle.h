@@ -44,6 +44,8 @@ void tso_rope_normalize_rows(int dtype, const void *src, int src_is_i32, int64_t
                              const int32_t *pos, const float *rope, float rotate_dir, int n_heads, int head_dim,
                              float vec_scale, float scale_mult, uint8_t *q, int64_t q_pitch, float *scale,
                              int64_t scale_pitch);
+void tso_kv_product(const int8_t *k, int64_t k_pitch, const float *val, int64_t val_pitch, int64_t n_rows, int n_heads,
+                    int head_dim, int rep, float mult, int8_t *kv, int64_t kv_pitch);
 void tso_quantize_rows_bf16(int dtype, const uint16_t *x, int64_t x_pitch, int64_t n_rows,
                             int n_heads, int head_dim, uint8_t *q, int64_t q_pitch, float *scale,
                             int64_t scale_pitch);

@@ -83,3 +83,20 @@ def test_producer_feeds_prefill(ctx):
     gst, gfi = ctx.build_spans(off, n, 10 ** 6)
     out = ctx.compute_val_lookup(capi.I8, H, gq, gk, gv, VEC, gks, VEC, gst, gfi, 0.0).cpu().numpy()
     assert_within_tolerance(out, want, "producer -> prefill")
+
+
+@pytest.mark.parametrize("d,H", [(64, 12), (128, 3)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_kv_product_bit_exact(ctx, d, H, f16):
+    """tsattn_kv_product against KVProduct of cpu_infer.cpp:320-337 on the same inputs: identical bytes."""
+    n = 77
+    rng = np.random.default_rng(d)
+    k = rng.integers(-127, 128, (n, H * d)).astype(np.int8)
+    val = (rng.standard_normal((n, H * d)) * 0.4).astype(np.float32)
+    if f16:
+        val = val.astype(np.float16).astype(np.float32)      # what the kernel sees when the attention output is half
+    for mult in (1.0, 0.73):
+        want = orc.kv_product(k, val, H, mult=mult)
+        tv = torch.from_numpy(val).cuda()
+        got = ctx.kv_product(torch.from_numpy(k.view(np.uint8)).cuda(), tv.half() if f16 else tv, H, mult=mult)
+        assert np.array_equal(got.cpu().numpy().view(np.int8), want)

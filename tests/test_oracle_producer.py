@@ -140,3 +140,25 @@ def test_int32_source_and_rope_composition():
     rot = np.stack([orc.apply_rope(rope[p], 1.0, x[i], 64) for i, p in enumerate(pos)])
     q2, s2 = orc.rope_normalize_rows(orc.I8, rot, 2)
     assert np.array_equal(q, q2) and np.array_equal(s, s2)
+
+
+def test_kv_product_against_numpy():
+    """KVProduct (cpu_infer.cpp:320-337): index shuffle z ^ blk inside each head, product, int8 rounding."""
+    rng = np.random.default_rng(12)
+    n, H, d = 5, 3, 64
+    k = rng.integers(-127, 128, (n, H * d)).astype(np.int8)
+    val = (rng.standard_normal((n, H * d)) * 0.3).astype(np.float32)
+    kv = orc.kv_product(k, val, H)
+    assert kv.shape == (n, H * d * 4)
+    k3 = k.reshape(n, H, d).astype(np.float32); v3 = val.reshape(n, H, d)
+    z = np.arange(d)
+    for blk in range(4):
+        want = np.clip(np.rint(k3[:, :, z ^ blk] * v3), -127, 127).astype(np.int8)
+        assert np.array_equal(kv.reshape(n, H, 4, d)[:, :, blk], want)
+    # blk 0 is the plain product; with a constant value the blocks are permutations of block 0
+    kv1 = orc.kv_product(k, np.full_like(val, 0.5), H).reshape(n, H, 4, d)
+    for blk in range(4):
+        assert np.array_equal(kv1[:, :, blk], kv1[:, :, 0][:, :, z ^ blk])
+    # clamp
+    big = orc.kv_product(np.full((1, 64), 100, np.int8), np.full((1, 64), 3.0, np.float32), 1)
+    assert (big == 127).all()

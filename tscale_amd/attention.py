@@ -111,6 +111,16 @@ class AttentionContext:
         capi.check(self.lib.tsattn_rope_normalize_rows(self.handle, ctypes.byref(a), _stream_ptr()))
         return q, scale
 
+    def kv_product(self, k, value, n_heads, rep=4, mult=1.0):
+        """KVProduct (cpu_infer.cpp:320-337): k uint8 (int8 bytes) [n, H*d], value f32/f16 [n, H*d] -> uint8 [n, H*d*rep]."""
+        n, hd = k.shape
+        assert value.shape == k.shape and value.is_contiguous() and k.is_contiguous()
+        kv = torch.empty((n, hd * rep), dtype=torch.uint8, device=k.device)
+        vdt = capi.OUT_F16 if value.dtype == torch.float16 else capi.OUT_F32
+        capi.check(self.lib.tsattn_kv_product(self.handle, n, n_heads, hd // n_heads, rep, _ptr(k), hd, vdt, _ptr(value), hd,
+                                              float(mult), _ptr(kv), hd * rep, _stream_ptr()))
+        return kv
+
     def build_spans(self, seq_offset, n_tokens, window, doc_start_flag=None):
         """seq_offset: int32 [n_seqs+1] on the device.  Returns (span_start, span_finish) int32 [n_tokens]."""
         st = torch.empty(n_tokens, dtype=torch.int32, device=self.device)

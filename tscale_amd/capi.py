@@ -93,7 +93,7 @@ class FillArgs(_c.Structure):
 
 
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
+           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
 
 _lib = None
 
@@ -131,6 +131,9 @@ def load():
         L.tsattn_rope_normalize_rows.argtypes = [_c.c_void_p, _c.POINTER(ProduceArgs), _c.c_void_p]
         L.tsattn_fill_rope_table.restype = None
         L.tsattn_fill_rope_table.argtypes = [_c.c_int, _c.c_int64, _c.c_void_p]
+        L.tsattn_kv_product.restype = _c.c_int
+        L.tsattn_kv_product.argtypes = [_c.c_void_p, _c.c_int64, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int,
+                                        _c.c_void_p, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64, _c.c_void_p]
         L.tsattn_quantize_rows.restype = _c.c_int
         L.tsattn_quantize_rows.argtypes = [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64,
                                            _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64,

@@ -293,6 +293,30 @@ int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, 
     return TSATTN_OK;
 }
 
+int tsattn_kv_product(tsattn_handle_t h, int64_t n_rows, int n_heads, int head_dim, int rep, const void *k, int64_t k_pitch,
+                      int value_dtype, const void *value, int64_t value_pitch, float mult, void *kv, int64_t kv_pitch,
+                      void *stream)
+{
+    if (!h) return fail(TSATTN_ERR_BAD_ARG, "tsattn_kv_product: null handle");
+    if (!head_dim_ok(head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_kv_product: head_dim %d (64 or 128 supported)", head_dim);
+    if (rep < 1 || rep > 4) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_kv_product: rep %d (1..4 supported)", rep);
+    if (value_dtype != TSATTN_OUT_F32 && value_dtype != TSATTN_OUT_F16) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_kv_product: value dtype %d", value_dtype);
+    if (n_rows < 0 || n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_kv_product: negative size");
+    if (n_rows == 0) return TSATTN_OK;
+    if (!k || !value || !kv) return fail(TSATTN_ERR_BAD_ARG, "tsattn_kv_product: null data pointer");
+    const int64_t row = (int64_t)n_heads * head_dim;
+    const int vsz = value_dtype == TSATTN_OUT_F16 ? 2 : 4;
+    if (k_pitch < row || value_pitch < row || kv_pitch < row * rep || k_pitch % 16 || kv_pitch % 16 || (value_pitch * vsz) % 16 ||
+        !aligned16(k) || !aligned16(value) || !aligned16(kv))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_kv_product: pitches must cover a row and, like the pointers, be multiples of 16 bytes");
+    tsattn::KvProductParams p;
+    p.k = (const uint8_t *)k; p.k_pitch = k_pitch; p.val = value; p.val_pitch = value_pitch; p.n_rows = n_rows;
+    p.n_heads = n_heads; p.head_dim = head_dim; p.rep = rep; p.mult = mult; p.kv = (uint8_t *)kv; p.kv_pitch = kv_pitch;
+    hipError_t e = tsattn::launch_kv_product(p, value_dtype == TSATTN_OUT_F16, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "kv product launch");
+    return TSATTN_OK;
+}
+
 void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table)
 {
     if (!table || head_dim <= 0 || head_dim % 64 || max_len <= 0) return;

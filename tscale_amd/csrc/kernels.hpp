@@ -108,6 +108,20 @@ struct ProduceParams {
 hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head_dim, bool src_i32, hipStream_t st);
 void fill_rope_table(int width, int64_t max_len, float *table);
 
+struct KvProductParams {
+    const uint8_t *k;
+    int64_t k_pitch;   // bytes
+    const void *val;
+    int64_t val_pitch; // elements
+    int64_t n_rows;
+    int n_heads, head_dim, rep;
+    float mult;
+    uint8_t *kv;
+    int64_t kv_pitch;  // bytes
+};
+
+hipError_t launch_kv_product(const KvProductParams &p, bool val_f16, hipStream_t st);
+
 struct FillParams {
     const int32_t *seq_offset;
     const uint8_t *k_src, *v_src;

@@ -153,6 +153,60 @@ hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head
     return hipGetLastError();
 }
 
+// KVProduct, gpt/train/cpu_infer.cpp:320-337 (GPU form compute/gpt_combiner.cuh:13-37): the step after attention,
+// kv[head][blk][z] = int8(k[head][z ^ blk] * value[head][z] * mult) for blk < 4.  One thread per 16 consecutive z of a
+// (row, head): z ^ blk stays inside an aligned group of four, so a thread needs only its own 16 key bytes.
+template <bool VAL_F16>
+__global__ __launch_bounds__(256) void kv_product_kernel(KvProductParams p)
+{
+    const int chunks = p.head_dim / 16;
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t total = p.n_rows * p.n_heads * chunks;
+    if (id >= total) return;
+    const int c = (int)(id % chunks);
+    const int head = (int)((id / chunks) % p.n_heads);
+    const int64_t row = id / ((int64_t)chunks * p.n_heads);
+    const int64_t e = (int64_t)head * p.head_dim + c * 16;
+    const v4i kw = *(const v4i *)(p.k + row * p.k_pitch + e);
+    const int kws[4] = {kw.x, kw.y, kw.z, kw.w};
+    float key[16], val[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) key[i] = (float)(int8_t)((kws[i / 4] >> (8 * (i % 4))) & 0xff);
+    if (VAL_F16) {
+        const v8h a = *(const v8h *)((const _Float16 *)p.val + row * p.val_pitch + e);
+        const v8h b = *(const v8h *)((const _Float16 *)p.val + row * p.val_pitch + e + 8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { val[i] = (float)a[i]; val[8 + i] = (float)b[i]; }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const v4f a = *(const v4f *)((const float *)p.val + row * p.val_pitch + e + 4 * i);
+            val[4 * i] = a.x; val[4 * i + 1] = a.y; val[4 * i + 2] = a.z; val[4 * i + 3] = a.w;
+        }
+    }
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+        if (blk >= p.rep) break;
+        uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int z = 0; z < 16; ++z) {
+            const float y = (key[z ^ blk] * val[z]) * p.mult;
+            w[z / 4] |= (uint32_t)(uint8_t)float_to_i8(y) << (8 * (z % 4));
+        }
+        *(v4i *)(p.kv + row * p.kv_pitch + ((int64_t)head * p.rep + blk) * p.head_dim + c * 16) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    }
+}
+
+hipError_t launch_kv_product(const KvProductParams &p, bool val_f16, hipStream_t st)
+{
+    const int64_t total = p.n_rows * p.n_heads * (p.head_dim / 16);
+    if (total == 0) return hipSuccess;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (val_f16) hipLaunchKernelGGL((kv_product_kernel<true>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((kv_product_kernel<false>), grid, block, 0, st, p);
+    return hipGetLastError();
+}
+
 // FillRopeBuf, gpt/att/rope.cpp:4-24 (host): table[t][base + k] = cos(t f), table[t][base + k + 32] = sin(t f),
 // f = theta^-(2 (base/2 + k) / width), theta = 500000.  The float/double mix follows the reference's C++ overloads.
 void fill_rope_table(int width, int64_t max_len, float *table)
