@@ -197,27 +197,37 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
     // With d = 64 one 128-byte line of K or V holds the rows of two heads: consecutive workgroups then
     // alternate between the two heads of a pair on the same query tile, so the pair shares the line in L2.
-    const int hg = (D == 64 && (p.n_heads & 1) == 0) ? 2 : 1;
-    int head = (wg / (hg * n_qtiles)) * hg + wg % hg;
-    int tile = n_qtiles - 1 - ((wg / hg) % n_qtiles); // long rows first
-    // When the caller has said that the batch repeats the same span structure every T query tiles (equal-length
-    // sequences, causal), each XCD still gets a contiguous run of (head, sequence) units, but walks groups of G
-    // units position by position from the end of the sequences to their start: the longest rows of every unit
-    // first, the shortest last, so the launch does not end on a few long-running workgroups.  G is chosen by
-    // the host so that the K/V rows of a group fit in the XCD's L2.
-    {
+    // All divisions are by launch constants whose reciprocals the host has prepared.
+    auto divmod = [](uint32_t x, PrefillParams::Div by, uint32_t &rem) {
+        uint32_t q = __umulhi(x, by.m);
+        int32_t r = (int32_t)(x - q * by.d);
+        if (r < 0) { --q; r += (int32_t)by.d; }
+        if (r >= (int32_t)by.d) { ++q; r -= (int32_t)by.d; }
+        rem = (uint32_t)r;
+        return q;
+    };
+    const int hs = p.hg_shift, hg = 1 << hs;
+    int head, tile;
+    if (p.period_group > 0) {
+        // The caller has said that the batch repeats the same span structure every T query tiles (equal-length
+        // sequences, causal): each XCD still gets a contiguous run of (head, sequence) units, but walks groups of
+        // G units position by position from the end of the sequences to their start: the longest rows of every
+        // unit first, the shortest last, so the launch does not end on a few long-running workgroups.  G is
+        // chosen by the host so that the K/V rows of a group fit in the XCD's L2.
         const int T = p.period_tiles, G = p.period_group;
-        const int per_xcd = n_wg >> 3;
-        if (T > 1 && G > 0) {
-            const int x = wg / per_xcd, i = wg % per_xcd;
-            const int R = per_xcd / (T * hg);
-            const int grp = i / (G * T * hg), j = i % (G * T * hg);
-            const int pos_rank = j / (G * hg), rem = j % (G * hg);
-            const int U = x * R + grp * G + rem / hg, hsel = rem % hg;
-            const int n_seq = n_qtiles / T;
-            head = (U / n_seq) * hg + hsel;
-            tile = (U % n_seq) * T + (T - 1 - pos_rank);
-        }
+        const uint32_t x = blockIdx.x & 7, i = blockIdx.x >> 3; // XCD and index inside its run
+        uint32_t j, rem, seq;
+        const uint32_t grp = divmod(i, p.by_group_wgs, j);          // / (G * T * hg)
+        const uint32_t pos_rank = divmod(j, p.by_group_units, rem); // / (G * hg)
+        const uint32_t U = x * p.units_per_xcd + grp * G + (rem >> hs);
+        const uint32_t hgrp = divmod(U, p.by_seqs, seq);            // / (n_qtiles / T)
+        head = (int)((hgrp << hs) + (rem & (hg - 1)));
+        tile = (int)(seq * T + (T - 1 - pos_rank));
+    } else {
+        uint32_t t;
+        const uint32_t hgrp = divmod((uint32_t)wg >> hs, p.by_qtiles, t);
+        head = (int)((hgrp << hs) + (wg & (hg - 1)));
+        tile = n_qtiles - 1 - (int)t; // long rows first
     }
     const int q0 = tile * PF_BM + wave * 32;
     const int from = q0 + qi;
@@ -679,10 +689,20 @@ static void launch_prefill_do(const PrefillParams &p_in, dim3 grid2, hipStream_t
     // units; units are then walked in groups whose K and V rows (2 * period * d bytes per head) stay within
     // about the size of the XCD's 4 MB L2 (the rows are streamed, so slightly more than it still pays).
     PrefillParams p = p_in;
+    auto make_div = [](uint32_t d) {
+        PrefillParams::Div r;
+        r.d = d ? d : 1;
+        r.m = (uint32_t)(((1ull << 32) + r.d - 1) / r.d);
+        return r;
+    };
     p.period_group = 0;
+    p.units_per_xcd = 0;
+    const int hg = (D == 64 && (p.n_heads & 1) == 0) ? 2 : 1;
+    p.hg_shift = hg == 2 ? 1 : 0;
+    p.by_qtiles = make_div((uint32_t)n_qtiles);
+    p.by_group_wgs = p.by_group_units = p.by_seqs = make_div(1);
     {
         const int T = p.period_tiles;
-        const int hg = (D == 64 && (p.n_heads & 1) == 0) ? 2 : 1;
         const int n_wg = (int)grid.x, per_xcd = n_wg / 8;
         if (T > 1 && n_wg % 8 == 0 && per_xcd % (T * hg) == 0 && n_qtiles % T == 0) {
             const int R = per_xcd / (T * hg);
@@ -691,6 +711,10 @@ static void launch_prefill_do(const PrefillParams &p_in, dim3 grid2, hipStream_t
             for (int c = 1; c <= R; ++c)
                 if (R % c == 0 && c * unit_bytes <= (5 << 20)) G = c;
             p.period_group = G;
+            p.units_per_xcd = R;
+            p.by_group_wgs = make_div((uint32_t)(G * T * hg));
+            p.by_group_units = make_div((uint32_t)(G * hg));
+            p.by_seqs = make_div((uint32_t)(n_qtiles / T));
         }
     }
     const bool dump = p.dbg != nullptr;
