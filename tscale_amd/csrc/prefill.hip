@@ -192,6 +192,17 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     const int g = lane >> 5;  // which half of the contraction this lane feeds
     // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of
     // (head, query tile) pairs: equal work per XCD, and the K/V rows a run shares stay in its L2.
+    // Ask for every kernel argument the prologue needs in one go: left to itself the compiler fetches them where
+    // they are first used, which chains five scalar-load round trips in front of the first K/V request.
+#define PF_TOUCH(x) asm volatile("" ::"s"(x))
+    PF_TOUCH(p.q); PF_TOUCH(p.k); PF_TOUCH(p.v); PF_TOUCH(p.q_pitch); PF_TOUCH(p.k_pitch); PF_TOUCH(p.v_pitch);
+    PF_TOUCH(p.qs); PF_TOUCH(p.ks); PF_TOUCH(p.vs); PF_TOUCH(p.scale_pitch); PF_TOUCH(p.span_start); PF_TOUCH(p.span_finish);
+    PF_TOUCH(p.span_tiles); PF_TOUCH(p.n_tokens); PF_TOUCH(p.n_heads); PF_TOUCH(p.k_global_scale);
+    PF_TOUCH(p.period_tiles); PF_TOUCH(p.period_group); PF_TOUCH(p.units_per_xcd); PF_TOUCH(p.hg_shift);
+    PF_TOUCH(p.by_qtiles.d); PF_TOUCH(p.by_qtiles.m); PF_TOUCH(p.by_group_wgs.d); PF_TOUCH(p.by_group_wgs.m);
+    PF_TOUCH(p.by_group_units.d); PF_TOUCH(p.by_group_units.m); PF_TOUCH(p.by_seqs.d); PF_TOUCH(p.by_seqs.m);
+    PF_TOUCH(p.qs_const); PF_TOUCH(p.ks_const); PF_TOUCH(p.vs_const); PF_TOUCH(p.slope); PF_TOUCH(p.out); PF_TOUCH(p.out_pitch);
+#undef PF_TOUCH
     int wg = blockIdx.x;
     const int n_wg = gridDim.x;
     if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
@@ -235,24 +246,14 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     const int64_t hoff = (int64_t)head * D;
 
     // ---- spans --------------------------------------------------------------------------------
-    int sp_a = 1, sp_b = 0;
-    if (row_ok) {
-        sp_a = p.span_start[from];
-        sp_b = p.span_finish[from];
-    }
-    // ---- query operand and per-row constants (issued before the span reductions so that their latency
-    //      runs under them) ---------------------------------------------------------------------------
-    Qk qk;
-    if (row_ok) qk.load_q(p.q + (int64_t)from * p.q_pitch + hoff, g);
-    else qk.clear_q();
-    const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
-    const bool has_keys = sp_b >= sp_a;
     // What the loop needs to know about the spans: the workgroup's key range and the extremes of this wave's 32
-    // spans.  Either read from the caller's summary (scalar loads, so K and V can be requested at once) or
-    // reduced here from the rows' spans (shuffles, LDS, a barrier).
-    bool w_all_have_keys;
-    int w_min_a, w_max_a, w_min_b, w_max_b, b_min_a, b_max_b;
-    if (p.span_tiles) {
+    // spans.  Either read from the caller's summary (scalar loads issued first of all, so K and V can be requested
+    // as soon as they return, without waiting for the per-row spans) or reduced below from the rows' spans
+    // (shuffles, LDS, a barrier).
+    bool w_all_have_keys = false;
+    int w_min_a = 0, w_max_a = 0, w_min_b = 0, w_max_b = 0, b_min_a = 0, b_max_b = 0;
+    const bool have_summary = p.span_tiles != nullptr;
+    if (have_summary) {
         typedef __attribute__((address_space(4))) const int32_t *const_i32_ptr;
         const const_i32_ptr t = (const_i32_ptr)(p.span_tiles + (int64_t)tile * SPAN_TILE_INTS);
         const const_i32_ptr w = t + SPAN_TILE_WAVE0 + __builtin_amdgcn_readfirstlane(wave) * SPAN_TILE_WAVE_INTS;
@@ -263,10 +264,22 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         w_min_b = w[2];
         w_max_b = w[3];
         w_all_have_keys = w[4] != 0;
-    } else {
-        w_all_have_keys = __all(has_keys);
-        w_min_a = has_keys ? sp_a : 0x7fffffff, w_max_a = has_keys ? sp_a : -1;
-        w_min_b = has_keys ? sp_b : 0x7fffffff, w_max_b = has_keys ? sp_b : -1;
+    }
+    int sp_a = 1, sp_b = 0;
+    if (row_ok) {
+        sp_a = p.span_start[from];
+        sp_b = p.span_finish[from];
+    }
+    // ---- query operand and per-row constants (issued before anything waits for the spans) -------------------
+    Qk qk;
+    if (row_ok) qk.load_q(p.q + (int64_t)from * p.q_pitch + hoff, g);
+    else qk.clear_q();
+    const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
+    if (!have_summary) {
+        const bool hk = sp_b >= sp_a;
+        w_all_have_keys = __all(hk);
+        w_min_a = hk ? sp_a : 0x7fffffff, w_max_a = hk ? sp_a : -1;
+        w_min_b = hk ? sp_b : 0x7fffffff, w_max_b = hk ? sp_b : -1;
         for (int o = 16; o > 0; o >>= 1) {
             w_min_a = min(w_min_a, __shfl_xor(w_min_a, o, WAVE));
             w_max_a = max(w_max_a, __shfl_xor(w_max_a, o, WAVE));
@@ -400,6 +413,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             // keys of register r of sub-tile kt: kb + kt*32 + 8*(r/4) + 4*g + r%4
             const int rel_a = sp_a - kb - 4 * g;            // span start relative to this lane's first key
             const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
+            const bool has_keys = sp_b >= sp_a;
             const float dist0 = (float)(from - kb - 4 * g);
 #pragma unroll
             for (int kt = 0; kt < PF_KT; ++kt) {
