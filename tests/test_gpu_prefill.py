@@ -227,3 +227,52 @@ def test_prefill_span_summary_gives_identical_results(ctx, window, slope):
     with_tiles = ctx.compute_val_lookup(*args, span_tiles=tiles).cpu().numpy()
     assert np.array_equal(base, with_tiles)
     assert_within_tolerance(base, orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, slope), "span summary")
+
+
+@pytest.mark.parametrize("dtype,d,H,n,window", [
+    (capi.E4M3, 64, 3, 333, 10 ** 6),    # odd head count with d=64: no head pairing; 9 workgroups: no XCD remap
+    (capi.I8, 64, 6, 1024, 100),         # 48 workgroups: remapped, heads paired
+    (capi.I8, 128, 5, 257, 10 ** 6),     # one row in the last query tile
+    (capi.E4M3, 128, 2, 640, 64),
+])
+def test_prefill_layout_variants(ctx, dtype, d, H, n, window):
+    """Row pitches larger than a row, a scale pitch larger than the token count, f32 output into a padded buffer,
+    a launch-order hint that does not apply, with and without the span summary: results as for packed arrays."""
+    q, qs, k, ks, v, vs = make_qkv(3 * d + H, n, H, d, dtype)
+    st, fi = orc.make_spans([n], window)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, 0.25)
+    pad = 48                      # bytes; keeps 16-byte alignment
+    sp = n + 37                   # scale pitch
+    def padded(a):
+        t = torch.zeros((n, H * d + pad), dtype=torch.uint8, device="cuda")
+        t[:, :H * d] = torch.from_numpy(a).cuda()
+        return t[:, :H * d]       # a view whose stride(0) is the padded pitch
+    def scale_plane(a):
+        t = torch.zeros((H, sp), dtype=torch.float32, device="cuda")
+        t[:, :n] = torch.from_numpy(a).cuda()
+        return t[:, :n]
+    out_buf = torch.full((n, H * d + 8), -7.0, dtype=torch.float32, device="cuda")
+    out = out_buf[:, :H * d]
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    for use_summary in (False, True):
+        out_buf.fill_(-7.0)
+        tiles = ctx.build_span_tiles(t(st), t(fi)) if use_summary else None
+        a = capi.PrefillArgs()   # straight through the C ABI: the Python helper insists on contiguous scale planes
+        qq, kk, vv = padded(q), padded(k), padded(v)
+        sq, sk, sv = scale_plane(qs), scale_plane(ks), scale_plane(vs)
+        a.dtype, a.out_dtype = dtype, capi.OUT_F32
+        a.n_tokens, a.n_heads, a.head_dim = n, H, d
+        a.q, a.k, a.v = qq.data_ptr(), kk.data_ptr(), vv.data_ptr()
+        a.q_pitch = a.k_pitch = a.v_pitch = H * d + pad
+        a.q_scale, a.k_scale, a.v_scale, a.scale_pitch = sq.data_ptr(), sk.data_ptr(), sv.data_ptr(), sp
+        st_d, fi_d = t(st), t(fi)
+        a.span_start, a.span_finish = st_d.data_ptr(), fi_d.data_ptr()
+        a.span_tiles = None if tiles is None else tiles.data_ptr()
+        a.alibi_slope = 0.25
+        a.out, a.out_pitch = out.data_ptr(), (H * d + 8) * 4
+        a.causal_period = 128
+        import ctypes
+        capi.check(ctx.lib.tsattn_prefill(ctx.handle, ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        assert_within_tolerance(out.cpu().numpy(), want, f"layout variant (summary {use_summary})")
+        assert (out_buf[:, H * d:] == -7.0).all(), "wrote outside the rows"
