@@ -32,6 +32,7 @@ constexpr int PF_BM = 128; // queries per workgroup (the C ABI's causal_period h
 #endif
 constexpr int PF_BN = TSATTN_PF_BN;  // keys per tile (32 or 64)
 constexpr int PF_KT = PF_BN / 32; // 32-key sub-tiles per tile
+constexpr int PF_SHORT_KEYS = 192; // key range a workgroup may handle without the tile loop (see the kernel)
 
 template <int D>
 struct PfLayout {
@@ -180,9 +181,17 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
     constexpr int NLD = (PF_BN * CHUNKS + PF_THREADS - 1) / PF_THREADS;
     constexpr bool LD_ALL = (PF_BN * CHUNKS) % PF_THREADS == 0; // every thread owns NLD chunks       // 16-byte chunks per thread per tile
 
-    __shared__ __attribute__((aligned(16))) uint8_t k_lds[2][L::K_BYTES];
-    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2][L::V_BYTES];
-    __shared__ __attribute__((aligned(16))) float ks_lds[2][PF_BN];
+    // One LDS block carved two ways.  Tile loop: two K tiles, two widened V tiles, two sets of key scales.
+    // Short key ranges (d = 64, at most PF_SHORT_KEYS keys for the whole workgroup): every widened V row and key
+    // scale of the range at once.
+    constexpr int LOOP_BYTES = 2 * L::K_BYTES + 2 * L::V_BYTES + 2 * PF_BN * 4;
+    constexpr int SHORT_BYTES = PF_SHORT_KEYS * L::V_PITCH + PF_SHORT_KEYS * 4;
+    constexpr bool HAS_SHORT = (D == 64) && !DUMP;
+    constexpr int LDS_BYTES = (HAS_SHORT && SHORT_BYTES > LOOP_BYTES) ? SHORT_BYTES : LOOP_BYTES;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
+    auto k_lds = [&](int b) -> uint8_t * { return lds_raw + b * L::K_BYTES; };
+    auto v_lds = [&](int b) -> uint8_t * { return lds_raw + 2 * L::K_BYTES + b * L::V_BYTES; };
+    auto ks_lds = [&](int b) -> float * { return (float *)(lds_raw + 2 * L::K_BYTES + 2 * L::V_BYTES) + b * PF_BN; };
     __shared__ int red_lds[2 * PF_WAVES];
 
     const int tid = threadIdx.x;
@@ -380,102 +389,110 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                 const int ch = tid + i * PF_THREADS;
                 if (!LD_ALL && ch >= PF_BN * CHUNKS) break;
                 const int r = ch / CHUNKS, c = ch % CHUNKS;
-                *(v4i *)(k_lds[buf] + r * L::K_PITCH + c * 16) = rk[i];
+                *(v4i *)(k_lds(buf) + r * L::K_PITCH + c * 16) = rk[i];
                 v8h lo, hi;
                 widen_v<DTYPE>(rv[i], rvs[i], lo, hi);
-                *(v8h *)(v_lds[buf] + r * L::V_PITCH + c * 32) = lo;
-                *(v8h *)(v_lds[buf] + r * L::V_PITCH + c * 32 + 16) = hi;
+                *(v8h *)(v_lds(buf) + r * L::V_PITCH + c * 32) = lo;
+                *(v8h *)(v_lds(buf) + r * L::V_PITCH + c * 32 + 16) = hi;
             }
-            if (tid < PF_BN) ks_lds[buf][tid] = rks * ads;
+            if (tid < PF_BN) ks_lds(buf)[tid] = rks * ads;
         };
 
         // V^T operands (A of the P.V MFMA) of one group: keys kt*32 + 16*i + 4*g + {0..3} and the same + 8
         const int i16 = lane & 15, dh = (lane >> 4) & 1;
         v8h va[2][DT];
-        auto vload = [&](int slot, int grp, int buf) {
-            const int kt = grp >> 1, i = grp & 1;
-            const int key0 = kt * 32 + 16 * i + 4 * g + (i16 >> 2);
+        auto vload_rows = [&](int slot, const uint8_t *rows16) { // rows16: the first of 16 consecutive V rows in LDS
+            const int key0 = 4 * g + (i16 >> 2);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const uint8_t *vb = v_lds[buf] + key0 * L::V_PITCH + (dt * 32 + 16 * dh + 4 * (i16 & 3)) * 2;
+                const uint8_t *vb = rows16 + key0 * L::V_PITCH + (dt * 32 + 16 * dh + 4 * (i16 & 3)) * 2;
                 v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb));
                 v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(vb + 8 * L::V_PITCH));
                 va[slot][dt] = __builtin_bit_cast(v8h, __builtin_shufflevector(a0, a1, 0, 1, 2, 3, 4, 5, 6, 7));
+            }
+        };
+        auto vload = [&](int slot, int grp, int buf) { vload_rows(slot, v_lds(buf) + grp * 16 * L::V_PITCH); };
+
+        // ---- one 64-key tile for this wave's 32 queries ---------------------------------------------------
+        // General form: any mix of rows, one 32-key sub-tile at a time (few live registers; a sub-tile outside
+        // every span of the wave is skipped, which for a short window is one in four).
+        // One 32-key sub-tile in general form: accumulators of K.Q^T in, weights and V^T.P^T out.  ksp: the sub-tile's
+        // 32 key scales in LDS; vrows: its 32 widened V rows in LDS; key0: the index of its first key.
+        auto sub_tile = [&](auto interior_tag, const typename Qk::acc_t &acc, const float *ksp, const uint8_t *vrows, int key0) {
+            constexpr bool INTERIOR = decltype(interior_tag)::value;
+            // key of register r: key0 + 8*(r/4) + 4*g + r%4
+            const int rel_a = sp_a - key0 - 4 * g;           // span start relative to this lane's first key
+            const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
+            const bool has_keys = sp_b >= sp_a;
+            const float dist0 = (float)(from - key0 - 4 * g);
+            float t[16];
+            float tmax = -INFINITY;
+            const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
+            vload_rows(0, vrows);
+            vload_rows(1, vrows + 16 * L::V_PITCH);
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+                v4f ksv = *(const v4f *)(ksp + 8 * c4 + 4 * g);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int r = c4 * 4 + j;
+                    const int off = 8 * c4 + j;
+                    const bool in_span = INTERIOR || ((unsigned)(off - rel_a) <= span_w && has_keys);
+                    if (DUMP) {
+                        if (in_span) {
+                            ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + key0 + off + 4 * g] = Qk::bits(acc, r);
+                        }
+                    }
+                    float x = Qk::to_float(acc, r) * ksv[j];
+                    float tv = fmaf(x, qs, base);
+                    if (SLOPE) tv += p.slope * (float)off;
+                    if (!INTERIOR) tv = in_span ? tv : -INFINITY;
+                    t[r] = tv;
+                    tmax = fmaxf(tmax, tv);
+                }
+            }
+            // the two lanes of a query exchange their maxima only if some lane of the wave is over the
+            // threshold: the common case has no cross-lane operation at all
+            if (__any(tmax > PF_RESCALE_THRESHOLD)) {
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+                const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
+                const float alpha = fast_exp2(-shift);
+                m_ref += shift;
+                l *= alpha;
+                l2 *= alpha;
+#pragma unroll
+                for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) t[r] -= shift;
+            }
+            // P = 2^t ; O^T += V^T . P^T in two groups of DT MFMAs (16 keys each)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                v2h pp[4];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const float p0 = fast_exp2(t[8 * i + 2 * x]);
+                    const float p1 = fast_exp2(t[8 * i + 2 * x + 1]);
+                    pp[x] = v2h{(_Float16)p0, (_Float16)p1};
+                    l += p0;
+                    l2 += p1;
+                }
+                const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[i][dt], pb, o_acc[dt], 0, 0, 0);
             }
         };
 
         // ---- one 64-key tile for this wave's 32 queries ---------------------------------------------------
         // General form: any mix of rows, one 32-key sub-tile at a time (few live registers; a sub-tile outside
         // every span of the wave is skipped, which for a short window is one in four).
-        auto compute_tile = [&](auto interior_tag, auto ref_tag, int buf, int kb) {
+        auto compute_tile = [&](auto interior_tag, int buf, int kb) {
             constexpr bool INTERIOR = decltype(interior_tag)::value;
-            constexpr bool REF = decltype(ref_tag)::value || SLOPE; // general form: logit * qs + base
-            // keys of register r of sub-tile kt: kb + kt*32 + 8*(r/4) + 4*g + r%4
-            const int rel_a = sp_a - kb - 4 * g;            // span start relative to this lane's first key
-            const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
-            const bool has_keys = sp_b >= sp_a;
-            const float dist0 = (float)(from - kb - 4 * g);
 #pragma unroll
             for (int kt = 0; kt < PF_KT; ++kt) {
                 if (!INTERIOR && (kb + kt * 32 + 31 < w_min_a || kb + kt * 32 > w_max_b)) continue;
-                float t[16];
-                float tmax = -INFINITY;
-                const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
-                const typename Qk::acc_t acc = qk.mma(k_lds[buf] + (kt * 32 + qi) * L::K_PITCH, g);
-                vload(0, 2 * kt, buf);
-                vload(1, 2 * kt + 1, buf);
-#pragma unroll
-                for (int c4 = 0; c4 < 4; ++c4) {
-                    const int off0 = kt * 32 + 8 * c4;
-                    v4f ksv = *(const v4f *)(ks_lds[buf] + off0 + 4 * g);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int r = c4 * 4 + j;
-                        const int off = off0 + j;
-                        const bool in_span = INTERIOR || ((unsigned)(off - rel_a) <= span_w && has_keys);
-                        if (DUMP) {
-                            if (in_span) {
-                                ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + kb + off + 4 * g] = Qk::bits(acc, r);
-                            }
-                        }
-                        float x = Qk::to_float(acc, r) * ksv[j];
-                        float tv = REF ? fmaf(x, qs, base) : x * qs;
-                        if (SLOPE) tv += p.slope * (float)off;
-                        if (!INTERIOR) tv = in_span ? tv : -INFINITY;
-                        t[r] = tv;
-                        tmax = fmaxf(tmax, tv);
-                    }
-                }
-                // the two lanes of a query exchange their maxima only if some lane of the wave is over the
-                // threshold: the common case has no cross-lane operation at all
-                if (__any(tmax > PF_RESCALE_THRESHOLD)) {
-                    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-                    const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
-                    const float alpha = fast_exp2(-shift);
-                    m_ref += shift;
-                    l *= alpha;
-                    l2 *= alpha;
-#pragma unroll
-                    for (int i = 0; i < DT; ++i) o_acc[i] *= alpha;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) t[r] -= shift;
-                }
-                // P = 2^t ; O^T += V^T . P^T in two groups of DT MFMAs (16 keys each)
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    v2h pp[4];
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        const float p0 = fast_exp2(t[8 * i + 2 * x]);
-                        const float p1 = fast_exp2(t[8 * i + 2 * x + 1]);
-                        pp[x] = v2h{(_Float16)p0, (_Float16)p1};
-                        l += p0;
-                        l2 += p1;
-                    }
-                    const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[i][dt], pb, o_acc[dt], 0, 0, 0);
-                }
+                const typename Qk::acc_t acc = qk.mma(k_lds(buf) + (kt * 32 + qi) * L::K_PITCH, g);
+                sub_tile(interior_tag, acc, ks_lds(buf) + kt * 32, v_lds(buf) + kt * 32 * L::V_PITCH, kb + kt * 32);
             }
         };
 
@@ -536,8 +553,8 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         auto fast_tile = [&](int buf) {
             static_assert(PF_KT == 2, "the common-tile path is written for 64-key tiles");
             constexpr int QS = Qk::STEPS;
-            const uint8_t *kr0 = k_lds[buf] + qi * L::K_PITCH, *kr1 = kr0 + 32 * L::K_PITCH;
-            const float *ksp = ks_lds[buf] + 4 * g;
+            const uint8_t *kr0 = k_lds(buf) + qi * L::K_PITCH, *kr1 = kr0 + 32 * L::K_PITCH;
+            const float *ksp = ks_lds(buf) + 4 * g;
             // ---- block 1: K.Q^T; sub-tile 0's weights between sub-tile 1's MFMAs ----
             typename Qk::kop_t k0[QS], k1[QS];
 #pragma unroll
@@ -611,14 +628,14 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                 if (w == 3) {
                     const int ch = tid + i * PF_THREADS;
                     const int r = ch / CHUNKS, c = ch % CHUNKS;
-                    uint8_t *vdst = v_lds[buf ^ 1] + r * L::V_PITCH + c * 32;
-                    *(v4i *)(k_lds[buf ^ 1] + r * L::K_PITCH + c * 16) = rk[i];
+                    uint8_t *vdst = v_lds(buf ^ 1) + r * L::V_PITCH + c * 32;
+                    *(v4i *)(k_lds(buf ^ 1) + r * L::K_PITCH + c * 16) = rk[i];
                     *(v8h *)(vdst) = v8h{hh[i][0][0], hh[i][0][1], hh[i][1][0], hh[i][1][1], hh[i][2][0], hh[i][2][1], hh[i][3][0], hh[i][3][1]};
                     *(v8h *)(vdst + 16) = v8h{hh[i][4][0], hh[i][4][1], hh[i][5][0], hh[i][5][1], hh[i][6][0], hh[i][6][1], hh[i][7][0], hh[i][7][1]};
                 }
                 PF_FENCE;
             }
-            if (tid < PF_BN) ks_lds[buf ^ 1][tid] = rks * ads;
+            if (tid < PF_BN) ks_lds(buf ^ 1)[tid] = rks * ads;
         };
 #undef PF_FENCE
 
@@ -648,8 +665,8 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                 // does this wave need the tile at all, and does it need the per-element mask?
                 if (!(kb + PF_BN - 1 < w_min_a || kb > w_max_b)) {
                     const bool interior = w_all_have_keys && (kb >= w_max_a) && (kb + PF_BN - 1 <= w_min_b);
-                    if (interior) compute_tile(std::true_type{}, std::true_type{}, buf, kb);
-                    else compute_tile(std::false_type{}, std::true_type{}, buf, kb);
+                    if (interior) compute_tile(std::true_type{}, buf, kb);
+                    else compute_tile(std::false_type{}, buf, kb);
                 }
                 if (it + 1 < n_tiles) store_tile(buf ^ 1);
                 if (it + 2 < n_tiles) load_tile();
