@@ -84,6 +84,13 @@ struct QkMma<TSATTN_E4M3, D> {
         return v8i{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
     }
     __device__ acc_t step(kop_t kk, int s, acc_t acc) const { return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kk, q[s], acc, 0, 0, 0, 0, 0, 0); }
+    // the same operand straight from global memory (row_off: byte offset of the key's row in the descriptor)
+    __device__ static kop_t load_k_global(__amdgpu_buffer_rsrc_t kr, int row_off, int g, int s)
+    {
+        const v4i a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(kr, row_off + 64 * s + 32 * g, 0, 0));
+        const v4i b = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(kr, row_off + 64 * s + 32 * g + 16, 0, 0));
+        return v8i{a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    }
     __device__ static float to_float(const acc_t &a, int r) { return a[r]; }
     __device__ static float bits(const acc_t &a, int r) { return a[r]; }
 };
@@ -114,6 +121,10 @@ struct QkMma<TSATTN_I8, D> {
     typedef v4i kop_t;
     __device__ static kop_t load_k(const uint8_t *krow, int g, int s) { return *(const v4i *)(krow + 32 * s + 16 * g); }
     __device__ acc_t step(kop_t kk, int s, acc_t acc) const { return __builtin_amdgcn_mfma_i32_32x32x32_i8(kk, q[s], acc, 0, 0, 0); }
+    __device__ static kop_t load_k_global(__amdgpu_buffer_rsrc_t kr, int row_off, int g, int s)
+    {
+        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(kr, row_off + 32 * s + 16 * g, 0, 0));
+    }
     __device__ static float to_float(const acc_t &a, int r) { return (float)a[r]; }
     __device__ static float bits(const acc_t &a, int r) { return __int_as_float(a[r]); }
 };
@@ -172,7 +183,7 @@ typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
 constexpr float PF_RESCALE_THRESHOLD = 8.0f;
 
 template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP>
-__global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(PrefillParams p, int n_qtiles)
+__global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefill_kernel(PrefillParams p, int n_qtiles)
 {
     typedef PfLayout<D> L;
     typedef QkMma<DTYPE, D> Qk;
@@ -352,7 +363,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         const __amdgpu_buffer_rsrc_t ksr = rsrc(ks_ptr, s_left), vsr = rsrc(vs_ptr, s_left);
         // scalar byte offsets of the next tile to load, relative to the descriptors' bases
         uint32_t k_soff = 0, v_soff = 0, s_soff = 0;
-        auto load_tile = [&]() { // loads the next tile in sequence
+        auto load_tile = [&]() __attribute__((always_inline)) { // loads the next tile in sequence
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
                 if (!LD_ALL && tid + i * PF_THREADS >= PF_BN * CHUNKS) break;
@@ -383,7 +394,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                 vr = rsrc(v_ptr, v_left);
             }
         };
-        auto store_tile = [&](int buf) {
+        auto store_tile = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
                 const int ch = tid + i * PF_THREADS;
@@ -401,7 +412,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         // V^T operands (A of the P.V MFMA) of one group: keys kt*32 + 16*i + 4*g + {0..3} and the same + 8
         const int i16 = lane & 15, dh = (lane >> 4) & 1;
         v8h va[2][DT];
-        auto vload_rows = [&](int slot, const uint8_t *rows16) { // rows16: the first of 16 consecutive V rows in LDS
+        auto vload_rows = [&](int slot, const uint8_t *rows16) __attribute__((always_inline)) { // rows16: the first of 16 consecutive V rows in LDS
             const int key0 = 4 * g + (i16 >> 2);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
@@ -413,14 +424,13 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         };
         auto vload = [&](int slot, int grp, int buf) { vload_rows(slot, v_lds(buf) + grp * 16 * L::V_PITCH); };
 
-        // ---- one 64-key tile for this wave's 32 queries ---------------------------------------------------
-        // General form: any mix of rows, one 32-key sub-tile at a time (few live registers; a sub-tile outside
-        // every span of the wave is skipped, which for a short window is one in four).
-        // One 32-key sub-tile in general form: accumulators of K.Q^T in, weights and V^T.P^T out.  ksp: the sub-tile's
-        // 32 key scales in LDS; vrows: its 32 widened V rows in LDS; key0: the index of its first key.
-        auto sub_tile = [&](auto interior_tag, const typename Qk::acc_t &acc, const float *ksp, const uint8_t *vrows, int key0) {
-            constexpr bool INTERIOR = decltype(interior_tag)::value;
-            // key of register r: key0 + 8*(r/4) + 4*g + r%4
+        // ---- one 32-key sub-tile: weights from the accumulators of K.Q^T, then V^T.P^T ---------------------------
+        // ksp: the sub-tile's 32 key scales in LDS; vrows: its 32 widened V rows in LDS; key0: its first key.
+        // Key of accumulator register r: key0 + 8*(r/4) + 4*g + r%4.
+        //
+        // Weights, general form: any mix of rows; exact maximum, and the reference maximum is raised (accumulators
+        // rescaled) when a logit is more than the threshold above it.
+        auto weights_general = [&](const typename Qk::acc_t &acc, const float *ksp, int key0, v2h (&pp)[8], float &s0, float &s1) __attribute__((always_inline)) {
             const int rel_a = sp_a - key0 - 4 * g;           // span start relative to this lane's first key
             const unsigned span_w = (unsigned)(sp_b - sp_a); // in-span <=> (unsigned)(off - rel_a) <= span_w
             const bool has_keys = sp_b >= sp_a;
@@ -428,8 +438,8 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             float t[16];
             float tmax = -INFINITY;
             const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
-            vload_rows(0, vrows);
-            vload_rows(1, vrows + 16 * L::V_PITCH);
+            float bias = base; // base + slope * off, advanced key by key
+            const float slope5 = p.slope * 5.0f;
 #pragma unroll
             for (int c4 = 0; c4 < 4; ++c4) {
                 v4f ksv = *(const v4f *)(ksp + 8 * c4 + 4 * g);
@@ -437,22 +447,21 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                 for (int j = 0; j < 4; ++j) {
                     const int r = c4 * 4 + j;
                     const int off = 8 * c4 + j;
-                    const bool in_span = INTERIOR || ((unsigned)(off - rel_a) <= span_w && has_keys);
+                    const bool in_span = (unsigned)(off - rel_a) <= span_w && has_keys;
                     if (DUMP) {
                         if (in_span) {
                             ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + key0 + off + 4 * g] = Qk::bits(acc, r);
                         }
                     }
                     float x = Qk::to_float(acc, r) * ksv[j];
-                    float tv = fmaf(x, qs, base);
-                    if (SLOPE) tv += p.slope * (float)off;
-                    if (!INTERIOR) tv = in_span ? tv : -INFINITY;
+                    float tv = fmaf(x, qs, bias);
+                    if (SLOPE) bias += (j == 3) ? slope5 : p.slope;
+                    tv = in_span ? tv : -INFINITY;
                     t[r] = tv;
                     tmax = fmaxf(tmax, tv);
                 }
             }
-            // the two lanes of a query exchange their maxima only if some lane of the wave is over the
-            // threshold: the common case has no cross-lane operation at all
+            // the two lanes of a query exchange their maxima only if some lane of the wave is over the threshold
             if (__any(tmax > PF_RESCALE_THRESHOLD)) {
                 tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
                 const float shift = (tmax > PF_RESCALE_THRESHOLD) ? tmax : 0.0f;
@@ -465,19 +474,74 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
 #pragma unroll
                 for (int r = 0; r < 16; ++r) t[r] -= shift;
             }
-            // P = 2^t ; O^T += V^T . P^T in two groups of DT MFMAs (16 keys each)
+            s0 = 0.0f;
+            s1 = 0.0f;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+                const float p0 = fast_exp2(t[2 * x]);
+                const float p1 = fast_exp2(t[2 * x + 1]);
+                pp[x] = v2h{(_Float16)p0, (_Float16)p1};
+                s0 += p0;
+                s1 += p1;
+            }
+        };
+        // Weights with fewer instructions for the usual edge cases: every row of the wave has keys and at most one
+        // end of the spans cuts through the sub-tile (LOW: some span starts after its first key; HIGH: some span
+        // ends before its last).  No maximum is computed; a masked weight is zeroed after the exponential (one
+        // compare against a per-lane bound and one select).  The caller checks the weight sum.
+        auto weights_quick = [&](auto low_tag, auto high_tag, const typename Qk::acc_t &acc, const float *ksp, int key0, v2h (&pp)[8], float &s0, float &s1) __attribute__((always_inline)) {
+            constexpr bool LOW = decltype(low_tag)::value, HIGH = decltype(high_tag)::value;
+            const int lo = sp_a - key0 - 4 * g, hi = sp_b - key0 - 4 * g; // in span <=> lo <= off <= hi
+            const float dist0 = (float)(from - key0 - 4 * g);
+            const float base = SLOPE ? -(p.slope * dist0) - m_ref : -m_ref;
+            s0 = 0.0f;
+            s1 = 0.0f;
+            float bias = base; // base + slope * off, advanced key by key (no per-key constants in registers)
+            const float slope5 = p.slope * 5.0f;
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) {
+                const v4f ksv = *(const v4f *)(ksp + 8 * c4 + 4 * g);
+                float w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int off = 8 * c4 + j;
+                    const float tv = fmaf(Qk::to_float(acc, c4 * 4 + j) * ksv[j], qs, bias);
+                    if (SLOPE) bias += (j == 3) ? slope5 : p.slope;
+                    float pw = fast_exp2(tv);
+                    if (LOW) pw = (lo <= off) ? pw : 0.0f;
+                    if (HIGH) pw = (hi >= off) ? pw : 0.0f;
+                    w[j] = pw;
+                }
+                s0 += w[0];
+                s1 += w[1];
+                s0 += w[2];
+                s1 += w[3];
+                pp[2 * c4] = v2h{(_Float16)w[0], (_Float16)w[1]};
+                pp[2 * c4 + 1] = v2h{(_Float16)w[2], (_Float16)w[3]};
+            }
+        };
+        // The form is chosen by what the wave's spans do inside [key0, key0 + 31]; the matrix part is common.
+        auto sub_tile = [&](const typename Qk::acc_t &acc, const float *ksp, const uint8_t *vrows, int key0) __attribute__((always_inline)) {
+            constexpr float SUM_LIMIT = 256.0f; // = 2^PF_RESCALE_THRESHOLD: one weight above it is enough
+            vload_rows(0, vrows);
+            vload_rows(1, vrows + 16 * L::V_PITCH);
+            v2h pp[8];
+            float s0 = 0.0f, s1 = 0.0f;
+            const bool low = w_max_a > key0, high = w_min_b < key0 + 31;
+            bool general = DUMP || !w_all_have_keys || (low && high);
+            if (!general) {
+                if (low) weights_quick(std::true_type{}, std::false_type{}, acc, ksp, key0, pp, s0, s1);
+                else if (high) weights_quick(std::false_type{}, std::true_type{}, acc, ksp, key0, pp, s0, s1);
+                else weights_quick(std::false_type{}, std::false_type{}, acc, ksp, key0, pp, s0, s1);
+                general = __any(!(s0 + s1 <= SUM_LIMIT)); // a logit far above the reference (or an overflowed sum)
+            }
+            if (general) weights_general(acc, ksp, key0, pp, s0, s1);
+            l += s0;
+            l2 += s1;
+            // O^T += V^T . P^T in two groups of DT MFMAs (16 keys each)
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                v2h pp[4];
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const float p0 = fast_exp2(t[8 * i + 2 * x]);
-                    const float p1 = fast_exp2(t[8 * i + 2 * x + 1]);
-                    pp[x] = v2h{(_Float16)p0, (_Float16)p1};
-                    l += p0;
-                    l2 += p1;
-                }
-                const v8h pb = v8h{pp[0][0], pp[0][1], pp[1][0], pp[1][1], pp[2][0], pp[2][1], pp[3][0], pp[3][1]};
+                const v8h pb = v8h{pp[4 * i][0], pp[4 * i][1], pp[4 * i + 1][0], pp[4 * i + 1][1], pp[4 * i + 2][0], pp[4 * i + 2][1], pp[4 * i + 3][0], pp[4 * i + 3][1]};
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[i][dt], pb, o_acc[dt], 0, 0, 0);
             }
@@ -486,13 +550,12 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         // ---- one 64-key tile for this wave's 32 queries ---------------------------------------------------
         // General form: any mix of rows, one 32-key sub-tile at a time (few live registers; a sub-tile outside
         // every span of the wave is skipped, which for a short window is one in four).
-        auto compute_tile = [&](auto interior_tag, int buf, int kb) {
-            constexpr bool INTERIOR = decltype(interior_tag)::value;
+        auto compute_tile = [&](int buf, int kb) __attribute__((always_inline)) {
 #pragma unroll
             for (int kt = 0; kt < PF_KT; ++kt) {
-                if (!INTERIOR && (kb + kt * 32 + 31 < w_min_a || kb + kt * 32 > w_max_b)) continue;
+                if (kb + kt * 32 + 31 < w_min_a || kb + kt * 32 > w_max_b) continue;
                 const typename Qk::acc_t acc = qk.mma(k_lds(buf) + (kt * 32 + qi) * L::K_PITCH, g);
-                sub_tile(interior_tag, acc, ks_lds(buf) + kt * 32, v_lds(buf) + kt * 32 * L::V_PITCH, kb + kt * 32);
+                sub_tile(acc, ks_lds(buf) + kt * 32, v_lds(buf) + kt * 32 * L::V_PITCH, kb + kt * 32);
             }
         };
 
@@ -507,7 +570,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         // on the slow path with a raised reference.
         constexpr float PF_SUM_LIMIT = 256.0f; // = 2^PF_RESCALE_THRESHOLD: one weight above it is enough to exceed it
         // weights of four keys (accumulator registers 4*c4 .. 4*c4+3)
-        auto weights_quarter = [&](const typename Qk::acc_t &acc, int c4, v4f ksv, float nbase, v2h &pa, v2h &pb, float &s0, float &s1) {
+        auto weights_quarter = [&](const typename Qk::acc_t &acc, int c4, v4f ksv, float nbase, v2h &pa, v2h &pb, float &s0, float &s1) __attribute__((always_inline)) {
             const int r = 4 * c4;
             const float p0 = fast_exp2(fmaf(Qk::to_float(acc, r) * ksv[0], qs, nbase));
             const float p1 = fast_exp2(fmaf(Qk::to_float(acc, r + 1) * ksv[1], qs, nbase));
@@ -520,7 +583,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             pa = v2h{(_Float16)p0, (_Float16)p1};
             pb = v2h{(_Float16)p2, (_Float16)p3};
         };
-        auto weights_sub_rescale = [&](const typename Qk::acc_t &acc, const float *ksp, v8h &pa, v8h &pb, float &s0, float &s1) {
+        auto weights_sub_rescale = [&](const typename Qk::acc_t &acc, const float *ksp, v8h &pa, v8h &pb, float &s0, float &s1) __attribute__((always_inline)) {
             float xs[16];
             float tmax = -INFINITY;
 #pragma unroll
@@ -550,7 +613,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             pb = v8h{pp[4][0], pp[4][1], pp[5][0], pp[5][1], pp[6][0], pp[6][1], pp[7][0], pp[7][1]};
         };
 #define PF_FENCE __builtin_amdgcn_sched_barrier(0)
-        auto fast_tile = [&](int buf) {
+        auto fast_tile = [&](int buf) __attribute__((always_inline)) {
             static_assert(PF_KT == 2, "the common-tile path is written for 64-key tiles");
             constexpr int QS = Qk::STEPS;
             const uint8_t *kr0 = k_lds(buf) + qi * L::K_PITCH, *kr1 = kr0 + 32 * L::K_PITCH;
@@ -639,6 +702,79 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
         };
 #undef PF_FENCE
 
+        // ---- short key ranges: no tile loop ------------------------------------------------------------------
+        // When the whole workgroup needs at most PF_SHORT_KEYS keys (a short window, or the first rows of a
+        // sequence) everything is requested at once: the V rows and key scales of the range (widened into LDS by
+        // all threads) and each wave's K operands (straight into registers: a key's row slice is exactly what the
+        // MFMA operand of that lane holds).  One round trip to memory and one barrier instead of one per tile.
+        bool short_done = false;
+        if constexpr (HAS_SHORT) {
+            if (n_tiles * PF_BN <= PF_SHORT_KEYS) {
+                short_done = true;
+                const int n_keys = n_tiles * PF_BN;
+                uint8_t *const v_short = lds_raw;
+                float *const ks_short = (float *)(lds_raw + PF_SHORT_KEYS * L::V_PITCH);
+                constexpr int NSH = PF_SHORT_KEYS * CHUNKS / PF_THREADS;
+                static_assert(PF_SHORT_KEYS * CHUNKS % PF_THREADS == 0 && PF_SHORT_KEYS <= PF_THREADS, "short range layout");
+                v4i svv[NSH];
+                float svs[NSH], sks = 0.0f;
+#pragma unroll
+                for (int i = 0; i < NSH; ++i) {
+                    const int ch = tid + i * PF_THREADS;
+                    const int r = ch / CHUNKS, c = ch % CHUNKS;
+                    svv[i] = v4i{0, 0, 0, 0};
+                    svs[i] = 0.0f;
+                    if (r < n_keys) {
+                        svv[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(vr, r * (int)p.v_pitch + c * 16, 0, 0));
+                        svs[i] = vs_ptr ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(vsr, r * 4, 0, 0)) : p.vs_const;
+                    }
+                }
+                if (tid < n_keys) sks = ks_ptr ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ksr, tid * 4, 0, 0)) : p.ks_const;
+                // this wave's 32-key sub-tiles: [s_lo, s_hi] (empty if none of its rows has keys)
+                const int s_lo = __builtin_amdgcn_readfirstlane(max(0, (w_min_a - kb_first) >> 5));
+                const int s_hi = __builtin_amdgcn_readfirstlane(min(n_keys / 32 - 1, (w_max_b - kb_first) >> 5));
+                constexpr int QS = Qk::STEPS;
+                constexpr int KREG = 3; // sub-tiles whose K operands are requested up front
+                typename Qk::kop_t kk[KREG][QS];
+#pragma unroll
+                for (int j = 0; j < KREG; ++j) {
+                    if (s_lo + j <= s_hi) {
+#pragma unroll
+                        for (int st = 0; st < QS; ++st) kk[j][st] = Qk::load_k_global(kr, ((s_lo + j) * 32 + qi) * (int)p.k_pitch, g, st);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < NSH; ++i) {
+                    const int ch = tid + i * PF_THREADS;
+                    const int r = ch / CHUNKS, c = ch % CHUNKS;
+                    if (r < n_keys) {
+                        v8h lo, hi;
+                        widen_v<DTYPE>(svv[i], svs[i], lo, hi);
+                        *(v8h *)(v_short + r * L::V_PITCH + c * 32) = lo;
+                        *(v8h *)(v_short + r * L::V_PITCH + c * 32 + 16) = hi;
+                    }
+                }
+                if (tid < n_keys) ks_short[tid] = sks * ads;
+                __syncthreads();
+#pragma unroll 1
+                for (int j = 0; s_lo + j <= s_hi; ++j) {
+                    const int sub = s_lo + j;
+                    typename Qk::kop_t kop[QS];
+#pragma unroll
+                    for (int st = 0; st < QS; ++st) { // the operands requested up front, or (long ranges) fetched now
+                        if (j == 0) kop[st] = kk[0][st];
+                        else if (j == 1) kop[st] = kk[1][st];
+                        else if (j == 2) kop[st] = kk[2][st];
+                        else kop[st] = Qk::load_k_global(kr, (sub * 32 + qi) * (int)p.k_pitch, g, st);
+                    }
+                    typename Qk::acc_t acc = {0};
+#pragma unroll
+                    for (int st = 0; st < QS; ++st) acc = qk.step(kop[st], st, acc);
+                    sub_tile(acc, ks_short + 32 * sub, v_short + 32 * sub * L::V_PITCH, kb_first + 32 * sub);
+                }
+            }
+        }
+        if (!short_done) {
         load_tile();
         store_tile(0);
         if (n_tiles > 1) load_tile();
@@ -662,12 +798,8 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
             for (; it < end; ++it) {
                 const int buf = it & 1;
                 const int kb = kb_first + it * PF_BN;
-                // does this wave need the tile at all, and does it need the per-element mask?
-                if (!(kb + PF_BN - 1 < w_min_a || kb > w_max_b)) {
-                    const bool interior = w_all_have_keys && (kb >= w_max_a) && (kb + PF_BN - 1 <= w_min_b);
-                    if (interior) compute_tile(std::true_type{}, buf, kb);
-                    else compute_tile(std::false_type{}, buf, kb);
-                }
+                // does this wave need the tile at all?
+                if (!(kb + PF_BN - 1 < w_min_a || kb > w_max_b)) compute_tile(buf, kb);
                 if (it + 1 < n_tiles) store_tile(buf ^ 1);
                 if (it + 2 < n_tiles) load_tile();
                 __syncthreads();
@@ -682,6 +814,7 @@ __global__ __launch_bounds__(PF_THREADS, TSATTN_PF_OCC) void prefill_kernel(Pref
                 }
             }
         }
+        } // tile loop
     }
 
     // ---- epilogue: add the zero vector's weight, normalise, store -----------------------------------
