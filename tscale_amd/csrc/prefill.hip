@@ -198,6 +198,8 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
     constexpr int LOOP_BYTES = 2 * L::K_BYTES + 2 * L::V_BYTES + 2 * PF_BN * 4;
     constexpr int SHORT_BYTES = PF_SHORT_KEYS * L::V_PITCH + PF_SHORT_KEYS * 4;
     constexpr bool HAS_SHORT = (D == 64) && !DUMP;
+    // the common-tile loop with ALiBi only where it fits into the registers without spilling
+    constexpr bool FAST_LOOP = !DUMP && (!SLOPE || (D == 128 && DTYPE == TSATTN_E4M3));
     constexpr int LDS_BYTES = (HAS_SHORT && SHORT_BYTES > LOOP_BYTES) ? SHORT_BYTES : LOOP_BYTES;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
     auto k_lds = [&](int b) -> uint8_t * { return lds_raw + b * L::K_BYTES; };
@@ -559,7 +561,7 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             }
         };
 
-        // ---- the common tile: every key inside every span of the wave, no ALiBi ------------------------
+        // ---- the common tile: every key inside every span of the wave ------------------------------------
         // Written so that matrix and vector instructions alternate in the instruction stream (a wave issues
         // in order: vector work placed between two MFMAs runs while the first one executes):
         //   block 1: K.Q^T of both 32-key sub-tiles; the weights of sub-tile 0 overlap the MFMAs of sub-tile 1
@@ -570,12 +572,21 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
         // on the slow path with a raised reference.
         constexpr float PF_SUM_LIMIT = 256.0f; // = 2^PF_RESCALE_THRESHOLD: one weight above it is enough to exceed it
         // weights of four keys (accumulator registers 4*c4 .. 4*c4+3)
-        auto weights_quarter = [&](const typename Qk::acc_t &acc, int c4, v4f ksv, float nbase, v2h &pa, v2h &pb, float &s0, float &s1) __attribute__((always_inline)) {
+        // nbase: minus the reference maximum plus, with ALiBi, the term of the quarter's first key; advanced here
+        // to the next quarter's first key (+8 keys)
+        auto weights_quarter = [&](const typename Qk::acc_t &acc, int c4, v4f ksv, float &nbase, v2h &pa, v2h &pb, float &s0, float &s1) __attribute__((always_inline)) {
             const int r = 4 * c4;
+            float b1 = nbase, b2 = nbase, b3 = nbase;
+            if (SLOPE) {
+                b1 = nbase + p.slope;
+                b2 = b1 + p.slope;
+                b3 = b2 + p.slope;
+            }
             const float p0 = fast_exp2(fmaf(Qk::to_float(acc, r) * ksv[0], qs, nbase));
-            const float p1 = fast_exp2(fmaf(Qk::to_float(acc, r + 1) * ksv[1], qs, nbase));
-            const float p2 = fast_exp2(fmaf(Qk::to_float(acc, r + 2) * ksv[2], qs, nbase));
-            const float p3 = fast_exp2(fmaf(Qk::to_float(acc, r + 3) * ksv[3], qs, nbase));
+            const float p1 = fast_exp2(fmaf(Qk::to_float(acc, r + 1) * ksv[1], qs, b1));
+            const float p2 = fast_exp2(fmaf(Qk::to_float(acc, r + 2) * ksv[2], qs, b2));
+            const float p3 = fast_exp2(fmaf(Qk::to_float(acc, r + 3) * ksv[3], qs, b3));
+            if (SLOPE) nbase = b3 + 5.0f * p.slope;
             s0 += p0;
             s1 += p1;
             s0 += p2;
@@ -583,12 +594,13 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             pa = v2h{(_Float16)p0, (_Float16)p1};
             pb = v2h{(_Float16)p2, (_Float16)p3};
         };
-        auto weights_sub_rescale = [&](const typename Qk::acc_t &acc, const float *ksp, v8h &pa, v8h &pb, float &s0, float &s1) __attribute__((always_inline)) {
+        auto weights_sub_rescale = [&](const typename Qk::acc_t &acc, const float *ksp, float bias0, v8h &pa, v8h &pb, float &s0, float &s1) __attribute__((always_inline)) {
             float xs[16];
             float tmax = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                xs[r] = fmaf(Qk::to_float(acc, r) * ksp[8 * (r / 4) + (r & 3)], qs, -m_ref);
+                const float bias = SLOPE ? bias0 + p.slope * (float)(8 * (r / 4) + (r & 3)) : bias0;
+                xs[r] = fmaf(Qk::to_float(acc, r) * ksp[8 * (r / 4) + (r & 3)], qs, bias);
                 tmax = fmaxf(tmax, xs[r]);
             }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
@@ -613,7 +625,7 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             pb = v8h{pp[4][0], pp[4][1], pp[5][0], pp[5][1], pp[6][0], pp[6][1], pp[7][0], pp[7][1]};
         };
 #define PF_FENCE __builtin_amdgcn_sched_barrier(0)
-        auto fast_tile = [&](int buf) __attribute__((always_inline)) {
+        auto fast_tile = [&](int buf, int kb) __attribute__((always_inline)) {
             static_assert(PF_KT == 2, "the common-tile path is written for 64-key tiles");
             constexpr int QS = Qk::STEPS;
             const uint8_t *kr0 = k_lds(buf) + qi * L::K_PITCH, *kr1 = kr0 + 32 * L::K_PITCH;
@@ -637,7 +649,10 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             PF_FENCE;
             v2h pp0[8], pp1[8];
             float s0 = 0.0f, s1 = 0.0f;
-            const float nbase = -m_ref;
+            // ALiBi: -slope * (from - key), key of register r = kb + 8*(r/4) + 4*g + r%4 (+32 in sub-tile 1)
+            const float alibi0 = SLOPE ? -(p.slope * (float)(from - kb - 4 * g)) : 0.0f;
+            const float bias00 = alibi0 - m_ref;
+            float nbase = bias00;
 #pragma unroll
             for (int c4 = 0; c4 < 4; ++c4) {
                 weights_quarter(acc0, c4, ksv[c4], nbase, pp0[2 * c4], pp0[2 * c4 + 1], s0, s1);
@@ -649,7 +664,7 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             }
             v8h p0a = v8h{pp0[0][0], pp0[0][1], pp0[1][0], pp0[1][1], pp0[2][0], pp0[2][1], pp0[3][0], pp0[3][1]};
             v8h p0b = v8h{pp0[4][0], pp0[4][1], pp0[5][0], pp0[5][1], pp0[6][0], pp0[6][1], pp0[7][0], pp0[7][1]};
-            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc0, ksp, p0a, p0b, s0, s1);
+            if (__any(!(s0 + s1 <= PF_SUM_LIMIT))) weights_sub_rescale(acc0, ksp, bias00, p0a, p0b, s0, s1);
             l += s0;
             l2 += s1;
             // ---- block 2: V^T.P^T of sub-tile 0; sub-tile 1's weights between the MFMAs ----
@@ -657,7 +672,8 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             for (int c4 = 0; c4 < 4; ++c4) ksv[c4] = *(const v4f *)(ksp + 32 + 8 * c4);
             s0 = 0.0f;
             s1 = 0.0f;
-            const float nbase1 = -m_ref;
+            const float bias10 = alibi0 + (SLOPE ? 32.0f * p.slope : 0.0f) - m_ref; // m_ref may have been raised above
+            float nbase1 = bias10;
             PF_FENCE;
 #pragma unroll
             for (int c4 = 0; c4 < 4; ++c4) {
@@ -674,7 +690,7 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             vload(1, 3, buf);
             v8h p1a = v8h{pp1[0][0], pp1[0][1], pp1[1][0], pp1[1][1], pp1[2][0], pp1[2][1], pp1[3][0], pp1[3][1]};
             v8h p1b = v8h{pp1[4][0], pp1[4][1], pp1[5][0], pp1[5][1], pp1[6][0], pp1[6][1], pp1[7][0], pp1[7][1]};
-            if (__any(s0 + s1 > PF_SUM_LIMIT)) weights_sub_rescale(acc1, ksp + 32, p1a, p1b, s0, s1);
+            if (__any(!(s0 + s1 <= PF_SUM_LIMIT))) weights_sub_rescale(acc1, ksp + 32, bias10, p1a, p1b, s0, s1);
             l += s0;
             l2 += s1;
             // ---- block 3: V^T.P^T of sub-tile 1; the next tile's staging between the MFMAs ----
@@ -783,7 +799,7 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
         // inside (the diagonal), not needed.  The fully-inside run [f0, f1) takes the common-tile path (never
         // the last tile of the workgroup, which has no successor to stage); everything else the general one.
         int f0 = n_tiles, f1 = n_tiles;
-        if (!SLOPE && !DUMP && w_all_have_keys) {
+        if (FAST_LOOP && w_all_have_keys) {
             f0 = max(0, (w_max_a - kb_first + PF_BN - 1) / PF_BN);
             f1 = min(n_tiles - 1, (w_min_b + 1 - kb_first) / PF_BN); // tiles [.., f1) end at or before the smallest span end
             if (f1 < f0) f1 = f0;
@@ -804,10 +820,10 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
                 if (it + 2 < n_tiles) load_tile();
                 __syncthreads();
             }
-            if constexpr (!SLOPE && !DUMP) {
+            if constexpr (FAST_LOOP) {
                 if (pass == 0) {
                     for (; it < f1; ++it) {
-                        fast_tile(it & 1);
+                        fast_tile(it & 1, kb_first + it * PF_BN);
                         if (it + 2 < n_tiles) load_tile();
                         __syncthreads();
                     }
