@@ -276,3 +276,65 @@ def test_prefill_layout_variants(ctx, dtype, d, H, n, window):
         torch.cuda.synchronize()
         assert_within_tolerance(out.cpu().numpy(), want, f"layout variant (summary {use_summary})")
         assert (out_buf[:, H * d:] == -7.0).all(), "wrote outside the rows"
+
+
+@pytest.mark.parametrize("dtype,d,H,seq_lens,period", [
+    (capi.E4M3, 64, 12, [100], 0),        # one query tile, six head pairs: every division of the launch mapping is by 1
+    (capi.I8, 128, 5, [128], 0),          # one query tile, five heads
+    (capi.I8, 128, 8, [1024], 1024),      # one sequence with a usable period: one unit per XCD, groups of one unit
+    (capi.E4M3, 64, 16, [1024], 1024),    # the same with paired heads
+    (capi.E4M3, 128, 8, [256, 256], 256), # two sequences, two query tiles each
+])
+def test_prefill_launch_mapping_with_unit_divisors(ctx, dtype, d, H, seq_lens, period):
+    """Launch shapes in which the workgroup -> (head, query tile) mapping divides by 1 somewhere."""
+    n = sum(seq_lens)
+    q, qs, k, ks, v, vs = make_qkv(11 * H + d, n, H, d, dtype)
+    st, fi = orc.make_spans(seq_lens, 10 ** 6)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, 0.0)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    out = ctx.compute_val_lookup(dtype, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), 0.0, causal_period=period)
+    torch.cuda.synchronize()
+    assert_within_tolerance(out.cpu().numpy(), want, "unit divisors")
+
+
+@pytest.mark.parametrize("dtype,d,H,n,window", [
+    (capi.E4M3, 64, 2, 333, 10 ** 6),    # long key range (tile loop): the last 64-key tile ends 51 rows past the end
+    (capi.E4M3, 128, 2, 200, 10 ** 6),
+    (capi.I8, 64, 2, 150, 64),           # short key range path
+    (capi.I8, 128, 3, 333, 100),
+])
+def test_prefill_ignores_what_lies_past_the_last_token(ctx, dtype, d, H, n, window):
+    """Key tiles are 64 rows, so the last one usually reaches past n_tokens.  Whatever lies there (here: NaN scales
+    and 0xff bytes, the e4m3 NaN) must not reach the output: 0 * NaN is NaN, so a masked weight does not hide it."""
+    q, qs, k, ks, v, vs = make_qkv(5 * d + n, n, H, d, dtype)
+    st, fi = orc.make_spans([n], window)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, 0.125)
+    extra = 130
+    def rows(a):
+        t = torch.full((n + extra, H * d), 0xff, dtype=torch.uint8, device="cuda")
+        t[:n] = torch.from_numpy(a).cuda()
+        return t
+    def scales(a):
+        t = torch.full((H, n + extra), float("nan"), dtype=torch.float32, device="cuda")
+        t[:, :n] = torch.from_numpy(a).cuda()
+        return t
+    import ctypes
+    qq, kk, vv = rows(q), rows(k), rows(v)
+    sq, sk, sv = scales(qs), scales(ks), scales(vs)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    st_d, fi_d = t(st), t(fi)
+    out = torch.zeros((n, H * d), dtype=torch.float32, device="cuda")
+    a = capi.PrefillArgs()
+    a.dtype, a.out_dtype = dtype, capi.OUT_F32
+    a.n_tokens, a.n_heads, a.head_dim = n, H, d
+    a.q, a.k, a.v = qq.data_ptr(), kk.data_ptr(), vv.data_ptr()
+    a.q_pitch = a.k_pitch = a.v_pitch = H * d
+    a.q_scale, a.k_scale, a.v_scale, a.scale_pitch = sq.data_ptr(), sk.data_ptr(), sv.data_ptr(), n + extra
+    a.span_start, a.span_finish = st_d.data_ptr(), fi_d.data_ptr()
+    a.alibi_slope = 0.125
+    a.out, a.out_pitch = out.data_ptr(), H * d * 4
+    capi.check(ctx.lib.tsattn_prefill(ctx.handle, ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.isfinite(got).all(), "rows past the last token reached the output"
+    assert_within_tolerance(got, want, "rows past the end")

@@ -1,9 +1,13 @@
 """CPU: host-side logic of the package that needs no device."""
+import os
+
 import numpy as np
 import pytest
 
 from oracle import pyoracle as orc
 from tscale_amd.attention import alibi_layer_schedule
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 @pytest.mark.parametrize("wide", [1024, 4096])
@@ -23,3 +27,14 @@ def test_layer_schedule_of_the_documented_models():
     # 24 layers: two leading pairs of width 1, ten alternating pairs
     sched = alibi_layer_schedule(24, 2048)
     assert [w for w, _ in sched].count(1) == 4 and [w for w, _ in sched].count(64) == 10 and len(sched) == 24
+
+
+def test_prefill_workgroup_mapping_visits_every_head_and_tile_once(tmp_path):
+    """tests/cpp/test_wg_map.cpp walks the launch mapping of tscale_amd/csrc/wg_map.h (the code the kernel runs) over
+    ~1500 launch shapes on the CPU, divisors of 1 (one query tile, one sequence, one unit per group) included."""
+    import subprocess
+    exe = tmp_path / "test_wg_map"
+    subprocess.run(["g++", "-O2", "-std=c++17", "-o", str(exe), os.path.join(ROOT, "tests", "cpp", "test_wg_map.cpp")], check=True)
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert r.stdout.startswith("OK")

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "wg_map.h"
+
 namespace tsattn {
 
 struct DecodeParams {
@@ -55,13 +57,7 @@ struct PrefillParams {
     int n_tokens;
     int n_heads;
     int period_tiles; // query tiles per period of equal span structure, 0 = unknown (launch order only)
-    // Set by the launcher: how workgroup ids map to (head, query tile).  Divisors come with their reciprocals
-    // (ceil(2^32 / d)) so that the kernel divides with one multiply-high.
-    struct Div { uint32_t d, m; };
-    int period_group;  // units per group of the period-aware launch order, 0 = not used
-    int units_per_xcd; // R of the period-aware order
-    int hg_shift;      // log2 of heads that share a cache line (d = 64 with an even head count: 1)
-    Div by_qtiles, by_group_wgs, by_group_units, by_seqs;
+    WgMap map;        // set by the launcher: how workgroup ids map to (head, query tile)
 };
 
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int head_dim, int out_dtype, hipStream_t st);

@@ -212,56 +212,21 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
     const int wave = tid / WAVE;
     const int qi = lane & 31; // query column of this lane
     const int g = lane >> 5;  // which half of the contraction this lane feeds
-    // Workgroups are handed to the 8 XCDs round-robin; give each XCD a contiguous run of
-    // (head, query tile) pairs: equal work per XCD, and the K/V rows a run shares stay in its L2.
     // Ask for every kernel argument the prologue needs in one go: left to itself the compiler fetches them where
     // they are first used, which chains five scalar-load round trips in front of the first K/V request.
 #define PF_TOUCH(x) asm volatile("" ::"s"(x))
     PF_TOUCH(p.q); PF_TOUCH(p.k); PF_TOUCH(p.v); PF_TOUCH(p.q_pitch); PF_TOUCH(p.k_pitch); PF_TOUCH(p.v_pitch);
     PF_TOUCH(p.qs); PF_TOUCH(p.ks); PF_TOUCH(p.vs); PF_TOUCH(p.scale_pitch); PF_TOUCH(p.span_start); PF_TOUCH(p.span_finish);
     PF_TOUCH(p.span_tiles); PF_TOUCH(p.n_tokens); PF_TOUCH(p.n_heads); PF_TOUCH(p.k_global_scale);
-    PF_TOUCH(p.period_tiles); PF_TOUCH(p.period_group); PF_TOUCH(p.units_per_xcd); PF_TOUCH(p.hg_shift);
-    PF_TOUCH(p.by_qtiles.d); PF_TOUCH(p.by_qtiles.m); PF_TOUCH(p.by_group_wgs.d); PF_TOUCH(p.by_group_wgs.m);
-    PF_TOUCH(p.by_group_units.d); PF_TOUCH(p.by_group_units.m); PF_TOUCH(p.by_seqs.d); PF_TOUCH(p.by_seqs.m);
+    PF_TOUCH(p.map.period_tiles); PF_TOUCH(p.map.period_group); PF_TOUCH(p.map.units_per_xcd); PF_TOUCH(p.map.hg_shift);
+    PF_TOUCH(p.map.by_qtiles.d); PF_TOUCH(p.map.by_qtiles.m); PF_TOUCH(p.map.by_group_wgs.d); PF_TOUCH(p.map.by_group_wgs.m);
+    PF_TOUCH(p.map.by_group_units.d); PF_TOUCH(p.map.by_group_units.m); PF_TOUCH(p.map.by_seqs.d); PF_TOUCH(p.map.by_seqs.m);
     PF_TOUCH(p.qs_const); PF_TOUCH(p.ks_const); PF_TOUCH(p.vs_const); PF_TOUCH(p.slope); PF_TOUCH(p.out); PF_TOUCH(p.out_pitch);
 #undef PF_TOUCH
-    int wg = blockIdx.x;
-    const int n_wg = gridDim.x;
-    if ((n_wg & 7) == 0) wg = (wg & 7) * (n_wg >> 3) + (wg >> 3);
-    // With d = 64 one 128-byte line of K or V holds the rows of two heads: consecutive workgroups then
-    // alternate between the two heads of a pair on the same query tile, so the pair shares the line in L2.
-    // All divisions are by launch constants whose reciprocals the host has prepared.
-    auto divmod = [](uint32_t x, PrefillParams::Div by, uint32_t &rem) {
-        uint32_t q = __umulhi(x, by.m);
-        int32_t r = (int32_t)(x - q * by.d);
-        if (r < 0) { --q; r += (int32_t)by.d; }
-        if (r >= (int32_t)by.d) { ++q; r -= (int32_t)by.d; }
-        rem = (uint32_t)r;
-        return q;
-    };
-    const int hs = p.hg_shift, hg = 1 << hs;
+    // which (head, query tile) this workgroup computes: divisions by launch constants whose reciprocals the host
+    // has prepared
     int head, tile;
-    if (p.period_group > 0) {
-        // The caller has said that the batch repeats the same span structure every T query tiles (equal-length
-        // sequences, causal): each XCD still gets a contiguous run of (head, sequence) units, but walks groups of
-        // G units position by position from the end of the sequences to their start: the longest rows of every
-        // unit first, the shortest last, so the launch does not end on a few long-running workgroups.  G is
-        // chosen by the host so that the K/V rows of a group fit in the XCD's L2.
-        const int T = p.period_tiles, G = p.period_group;
-        const uint32_t x = blockIdx.x & 7, i = blockIdx.x >> 3; // XCD and index inside its run
-        uint32_t j, rem, seq;
-        const uint32_t grp = divmod(i, p.by_group_wgs, j);          // / (G * T * hg)
-        const uint32_t pos_rank = divmod(j, p.by_group_units, rem); // / (G * hg)
-        const uint32_t U = x * p.units_per_xcd + grp * G + (rem >> hs);
-        const uint32_t hgrp = divmod(U, p.by_seqs, seq);            // / (n_qtiles / T)
-        head = (int)((hgrp << hs) + (rem & (hg - 1)));
-        tile = (int)(seq * T + (T - 1 - pos_rank));
-    } else {
-        uint32_t t;
-        const uint32_t hgrp = divmod((uint32_t)wg >> hs, p.by_qtiles, t);
-        head = (int)((hgrp << hs) + (wg & (hg - 1)));
-        tile = n_qtiles - 1 - (int)t; // long rows first
-    }
+    wg_locate(p.map, blockIdx.x, gridDim.x, n_qtiles, head, tile);
     const int q0 = tile * PF_BM + wave * 32;
     const int from = q0 + qi;
     const bool row_ok = from < p.n_tokens;
@@ -335,9 +300,10 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
         const int n_tiles = __builtin_amdgcn_readfirstlane((b_max_b - kb_first) / PF_BN + 1);
 
         // ---- staging: global -> registers -> LDS (K as is; V widened to f16 * row scale) -----------------
-        // Loads go through buffer descriptors whose base (a scalar) advances by one tile per load, so the
+        // Loads go through buffer descriptors plus a scalar byte offset that advances by one tile per load, so the
         // per-lane offsets are loop constants and no vector address arithmetic is left in the loop.  A
-        // descriptor ends at the last token's row: rows past it read as zeros (their logits are masked).
+        // descriptor ends at the last token's row: rows past it read as zeros (their logits are masked); on this
+        // hardware generation the range check counts the scalar offset too.
         v4i rk[NLD], rv[NLD];
         float rvs[NLD], rks = 0.0f;
         int k_voff[NLD], v_voff[NLD];
@@ -865,38 +831,8 @@ static void launch_prefill_do(const PrefillParams &p_in, dim3 grid2, hipStream_t
 {
     const int n_qtiles = (int)grid2.x;
     dim3 grid(grid2.x * grid2.y);
-    // Launch-order hint: usable only if every XCD's share of the grid is a whole number of (head group, sequence)
-    // units; units are then walked in groups whose K and V rows (2 * period * d bytes per head) stay within
-    // about the size of the XCD's 4 MB L2 (the rows are streamed, so slightly more than it still pays).
     PrefillParams p = p_in;
-    auto make_div = [](uint32_t d) {
-        PrefillParams::Div r;
-        r.d = d ? d : 1;
-        r.m = (uint32_t)(((1ull << 32) + r.d - 1) / r.d);
-        return r;
-    };
-    p.period_group = 0;
-    p.units_per_xcd = 0;
-    const int hg = (D == 64 && (p.n_heads & 1) == 0) ? 2 : 1;
-    p.hg_shift = hg == 2 ? 1 : 0;
-    p.by_qtiles = make_div((uint32_t)n_qtiles);
-    p.by_group_wgs = p.by_group_units = p.by_seqs = make_div(1);
-    {
-        const int T = p.period_tiles;
-        const int n_wg = (int)grid.x, per_xcd = n_wg / 8;
-        if (T > 1 && n_wg % 8 == 0 && per_xcd % (T * hg) == 0 && n_qtiles % T == 0) {
-            const int R = per_xcd / (T * hg);
-            const int64_t unit_bytes = (int64_t)2 * T * PF_BM * D * hg;
-            int G = 1;
-            for (int c = 1; c <= R; ++c)
-                if (R % c == 0 && c * unit_bytes <= (5 << 20)) G = c;
-            p.period_group = G;
-            p.units_per_xcd = R;
-            p.by_group_wgs = make_div((uint32_t)(G * T * hg));
-            p.by_group_units = make_div((uint32_t)(G * hg));
-            p.by_seqs = make_div((uint32_t)(n_qtiles / T));
-        }
-    }
+    p.map = wg_plan(n_qtiles, p.n_heads, D, PF_BM, p.period_tiles);
     const bool dump = p.dbg != nullptr;
     const bool slope = p.slope != 0.0f;
     dim3 block(PF_THREADS);
