@@ -141,9 +141,10 @@ typedef struct tsattn_decode_args {
     void *debug_qk_acc;        /* optional [n_seqs][n_heads][debug_pitch] int32 / f32 */
     int64_t debug_pitch;
     /* Optional fused append.  With k_new non-NULL the call does what tsattn_cache_append followed by tsattn_decode
-     * would do with the same arguments (kvCache.AddVectors then ComputeValLookup, cpu_infer.cpp:506-509), in two
-     * launches instead of four: cache_len is then the length BEFORE the append and is updated by the call, and
-     * the caches, scale planes and cache_len must be writable.  Not available with window == 0 (the token would
+     * would do with the same arguments (kvCache.AddVectors then ComputeValLookup, cpu_infer.cpp:506-509), in one
+     * launch (one split: short windows) or two instead of three or four: cache_len is then the length BEFORE the
+     * append and is updated by the call, and the caches, scale planes and cache_len must be writable.  Such calls
+     * use counters in the handle: calls on one handle must not overlap on the device (one stream, or ordered).  Not available with window == 0 (the token would
      * attend to the row being written): make the two calls then. */
     const void *k_new, *v_new; /* [n_seqs][n_heads*head_dim] 8-bit */
     int64_t new_pitch;         /* bytes per sequence, multiple of 16 */

@@ -70,4 +70,4 @@ def test_scratch_bytes_is_a_pure_host_function():
     lib = capi.load()
     cfg = capi.Config(0, 64, 16, 128, 32)
     n = lib.tsattn_scratch_bytes(ctypes.byref(cfg))
-    assert n == 64 * 16 * 32 * (128 + 2) * 4
+    assert n == 64 * 16 * 32 * (128 + 2) * 4 + 64 * 4   # split partials + per-sequence arrival counters

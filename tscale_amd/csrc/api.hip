@@ -13,6 +13,7 @@ struct tsattn_ctx {
     int max_seqs, max_heads, max_head_dim, max_splits;
     float *part_acc;
     float *part_ml;
+    int32_t *seq_done;
 };
 
 namespace {
@@ -53,7 +54,7 @@ size_t tsattn_scratch_bytes(const tsattn_config *cfg)
 {
     if (!cfg || cfg->max_seqs < 0 || cfg->max_heads < 0 || cfg->max_head_dim < 0) return 0;
     size_t parts = (size_t)cfg->max_seqs * cfg->max_heads * cfg_splits(cfg);
-    return parts * ((size_t)cfg->max_head_dim + 2) * sizeof(float);
+    return parts * ((size_t)cfg->max_head_dim + 2) * sizeof(float) + (size_t)cfg->max_seqs * sizeof(int32_t);
 }
 
 int tsattn_create(const tsattn_config *cfg, tsattn_handle_t *out)
@@ -77,12 +78,25 @@ int tsattn_create(const tsattn_config *cfg, tsattn_handle_t *out)
     c->max_splits = cfg_splits(cfg);
     c->part_acc = nullptr;
     c->part_ml = nullptr;
+    c->seq_done = nullptr;
     size_t parts = (size_t)c->max_seqs * c->max_heads * c->max_splits;
     if (parts > 0 && c->max_head_dim > 0) {
         e = hipMalloc((void **)&c->part_acc, parts * c->max_head_dim * sizeof(float));
         if (e != hipSuccess) { delete c; return hip_fail(e, "hipMalloc(split partials)"); }
         e = hipMalloc((void **)&c->part_ml, parts * 2 * sizeof(float));
         if (e != hipSuccess) { (void)hipFree(c->part_acc); delete c; return hip_fail(e, "hipMalloc(split max/sum)"); }
+    }
+    if (c->max_seqs > 0) {
+        // arrival counters of the single-split fused append: zero here, and left at zero by every launch
+        e = hipMalloc((void **)&c->seq_done, (size_t)c->max_seqs * sizeof(int32_t));
+        if (e == hipSuccess) e = hipMemset(c->seq_done, 0, (size_t)c->max_seqs * sizeof(int32_t));
+        if (e != hipSuccess) {
+            if (c->seq_done) (void)hipFree(c->seq_done);
+            if (c->part_acc) (void)hipFree(c->part_acc);
+            if (c->part_ml) (void)hipFree(c->part_ml);
+            delete c;
+            return hip_fail(e, "hipMalloc(arrival counters)");
+        }
     }
     *out = c;
     return TSATTN_OK;
@@ -93,6 +107,7 @@ int tsattn_destroy(tsattn_handle_t h)
     if (!h) return TSATTN_OK;
     if (h->part_acc) (void)hipFree(h->part_acc);
     if (h->part_ml) (void)hipFree(h->part_ml);
+    if (h->seq_done) (void)hipFree(h->seq_done);
     delete h;
     return TSATTN_OK;
 }
@@ -186,6 +201,7 @@ int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
     p.k_new = (const uint8_t *)a->k_new; p.v_new = (const uint8_t *)a->v_new; p.new_pitch = a->new_pitch;
     p.ks_new = a->k_scale_new; p.vs_new = a->v_scale_new;
     p.cache_len_rw = const_cast<int32_t *>(a->cache_len); p.max_len = a->max_len;
+    p.seq_done = h->seq_done;
     if (a->k_new || a->v_new) {
         if (!a->k_new || !a->v_new) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: fused append needs both k_new and v_new");
         if (a->window == 0) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: fused append is not available with window 0; call tsattn_cache_append first");

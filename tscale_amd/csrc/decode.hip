@@ -160,7 +160,21 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
             }
         }
     }
-    const bool direct = p.n_splits == 1 && !p.k_new; // no merge kernel follows: this workgroup writes the output
+    const bool direct = p.n_splits == 1; // no merge kernel follows: this workgroup writes the output
+    // A single-split launch with a fused append has no merge kernel to count the new row either: every workgroup
+    // of a sequence (one per head) reports when it is done with the old length, and the last to report adds one.
+    // (The counter is back at zero when the launch ends; launches that share a handle must not overlap.)
+    auto report_done = [&]() {
+        if (tid == 0) {
+            const int done = atomicAdd(&p.seq_done[seq], 1);
+            if (done == p.n_heads - 1) {
+                p.seq_done[seq] = 0;
+                const int len = p.cache_len_rw[seq];
+                if (len >= 0 && len < p.max_len) p.cache_len_rw[seq] = len + 1;
+            }
+        }
+    };
+    const bool count_row = direct && p.k_new != nullptr;
     int lo, n;
     if (cur < 0) {
         lo = 0; n = 0;
@@ -180,6 +194,10 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
     if (s0 >= s1) { // nothing to do: neutral partial (max 0, sum 0, zeros)
         if (direct) {
             if (tid < D) p.out[((int64_t)seq * p.n_heads + head) * D + tid] = 0.0f;
+            if (count_row) {
+                __syncthreads(); // every thread has read the old length
+                report_done();
+            }
             return;
         }
         if (tid < D) p.part_acc[part * D + tid] = 0.0f;
@@ -317,6 +335,7 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
             if (tid == 0) { p.part_ml[part * 2] = M; p.part_ml[part * 2 + 1] = L; }
         }
     }
+    if (count_row) report_done(); // after the barrier above: every thread has read the old length
 }
 
 // out = sum_s acc_s 2^(m_s - M) / (2^-M + sum_s l_s 2^(m_s - M)),  M = max(0, max_s m_s)
@@ -367,7 +386,7 @@ hipError_t launch_decode(const DecodeParams &p, int dtype, int head_dim, bool qb
     else return hipErrorInvalidValue;
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    if (p.n_splits == 1 && !p.k_new) return hipSuccess; // the split kernel wrote the output itself
+    if (p.n_splits == 1) return hipSuccess; // the split kernel wrote the output (and counted a fused append's row) itself
     dim3 mgrid((unsigned)(n_seqs * p.n_heads));
     int32_t *bump = p.k_new ? p.cache_len_rw : nullptr;
     if (head_dim == 128) hipLaunchKernelGGL((decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p.part_acc, p.part_ml, p.n_splits, out, bump, p.n_heads, p.max_len);

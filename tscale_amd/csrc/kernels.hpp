@@ -35,6 +35,7 @@ struct DecodeParams {
     const float *ks_new, *vs_new;
     int32_t *cache_len_rw;
     int max_len;
+    int32_t *seq_done; // [n_seqs] arrival counters of the single-split fused append, zero between launches
 };
 
 hipError_t launch_decode(const DecodeParams &p, int dtype, int head_dim, bool qbf16, int n_seqs, float *out, hipStream_t st);
