@@ -271,6 +271,107 @@ def bench_kv_product(ctx, steps):
             "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4), "bytes": nbytes}
 
 
+def bench_matmul(ctx, steps):
+    """The combiner product of the 1.5B-style configuration (kv [rows][16 heads x 128 x 4] int8 times the combiner
+    matrix [2048][8192] int8, added to the f32 state): once for the prompt batch (32 x 2048 rows: matrix cores),
+    once for one generated token per sequence (32 rows: each layer's matrix is read from HBM once per token; 24
+    layers' matrices in turn, launched as one HIP graph like the generation loop)."""
+    import torch
+    from tscale_amd import capi
+    k, n, depth = 16 * 128 * 4, 2048, 24
+    g = torch.Generator(device="cuda").manual_seed(1313 + 8)
+    ws = [torch.randint(0, 256, (n, k), dtype=torch.uint8, device="cuda", generator=g) for _ in range(depth)]
+    res = {"config": "combiner: int8 [rows][8192] x int8 [2048][8192]^T, f32 state += sums * scale"}
+    m = 32 * 2048
+    a = torch.randint(0, 256, (m, k), dtype=torch.uint8, device="cuda", generator=g)
+    state = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    ms = gpu_time_ms(lambda: ctx.matmul_i8(a, ws[0], mode=capi.MM_ADD_SCALED, scale=1e-6, out=state), max(3, steps // 10), 2)
+    ops = 2.0 * m * n * k
+    res["prompt"] = {"rows": m, "ms": round(ms, 4), "TOP/s": round(ops / ms / 1e9, 2), "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_I8_TOPS, 4)}
+    del a, state
+    m = 32
+    a = torch.randint(0, 256, (m, k), dtype=torch.uint8, device="cuda", generator=g)
+    state = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    room = torch.empty(16 * 4 * m * n, dtype=torch.uint8, device="cuda")   # split-K partial sums
+    def step():
+        for w in ws:
+            ctx.matmul_i8(a, w, mode=capi.MM_ADD_SCALED, scale=1e-6, out=state, workspace=room)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    ms = gpu_time_ms(graph.replay, steps, 2) / depth
+    nbytes = m * k + n * k + 2 * m * n * 4
+    res["token"] = {"rows": m, "us_per_layer": round(ms * 1e3, 2), "GB/s": round(nbytes / ms / 1e6, 1),
+                    "frac_of_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4), "bytes": nbytes,
+                    "launch": "HIP graph of 24 layers' products, K split with a workspace"}
+    return res
+
+
+def bench_token_step(ctx, steps):
+    """One generated token per sequence through all 24 layers of the int8 inference path (AddLookupProduct,
+    gpt/train/cpu_infer.cpp:465-527, per layer: state normalisation, four projections, RoPE + per-head normalisation,
+    cache append + attention over the cache, KVProduct, combiner, feed-forward), B32 at cache length 2048+, model width
+    2048, 16 heads x 128, random int8 weights.  Embedding, final layer and sampling are not part of it."""
+    import torch
+    from tscale_amd import KVCache, capi
+    from tscale_amd.attention import add_lookup_product, alibi_layer_schedule, VEC_SCALE
+    B, H, d, dim, depth, prompt, n_new = 32, 16, 128, 2048, 24, 2048, 64
+    L = prompt + n_new
+    qsum = H * d
+    g = torch.Generator(device="cuda").manual_seed(1313 + 9)
+    def matrix(n, k):   # int8 of rms 32, what the reference's matrix conversion leaves (MODEL_DISCR_SCALE = 1/32)
+        return (torch.randn((n, k), device="cuda", generator=g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
+    sched = alibi_layer_schedule(depth, L)
+    layers, caches = [], []
+    for w, slope in sched:
+        layers.append({"qk": matrix(qsum, dim), "qv": matrix(qsum, dim), "k": matrix(qsum, dim), "v": matrix(qsum, dim),
+                       "combiner": matrix(dim, qsum * 4), "expand": matrix(qsum, dim), "contract": matrix(dim, qsum),
+                       "qv_scale": 0.03, "combiner_scale": 0.03, "contract_scale": 0.03, "width": w, "slope": slope})
+        c = KVCache(ctx, capi.I8, B, H, L, d)
+        c.k.copy_(torch.randint(0, 256, c.k.shape, dtype=torch.uint8, device="cuda", generator=g))
+        c.v.copy_(torch.randint(0, 256, c.v.shape, dtype=torch.uint8, device="cuda", generator=g))
+        c.k_scale.copy_((torch.rand(c.k_scale.shape, device="cuda", generator=g) + 0.5) * 1e-4)
+        c.v_scale.fill_(VEC_SCALE)
+        c.cache_len.fill_(prompt)
+        caches.append(c)
+    rope = ctx.fill_rope_table(d, L)
+    state = torch.randn((B, dim), device="cuda", generator=g)
+    t = torch.full((B,), prompt, dtype=torch.int32, device="cuda")
+    room = torch.empty(16 * 4 * B * max(dim, qsum), dtype=torch.uint8, device="cuda")
+    def step():
+        for layer, c in zip(layers, caches):
+            add_lookup_product(ctx, layer, c, t, rope, state, workspace=room)
+        t.add_(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    torch.cuda.synchronize()
+    reps = min(n_new - 2, max(10, steps))
+    ms = gpu_time_ms(graph.replay, reps, 0)
+    assert bool(torch.isfinite(state).all())
+    weight_bytes = sum(sum(v.numel() for v in layer.values() if isinstance(v, torch.Tensor)) for layer in layers)
+    n = prompt + 1 + reps // 2
+    cache_bytes = sum(B * H * min(n - 1, w) * (2 * d + 8) for w, _ in sched)
+    return {"config": "24 layers, B32, cache length ~2048+, model width 2048, 16 heads x 128, int8 weights and KV cache; "
+                      "13 launches per layer in one HIP graph per token",
+            "ms_per_token_step": round(ms, 4), "tokens_per_s": round(B / ms * 1e3, 1),
+            "weight_bytes": weight_bytes, "cache_bytes_per_step": cache_bytes,
+            "GB/s": round((weight_bytes + cache_bytes) / ms / 1e6, 1),
+            "frac_of_hbm_peak": round((weight_bytes + cache_bytes) / ms / 1e6 / PEAK_HBM_GBPS, 4)}
+
+
 def cpu_baseline_prefill(wl, n_seq_sample):
     """The oracle (a port of the reference's CPU attention) on the same quantised inputs: the first
     `n_seq_sample` sequences of every layer of the pass, all host threads; plus one sequence of one
@@ -346,6 +447,12 @@ def run_only(ctx, args):
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
+    if name == "token-step":
+        print(json.dumps({"only": name, **bench_token_step(ctx, args.steps)}))
+        return
+    if name == "matmul":
+        print(json.dumps({"only": name, **bench_matmul(ctx, args.steps)}))
+        return
     if name == "producer":
         print(json.dumps({"only": name, **bench_producer(ctx, args.steps * 5)}))
         return
@@ -377,7 +484,7 @@ def main():
     ap.add_argument("--extra", action="store_true",
                     help="also time the 1.5B-style prefill shapes and the attention share of the 1.5B-style generation run")
     ap.add_argument("--only", default=None,
-                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer"],
+                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step"],
                     help="profiling aid: run just this launch --steps times and print its timing")
     ap.add_argument("--calibrate", action="store_true",
                     help="with --only: first run three 256 MiB device copies (counter calibration)")
@@ -462,6 +569,8 @@ def main():
         result["producer"] = bench_producer(ctx, args.steps)
         torch.cuda.empty_cache()
         result["kv_product"] = bench_kv_product(ctx, args.steps)
+        result["combiner_matmul"] = bench_matmul(ctx, args.steps)
+        result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
     print(json.dumps(result))
 
 

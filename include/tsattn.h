@@ -230,6 +230,13 @@ typedef struct tsattn_produce_args {
     int64_t dst_pitch;         /* bytes per row, multiple of 16 */
     float *scale;              /* [n_heads][scale_pitch] or NULL */
     int64_t scale_pitch;
+    /* Element (head, row) of scale is scale[head * scale_pitch + row * scale_row_stride]; 0 means 1 (planes
+     * [n_heads][scale_pitch], what tsattn_prefill reads).  scale_pitch = 1 with scale_row_stride = n_heads gives
+     * [n_rows][n_heads], what tsattn_cache_append and the fused append of tsattn_decode read. */
+    int64_t scale_row_stride;
+    /* Non-zero: negative results become 0 after the conversion, the ReLU of the reference's int8 feed-forward
+     * block (gpt/train/cpu_infer.cpp:520-524).  int8 only. */
+    int relu;
 } tsattn_produce_args;
 
 int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, void *stream);
@@ -243,6 +250,37 @@ int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, 
 int tsattn_kv_product(tsattn_handle_t h, int64_t n_rows, int n_heads, int head_dim, int rep, const void *k, int64_t k_pitch,
                       int value_dtype, const void *value, int64_t value_pitch, float mult, void *kv, int64_t kv_pitch,
                       void *stream);
+
+/* int8 matrix product of the reference's int8 inference path: out[m][n] (op)= sum_k a[m][k] * w[n][k], exact in
+ * int32.  Replaces MulForward, gpt/train/cpu_infer.cpp:294-305 (one weight row per output; calls :481-488, :513,
+ * :519, :525, :558: the four projections, the combiner, the two FFN matrices, the final layer) and, with
+ * TSATTN_MM_ADD_SCALED, the AddScaled that follows the combiner and the FFN (:308-316, calls :514, :526).
+ * a: int8 [m][k], w: int8 [n][k], pitches in bytes; k a positive multiple of 64 (DotInt8 asks the same, :184-210);
+ * out: [m][n], pitch in elements; pointers and byte pitches multiples of 16, out 4-byte aligned. */
+enum tsattn_mm_mode {
+    TSATTN_MM_I32 = 0,        /* out (int32) = sum */
+    TSATTN_MM_F32 = 1,        /* out (f32) = (float)sum * scale   (MulForward into TVector<float>: scale 1) */
+    TSATTN_MM_ADD_SCALED = 2, /* out (f32) += (float)sum * scale  (AddScaled) */
+};
+
+typedef struct tsattn_matmul_args {
+    int64_t m, n, k;
+    const void *a;
+    int64_t a_pitch;
+    const void *w;
+    int64_t w_pitch;
+    int mode;                  /* tsattn_mm_mode */
+    float scale;
+    void *out;
+    int64_t out_pitch;
+    /* Optional scratch of the caller's (16-byte aligned): with at most 128 rows the weights are streamed once and K
+     * is split over more workgroups if there is room for the parts' sums (2 x 4 x m x n bytes or more; 16 x 4 x m x n
+     * is never exceeded).  The result is the same with and without it. */
+    void *workspace;
+    int64_t workspace_bytes;
+} tsattn_matmul_args;
+
+int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *stream);
 
 /* The table ApplyRope reads: FillRopeBuf, gpt/att/rope.cpp:4-24.  Host function, host memory:
  * table[t * head_dim + x], t < max_len; copy it to the device once. */

@@ -193,6 +193,59 @@ def kv_product(k, val, n_heads, rep=4, mult=1.0):
     return kv
 
 
+def matmul_i8(a, w, mode=0, scale=1.0, out=None):
+    """a: int8 [m, k], w: int8 [n, k] -> [m, n]: int32 sums (mode 0), float32 sums * scale (1), out += sums * scale (2)."""
+    L = lib()
+    a = _c_arr(np.asarray(a).view(np.int8), np.int8)
+    w = _c_arr(np.asarray(w).view(np.int8), np.int8)
+    m, k = a.shape
+    n = w.shape[0]
+    assert w.shape[1] == k and k % 64 == 0
+    if mode == 2:
+        out = _c_arr(out, np.float32).copy()
+    else:
+        out = np.empty((m, n), dtype=np.int32 if mode == 0 else np.float32)
+    L.tso_matmul_i8(_p(a), ctypes.c_int64(k), _p(w), ctypes.c_int64(k), ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k),
+                    int(mode), ctypes.c_float(scale), _p(out), ctypes.c_int64(n))
+    return out
+
+
+class LayerParams(ctypes.Structure):
+    _fields_ = [("dim", ctypes.c_int), ("head_count", ctypes.c_int), ("head_dim", ctypes.c_int), ("relu_dim", ctypes.c_int),
+                ("qk", ctypes.c_void_p), ("qv", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+                ("combiner", ctypes.c_void_p), ("expand", ctypes.c_void_p), ("contract", ctypes.c_void_p),
+                ("qv_scale", ctypes.c_float), ("combiner_scale", ctypes.c_float), ("contract_scale", ctypes.c_float),
+                ("attention_width", ctypes.c_int64), ("alibi_slope", ctypes.c_float)]
+
+
+def add_lookup_product(mats, scales, width, slope, head_count, head_dim, t, rope, state, k_cache, v_cache, k_scale_cache, cache_len):
+    """AddLookupProduct (cpu_infer.cpp:465-527) for one token per sequence.  mats: dict of int8 arrays qk, qv, k, v
+    [H*d, dim], combiner [dim, 4*H*d], expand [relu, dim], contract [dim, relu]; scales: (qv, combiner, contract).
+    Caches planar [n_seq, H, max_len, d] (uint8) and [n_seq, H, max_len] (float32), cache_len int32 [n_seq]: all updated
+    in place.  Returns (new state, attention output)."""
+    L = lib()
+    keep = {k: _c_arr(np.asarray(v).view(np.int8), np.int8) for k, v in mats.items()}
+    n_seq, dim = state.shape
+    P = LayerParams()
+    P.dim, P.head_count, P.head_dim, P.relu_dim = dim, head_count, head_dim, keep["expand"].shape[0]
+    for name in ("qk", "qv", "k", "v", "combiner", "expand", "contract"):
+        setattr(P, name, keep[name].ctypes.data)
+    P.qv_scale, P.combiner_scale, P.contract_scale = scales
+    P.attention_width, P.alibi_slope = int(width), float(slope)
+    out = _c_arr(state, np.float32).copy()
+    val = np.zeros((n_seq, head_count * head_dim), dtype=np.float32)
+    t = _c_arr(t, np.int32)
+    rope = _c_arr(rope, np.float32)
+    for a, dt in ((k_cache, np.uint8), (v_cache, np.uint8), (k_scale_cache, np.float32), (cache_len, np.int32)):
+        assert a.dtype == dt and a.flags["C_CONTIGUOUS"]
+    max_len = k_cache.shape[2]
+    L.tso_add_lookup_product(ctypes.byref(P), ctypes.c_int64(n_seq), _p(t), _p(rope), _p(out), _p(k_cache), _p(v_cache),
+                             ctypes.c_int64(head_count * max_len * head_dim), ctypes.c_int64(max_len * head_dim), ctypes.c_int64(head_dim),
+                             _p(k_scale_cache), ctypes.c_int64(head_count * max_len), ctypes.c_int64(max_len), _p(cache_len), int(max_len),
+                             _p(val), 2)
+    return out, val
+
+
 def make_spans(seq_lens, window, doc_start_flag=None):
     L = lib()
     off = np.zeros(len(seq_lens) + 1, dtype=np.int64)

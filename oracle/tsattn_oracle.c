@@ -42,6 +42,16 @@
  *   tso_kv_product         train/cpu_infer.cpp:320-337   pinned: numpy restatement (index shuffle z ^ blk, products,
  *                                                         rounding), blk 0 = plain product, the four blocks are
  *                                                         permutations of each other when value is constant
+ *   tso_matmul_i8          train/cpu_infer.cpp:294-316   pinned: numpy int64 matrix product (a library routine), +-127
+ *                                                         extremes; the scaled forms against the same product in
+ *                                                         float64
+ *   tso_add_lookup_product train/cpu_infer.cpp:465-527   a composition of the functions above in the reference's order;
+ *                                                         pinned as a whole only by invariants (the input state's
+ *                                                         scale does not matter to the attention half, zero combiner and contract matrices
+ *                                                         leave the state alone, the first token sees no keys, the
+ *                                                         update is linear in the two matrix scales): the order of
+ *                                                         the steps and which scale goes where were checked by
+ *                                                         reading -- parity unpinned beyond its parts
  *
  * The reference holds no golden vectors or known-answer tests for this path, and the two files
  * that contain it (gpt_cpu.cpp, cpu_infer.cpp) cannot be compiled without the CUDA SDK, so the
@@ -325,6 +335,30 @@ void tso_kv_product(const int8_t *k, int64_t k_pitch, const float *val, int64_t 
                     float value = val[t * val_pitch + head_offset + z];
                     kv[t * kv_pitch + base + z] = tso_float_to_i8((key_shfl * value) * mult);
                 }
+            }
+        }
+    }
+}
+
+/* MulForward, train/cpu_infer.cpp:294-305: res[n] = DotInt8(vec, w[n]) for every weight row n (exact int32), kept as
+ * int32 (mode 0) or converted to float (mode 1: the TVector<float> instantiation, times `scale`, 1 in the
+ * reference); mode 2 is the AddScaled that follows it (:308-316): out[n] += delta[n] * scale.  One activation row
+ * per token. */
+void tso_matmul_i8(const int8_t *a, int64_t a_pitch, const int8_t *w, int64_t w_pitch, int64_t m, int64_t n, int64_t k, int mode,
+                   float scale, void *out, int64_t out_pitch)
+{
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+    for (int64_t i = 0; i < m; ++i) {
+        for (int64_t j = 0; j < n; ++j) {
+            int32_t sum = tso_dot_i8_simd(a + i * a_pitch, w + j * w_pitch, (int)k);
+            if (mode == 0) {
+                ((int32_t *)out)[i * out_pitch + j] = sum;
+            } else if (mode == 1) {
+                ((float *)out)[i * out_pitch + j] = (float)sum * scale;
+            } else {
+                ((float *)out)[i * out_pitch + j] += (float)sum * scale; /* (*pRes)[k] += delta[k] * scale */
             }
         }
     }
@@ -837,4 +871,74 @@ int tso_max_threads(void)
 #else
     return 1;
 #endif
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* one layer, one token per sequence                                                          */
+
+static const float TSO_VEC_SCALE = 1.0f / 24; /* train/cpu_infer.cpp:16 */
+#define TSO_STATE_NORM_TILE 128               /* model_params/model_dim.h:22 */
+#define TSO_COMBINER_REP 4                    /* model_params/model_dim.h:12 */
+
+void tso_add_lookup_product(const tso_layer_params *L, int64_t n_seq, const int32_t *t, const float *rope, float *state,
+                            uint8_t *k_cache, uint8_t *v_cache, int64_t seq_stride, int64_t head_stride, int64_t tok_stride,
+                            float *k_scale_cache, int64_t s_seq_stride, int64_t s_head_stride, int32_t *cache_len, int max_len,
+                            float *val_lookup, int n_threads)
+{
+    const int dim = L->dim, H = L->head_count, d = L->head_dim, qsum = H * d, kvdim = qsum * TSO_COMBINER_REP, rdim = L->relu_dim;
+    uint8_t *norm = (uint8_t *)malloc((size_t)n_seq * dim);
+    float *qk_src = (float *)malloc(sizeof(float) * (size_t)n_seq * qsum), *qv_src = (float *)malloc(sizeof(float) * (size_t)n_seq * qsum);
+    int32_t *k_src = (int32_t *)malloc(sizeof(int32_t) * (size_t)n_seq * qsum), *v_src = (int32_t *)malloc(sizeof(int32_t) * (size_t)n_seq * qsum);
+    uint8_t *qk = (uint8_t *)malloc((size_t)n_seq * qsum), *qv = (uint8_t *)malloc((size_t)n_seq * qsum);
+    uint8_t *k = (uint8_t *)malloc((size_t)n_seq * qsum), *v = (uint8_t *)malloc((size_t)n_seq * qsum);
+    float *qv_head_scale = (float *)malloc(sizeof(float) * (size_t)n_seq * H); /* [H][n_seq] */
+    float *val = (float *)malloc(sizeof(float) * (size_t)n_seq * qsum);
+    int8_t *kv = (int8_t *)malloc((size_t)n_seq * kvdim);
+    int32_t *relu_src = (int32_t *)malloc(sizeof(int32_t) * (size_t)n_seq * rdim);
+    uint8_t *relu = (uint8_t *)malloc((size_t)n_seq * rdim);
+
+    /* :476-477  NormalizeState(&normState, *pState, dim / STATE_NORM_TILE, nullptr) */
+    tso_rope_normalize_rows(TSO_I8, state, 0, dim, n_seq, NULL, NULL, 1.0f, dim / TSO_STATE_NORM_TILE, TSO_STATE_NORM_TILE, TSO_VEC_SCALE, 1.0f,
+                            norm, dim, NULL, 0);
+    /* :479-486  the four projections: qk and qv into float vectors, k and v into int32 */
+    tso_matmul_i8((const int8_t *)norm, dim, L->qk, dim, n_seq, qsum, dim, 1, 1.0f, qk_src, qsum);
+    tso_matmul_i8((const int8_t *)norm, dim, L->qv, dim, n_seq, qsum, dim, 1, 1.0f, qv_src, qsum);
+    tso_matmul_i8((const int8_t *)norm, dim, L->k, dim, n_seq, qsum, dim, 0, 1.0f, k_src, qsum);
+    tso_matmul_i8((const int8_t *)norm, dim, L->v, dim, n_seq, qsum, dim, 0, 1.0f, v_src, qsum);
+    /* :487-499  rope on qk and qv, per-head normalisation of all four; :501-503 the key scale takes the matrix scale */
+    tso_rope_normalize_rows(TSO_I8, qk_src, 0, qsum, n_seq, t, rope, 1.0f, H, d, TSO_VEC_SCALE, 1.0f, qk, qsum, NULL, 0);
+    const float key_mult = L->qv_scale * TSO_VEC_SCALE * sqrtf(1.0f / (float)dim);
+    tso_rope_normalize_rows(TSO_I8, qv_src, 0, qsum, n_seq, t, rope, 1.0f, H, d, TSO_VEC_SCALE, key_mult, qv, qsum, qv_head_scale, n_seq);
+    tso_rope_normalize_rows(TSO_I8, k_src, 1, qsum, n_seq, NULL, NULL, 1.0f, H, d, TSO_VEC_SCALE, 1.0f, k, qsum, NULL, 0);
+    tso_rope_normalize_rows(TSO_I8, v_src, 1, qsum, n_seq, NULL, NULL, 1.0f, H, d, TSO_VEC_SCALE, 1.0f, v, qsum, NULL, 0);
+    /* :504  kvCache.AddVectors(qv, qvHeadScale, v) */
+    for (int64_t s = 0; s < n_seq; ++s) {
+        int len = cache_len[s];
+        if (len < 0 || len >= max_len) continue;
+        for (int h = 0; h < H; ++h) {
+            memcpy(k_cache + s * seq_stride + h * head_stride + (int64_t)len * tok_stride, qv + s * qsum + h * d, (size_t)d);
+            memcpy(v_cache + s * seq_stride + h * head_stride + (int64_t)len * tok_stride, v + s * qsum + h * d, (size_t)d);
+            k_scale_cache[s * s_seq_stride + h * s_head_stride + len] = qv_head_scale[(int64_t)h * n_seq + s];
+        }
+        cache_len[s] = len + 1;
+    }
+    /* :506-507  ComputeValLookup(att.AttentionWidth, att.AlibiSlope, dims, kvCache, qk, &valLookup) */
+    tso_decode(TSO_I8, n_seq, H, d, qk, NULL, TSO_VEC_SCALE, k_cache, v_cache, seq_stride, head_stride, tok_stride, k_scale_cache, NULL,
+               s_seq_stride, s_head_stride, 0.0f, TSO_VEC_SCALE, cache_len, L->attention_width, L->alibi_slope, 0, 1, val, NULL, 0, n_threads);
+    if (val_lookup) memcpy(val_lookup, val, sizeof(float) * (size_t)n_seq * qsum);
+    /* :509-514  KVProduct, combiner, AddScaled */
+    tso_kv_product((const int8_t *)k, qsum, val, qsum, n_seq, H, d, TSO_COMBINER_REP, 1.0f, kv, kvdim);
+    tso_matmul_i8(kv, kvdim, L->combiner, kvdim, n_seq, dim, kvdim, 2, L->combiner_scale * TSO_VEC_SCALE * sqrtf(1.0f / (float)kvdim), state, dim);
+    /* :516-526  feed-forward: normalise, expand, normalise per head, ReLU, contract, AddScaled */
+    tso_rope_normalize_rows(TSO_I8, state, 0, dim, n_seq, NULL, NULL, 1.0f, dim / TSO_STATE_NORM_TILE, TSO_STATE_NORM_TILE, TSO_VEC_SCALE, 1.0f,
+                            norm, dim, NULL, 0);
+    tso_matmul_i8((const int8_t *)norm, dim, L->expand, dim, n_seq, rdim, dim, 0, 1.0f, relu_src, rdim);
+    tso_rope_normalize_rows(TSO_I8, relu_src, 1, rdim, n_seq, NULL, NULL, 1.0f, H, rdim / H, TSO_VEC_SCALE, 1.0f, relu, rdim, NULL, 0);
+    for (int64_t i = 0; i < n_seq * rdim; ++i) {
+        if ((int8_t)relu[i] < 0) relu[i] = 0; /* x = Max<i8>(0, x) */
+    }
+    tso_matmul_i8((const int8_t *)relu, rdim, L->contract, rdim, n_seq, dim, rdim, 2, L->contract_scale * TSO_VEC_SCALE * sqrtf(1.0f / (float)rdim), state, dim);
+
+    free(norm); free(qk_src); free(qv_src); free(k_src); free(v_src); free(qk); free(qv); free(k); free(v);
+    free(qv_head_scale); free(val); free(kv); free(relu_src); free(relu);
 }

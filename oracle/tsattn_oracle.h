@@ -46,6 +46,8 @@ void tso_rope_normalize_rows(int dtype, const void *src, int src_is_i32, int64_t
                              int64_t scale_pitch);
 void tso_kv_product(const int8_t *k, int64_t k_pitch, const float *val, int64_t val_pitch, int64_t n_rows, int n_heads,
                     int head_dim, int rep, float mult, int8_t *kv, int64_t kv_pitch);
+void tso_matmul_i8(const int8_t *a, int64_t a_pitch, const int8_t *w, int64_t w_pitch, int64_t m, int64_t n, int64_t k, int mode,
+                   float scale, void *out, int64_t out_pitch);
 void tso_quantize_rows_bf16(int dtype, const uint16_t *x, int64_t x_pitch, int64_t n_rows,
                             int n_heads, int head_dim, uint8_t *q, int64_t q_pitch, float *scale,
                             int64_t scale_pitch);
@@ -113,6 +115,29 @@ void tso_decode(int dtype, int64_t n_seq, int n_heads, int head_dim, const uint8
                 float k_scale_const, float v_scale_const, const int32_t *cache_len, int64_t window,
                 float alibi_slope, int exp2_mode, int use_simd, float *out, void *qk_acc,
                 int64_t qk_acc_pitch, int n_threads);
+
+/* ---- one layer of the int8 inference path for one new token per sequence: AddLookupProduct,
+ * train/cpu_infer.cpp:465-527 ----
+ * Matrices are int8 with one row per output (MulForward's kqv[k]); *_scale are the matrix scales ConvertMatrix
+ * returned (:94-121).  head_dim is QDim == TTDim.  state: [n_seq][dim] f32, updated in place.  t[seq]: the token's
+ * position (rope row).  The KV cache is addressed as in tso_decode (key scales only; queries and values carry the
+ * constant VEC_SCALE, :16); cache_len[seq] is the length before the call and is incremented (a full cache drops the
+ * row).  val_lookup (nullable): the attention output [n_seq][head_count*head_dim]. */
+typedef struct tso_layer_params {
+    int dim, head_count, head_dim, relu_dim;
+    const int8_t *qk, *qv, *k, *v;   /* [head_count*head_dim][dim] */
+    const int8_t *combiner;          /* [dim][head_count*head_dim*4] */
+    const int8_t *expand;            /* [relu_dim][dim] */
+    const int8_t *contract;          /* [dim][relu_dim] */
+    float qv_scale, combiner_scale, contract_scale;
+    int64_t attention_width;
+    float alibi_slope;
+} tso_layer_params;
+
+void tso_add_lookup_product(const tso_layer_params *L, int64_t n_seq, const int32_t *t, const float *rope, float *state,
+                            uint8_t *k_cache, uint8_t *v_cache, int64_t seq_stride, int64_t head_stride, int64_t tok_stride,
+                            float *k_scale_cache, int64_t s_seq_stride, int64_t s_head_stride, int32_t *cache_len, int max_len,
+                            float *val_lookup, int n_threads);
 
 /* softmax buffer of cpu_infer.cpp:220-281 on its own (for bounding the polynomial):
  * in: n logits (the caller includes the leading 0 if wanted); out: n weights already multiplied by

@@ -100,3 +100,22 @@ def test_kv_product_bit_exact(ctx, d, H, f16):
         tv = torch.from_numpy(val).cuda()
         got = ctx.kv_product(torch.from_numpy(k.view(np.uint8)).cuda(), tv.half() if f16 else tv, H, mult=mult)
         assert np.array_equal(got.cpu().numpy().view(np.int8), want)
+
+
+def test_producer_relu_and_row_major_scales(ctx):
+    """The two options the int8 layer uses: negative results zeroed after the conversion (cpu_infer.cpp:520-524), and
+    the scales laid out [row][head], the layout the cache append reads."""
+    rng = np.random.default_rng(21)
+    n, H, d = 37, 3, 128
+    x = (rng.standard_normal((n, H * d)) * 1000).astype(np.int32)
+    want_q, want_s = orc.rope_normalize_rows(capi.I8, x, H, scale_mult=0.5)
+    xd = torch.from_numpy(x).cuda()
+    q, s = ctx.rope_normalize_rows(xd, H, capi.I8, scale_mult=0.5, row_major_scale=True, relu=True)
+    torch.cuda.synchronize()
+    want_relu = want_q.view(np.int8).copy()
+    want_relu[want_relu < 0] = 0
+    assert np.array_equal(q.cpu().numpy().view(np.int8), want_relu)
+    assert (want_relu == 0).mean() > 0.4 and (want_relu > 0).any()
+    assert s.shape == (n, H) and np.array_equal(s.cpu().numpy(), want_s.T)
+    with pytest.raises(capi.TsattnError):
+        ctx.rope_normalize_rows(xd, H, capi.E4M3, relu=True)

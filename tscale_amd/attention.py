@@ -9,6 +9,7 @@ arithmetic happens in libtsattn.so.  There is no fallback path: a missing librar
 """
 import ctypes
 
+import numpy as np
 import torch
 
 from . import capi
@@ -91,13 +92,14 @@ class AttentionContext:
         return host.to(self.device)
 
     def rope_normalize_rows(self, x, n_heads, dtype, pos=None, rope=None, rotate_dir=1.0, vec_scale=1.0 / 24,
-                            scale_mult=1.0):
+                            scale_mult=1.0, row_major_scale=False, relu=False):
         """ApplyRope + NormalizeState of the reference's inference path (cpu_infer.cpp:486-499): x [n_rows, H*d]
-        float32 or int32 -> (uint8 [n_rows, H*d], f32 scale [H, n_rows]); pos int32 [n_rows] or None (no rotation)."""
+        float32 or int32 -> (uint8 [n_rows, H*d], f32 scale [H, n_rows], or [n_rows, H] with row_major_scale: what
+        the cache append reads); pos int32 [n_rows] or None (no rotation); relu: negative results become 0 (:520-524)."""
         assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.dtype in (torch.float32, torch.int32)
         n_rows, hd = x.shape
         q = torch.empty((n_rows, hd), dtype=torch.uint8, device=x.device)
-        scale = torch.empty((n_heads, n_rows), dtype=torch.float32, device=x.device)
+        scale = torch.empty((n_rows, n_heads) if row_major_scale else (n_heads, n_rows), dtype=torch.float32, device=x.device)
         a = capi.ProduceArgs()
         a.src_dtype = capi.SRC_F32 if x.dtype == torch.float32 else capi.SRC_I32
         a.dst_dtype = dtype
@@ -107,7 +109,9 @@ class AttentionContext:
         a.rope_len = 0 if rope is None else rope.shape[0]
         a.rotate_dir, a.vec_scale, a.scale_mult = float(rotate_dir), float(vec_scale), float(scale_mult)
         a.dst, a.dst_pitch = _ptr(q), hd
-        a.scale, a.scale_pitch = _ptr(scale), n_rows
+        a.scale, a.scale_pitch = _ptr(scale), (1 if row_major_scale else n_rows)
+        a.scale_row_stride = n_heads if row_major_scale else 1
+        a.relu = int(bool(relu))
         capi.check(self.lib.tsattn_rope_normalize_rows(self.handle, ctypes.byref(a), _stream_ptr()))
         return q, scale
 
@@ -120,6 +124,28 @@ class AttentionContext:
         capi.check(self.lib.tsattn_kv_product(self.handle, n, n_heads, hd // n_heads, rep, _ptr(k), hd, vdt, _ptr(value), hd,
                                               float(mult), _ptr(kv), hd * rep, _stream_ptr()))
         return kv
+
+    def matmul_i8(self, a, w, mode=capi.MM_I32, scale=1.0, out=None, workspace=None):
+        """MulForward / AddScaled (cpu_infer.cpp:294-316): a uint8 (int8 bytes) [m, k], w uint8 [n, k] (one row per
+        output) -> out[m, n]: int32 sums (MM_I32), f32 sums * scale (MM_F32), or out += sums * scale (MM_ADD_SCALED,
+        out given, f32)."""
+        m, k = a.shape
+        n = w.shape[0]
+        assert w.shape[1] == k and a.stride(1) == 1 and w.stride(1) == 1
+        if out is None:
+            assert mode != capi.MM_ADD_SCALED
+            out = torch.empty((m, n), dtype=torch.int32 if mode == capi.MM_I32 else torch.float32, device=a.device)
+        assert out.stride(1) == 1 and out.dtype == (torch.int32 if mode == capi.MM_I32 else torch.float32)
+        args = capi.MatmulArgs()
+        args.m, args.n, args.k = m, n, k
+        args.a, args.a_pitch = _ptr(a), a.stride(0)
+        args.w, args.w_pitch = _ptr(w), w.stride(0)
+        args.mode, args.scale = mode, float(scale)
+        args.out, args.out_pitch = _ptr(out), out.stride(0)
+        if workspace is not None:   # a uint8 tensor the caller keeps: room for split-K partial sums when m is small
+            args.workspace, args.workspace_bytes = _ptr(workspace), workspace.numel() * workspace.element_size()
+        capi.check(self.lib.tsattn_matmul_i8(self.handle, ctypes.byref(args), _stream_ptr()))
+        return out
 
     def build_spans(self, seq_offset, n_tokens, window, doc_start_flag=None):
         """seq_offset: int32 [n_seqs+1] on the device.  Returns (span_start, span_finish) int32 [n_tokens]."""
@@ -206,6 +232,51 @@ class AttentionContext:
             a.k_scale_new, a.v_scale_new = _ptr(ks_new), _ptr(vs_new)
         capi.check(self.lib.tsattn_decode(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
+
+
+VEC_SCALE = 1.0 / 24      # gpt/train/cpu_infer.cpp:16
+STATE_NORM_TILE = 128     # gpt/model_params/model_dim.h:22
+COMBINER_REP = 4          # gpt/model_params/model_dim.h:12
+
+
+def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None):
+    """One layer of the int8 inference path for one new token per sequence: AddLookupProduct,
+    gpt/train/cpu_infer.cpp:465-527, as a chain of library calls (the C++ form is NTsAttn::TLayerComputer).
+    layer: dict with uint8 (int8 bytes) matrices qk, qv, k, v [H*d, dim], combiner [dim, 4*H*d], expand [H*d, dim],
+    contract [dim, H*d], floats qv_scale, combiner_scale, contract_scale, and width, slope.  cache: KVCache whose value
+    scales are VEC_SCALE; t: int32 [B] positions; rope: table of fill_rope_table; state: f32 [B, dim], updated in place.
+    Returns the attention output [B, H*d]."""
+    B, dim = state.shape
+    H, d = cache.n_heads, cache.head_dim
+    qsum = H * d
+    groups = dim // STATE_NORM_TILE
+    norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
+    qk_src = ctx.matmul_i8(norm, layer["qk"], mode=capi.MM_F32, workspace=workspace)
+    qv_src = ctx.matmul_i8(norm, layer["qv"], mode=capi.MM_F32, workspace=workspace)
+    k_src = ctx.matmul_i8(norm, layer["k"], workspace=workspace)
+    v_src = ctx.matmul_i8(norm, layer["v"], workspace=workspace)
+    qk, _ = ctx.rope_normalize_rows(qk_src, H, capi.I8, pos=t, rope=rope)
+    key_mult = float(np.float32(layer["qv_scale"]) * np.float32(VEC_SCALE) * np.float32(np.sqrt(np.float32(1.0) / np.float32(dim))))
+    qv, qv_scale = ctx.rope_normalize_rows(qv_src, H, capi.I8, pos=t, rope=rope, scale_mult=key_mult, row_major_scale=True)
+    k, _ = ctx.rope_normalize_rows(k_src, H, capi.I8)
+    v, _ = ctx.rope_normalize_rows(v_src, H, capi.I8)
+    v_scale = torch.full((B, H), VEC_SCALE, dtype=torch.float32, device=state.device)
+    if layer["width"] == 0:   # the token attends to the row being written: append first
+        cache.add_vectors(qv, qv_scale, v, v_scale)
+        val = ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, 0, layer["slope"])
+    else:
+        val = ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, layer["width"], layer["slope"], append=(qv, qv_scale, v, v_scale))
+    kv = ctx.kv_product(k, val, H, COMBINER_REP)
+    f32 = np.float32
+    ctx.matmul_i8(kv, layer["combiner"], mode=capi.MM_ADD_SCALED, out=state, workspace=workspace,
+                  scale=float(f32(layer["combiner_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(qsum * COMBINER_REP)))))
+    norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
+    relu_src = ctx.matmul_i8(norm, layer["expand"], workspace=workspace)
+    relu, _ = ctx.rope_normalize_rows(relu_src, H, capi.I8, relu=True)
+    relu_dim = relu_src.shape[1]
+    ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state, workspace=workspace,
+                  scale=float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim)))))
+    return val
 
 
 class KVCache:

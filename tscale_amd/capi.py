@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libtsattn.so")
 I8, E4M3 = 0, 1
 OUT_F32, OUT_F16 = 0, 1
 SRC_F32, SRC_BF16, SRC_I32 = 0, 1, 2
+MM_I32, MM_F32, MM_ADD_SCALED = 0, 1, 2
 Q_8BIT, Q_BF16 = 0, 1
 SPAN_TILE_INTS = 32
 
@@ -76,7 +77,15 @@ class ProduceArgs(_c.Structure):
         ("head_dim", _c.c_int), ("src", _c.c_void_p), ("src_pitch", _c.c_int64), ("pos", _c.c_void_p),
         ("rope", _c.c_void_p), ("rope_len", _c.c_int64), ("rotate_dir", _c.c_float), ("vec_scale", _c.c_float),
         ("scale_mult", _c.c_float), ("dst", _c.c_void_p), ("dst_pitch", _c.c_int64), ("scale", _c.c_void_p),
-        ("scale_pitch", _c.c_int64),
+        ("scale_pitch", _c.c_int64), ("scale_row_stride", _c.c_int64), ("relu", _c.c_int),
+    ]
+
+
+class MatmulArgs(_c.Structure):
+    _fields_ = [
+        ("m", _c.c_int64), ("n", _c.c_int64), ("k", _c.c_int64), ("a", _c.c_void_p), ("a_pitch", _c.c_int64),
+        ("w", _c.c_void_p), ("w_pitch", _c.c_int64), ("mode", _c.c_int), ("scale", _c.c_float), ("out", _c.c_void_p),
+        ("out_pitch", _c.c_int64), ("workspace", _c.c_void_p), ("workspace_bytes", _c.c_int64),
     ]
 
 
@@ -93,7 +102,7 @@ class FillArgs(_c.Structure):
 
 
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
+           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
 
 _lib = None
 
@@ -134,6 +143,8 @@ def load():
         L.tsattn_kv_product.restype = _c.c_int
         L.tsattn_kv_product.argtypes = [_c.c_void_p, _c.c_int64, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int,
                                         _c.c_void_p, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64, _c.c_void_p]
+        L.tsattn_matmul_i8.restype = _c.c_int
+        L.tsattn_matmul_i8.argtypes = [_c.c_void_p, _c.POINTER(MatmulArgs), _c.c_void_p]
         L.tsattn_quantize_rows.restype = _c.c_int
         L.tsattn_quantize_rows.argtypes = [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64,
                                            _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64,

@@ -298,12 +298,17 @@ int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, 
     if (a->src_pitch < row || a->dst_pitch < row || a->dst_pitch % 16 || a->src_pitch % 4 || !aligned16(a->dst) || !aligned16(a->src) ||
         (a->rope && !aligned16(a->rope)))
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: pitches must cover a row; src, dst and rope 16-byte aligned, pitches multiples of 16 bytes");
-    if (a->scale && a->scale_pitch < a->n_rows) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale_pitch below n_rows");
+    const int64_t row_stride = a->scale_row_stride ? a->scale_row_stride : 1;
+    if (a->scale && (row_stride < 0 || a->scale_pitch <= 0 ||
+                     !((row_stride == 1 && a->scale_pitch >= a->n_rows) || (a->scale_pitch == 1 && row_stride >= a->n_heads))))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale layout must be [n_heads][scale_pitch >= n_rows] or [n_rows][scale_row_stride >= n_heads]");
+    if (a->relu && a->dst_dtype != TSATTN_I8) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_rope_normalize_rows: relu with an int8 result only");
     tsattn::ProduceParams p;
     p.src = a->src; p.src_pitch = a->src_pitch; p.n_rows = a->n_rows; p.n_heads = a->n_heads;
     p.pos = a->pos; p.rope = a->rope; p.rope_len = a->rope_len;
     p.rotate_dir = a->rotate_dir; p.vec_scale = a->vec_scale; p.scale_mult = a->scale_mult;
     p.dst = (uint8_t *)a->dst; p.dst_pitch = a->dst_pitch; p.scale = a->scale; p.scale_pitch = a->scale_pitch;
+    p.scale_row_stride = row_stride; p.relu = a->relu;
     hipError_t e = tsattn::launch_rope_normalize(p, a->dst_dtype, a->head_dim, a->src_dtype == TSATTN_SRC_I32, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "rope normalize launch");
     return TSATTN_OK;
@@ -330,6 +335,29 @@ int tsattn_kv_product(tsattn_handle_t h, int64_t n_rows, int n_heads, int head_d
     p.n_heads = n_heads; p.head_dim = head_dim; p.rep = rep; p.mult = mult; p.kv = (uint8_t *)kv; p.kv_pitch = kv_pitch;
     hipError_t e = tsattn::launch_kv_product(p, value_dtype == TSATTN_OUT_F16, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "kv product launch");
+    return TSATTN_OK;
+}
+
+int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: null argument");
+    if (a->mode != TSATTN_MM_I32 && a->mode != TSATTN_MM_F32 && a->mode != TSATTN_MM_ADD_SCALED)
+        return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: mode %d", a->mode);
+    if (a->m < 0 || a->n < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: negative size");
+    if (a->k <= 0 || a->k % 64) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: k %lld (a positive multiple of 64)", (long long)a->k);
+    if (a->m == 0 || a->n == 0) return TSATTN_OK;
+    if (!a->a || !a->w || !a->out) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: null data pointer");
+    if (a->a_pitch < a->k || a->w_pitch < a->k || a->out_pitch < a->n || a->a_pitch % 16 || a->w_pitch % 16 || !aligned16(a->a) ||
+        !aligned16(a->w) || (uintptr_t)a->out % 4)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: pitches must cover a row; a, w and their pitches multiples of 16 bytes");
+    if (a->a_pitch > (1 << 24) || a->w_pitch > (1 << 24)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: row pitch above 16 MiB");
+    tsattn::GemmParams p;
+    p.a = (const uint8_t *)a->a; p.w = (const uint8_t *)a->w; p.a_pitch = a->a_pitch; p.w_pitch = a->w_pitch;
+    p.m = a->m; p.n = a->n; p.k = a->k; p.mode = a->mode; p.scale = a->scale; p.out = a->out; p.out_pitch = a->out_pitch;
+    const bool ws_ok = a->workspace && a->workspace_bytes > 0 && aligned16(a->workspace);
+    p.workspace = ws_ok ? a->workspace : nullptr; p.workspace_bytes = ws_ok ? a->workspace_bytes : 0; p.split_stride = 0;
+    hipError_t e = tsattn::launch_matmul_i8(p, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "matmul launch");
     return TSATTN_OK;
 }
 

@@ -1,0 +1,291 @@
+// int8 x int8 -> int32 matrix product with the epilogues of the reference's int8 inference path:
+//   out[m][n] = sum_k a[m][k] * w[n][k]
+// MulForward (gpt/train/cpu_infer.cpp:294-305: one weight row per output, exact int32 sums, result as int32 or
+// converted to float) and AddScaled (:308-316: state += delta * scale).
+//
+// Two kernels.  Many rows (a prompt): 128 x 128 output tiles, K in steps of 64 bytes through LDS, four waves of
+// 64 x 64 each, v_mfma_i32_32x32x32_i8; bound by the matrix cores.  Few rows (one token per sequence): the
+// weights are read once from HBM, 32 weight rows per workgroup with K split over its four waves; bound by HBM.
+// Integer sums are exact, so every decomposition gives the same bits.
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace tsattn {
+
+namespace {
+
+constexpr int GT_THREADS = 256;
+constexpr int GT_BM = 128, GT_BN = 128, GT_BK = 64;
+constexpr int GT_PITCH = GT_BK + 16; // LDS row pitch: 16-lane phases of a 16-byte read hit distinct banks
+
+__device__ inline __amdgpu_buffer_rsrc_t rows_rsrc(const void *base, int64_t rows, int64_t pitch, int64_t row_bytes)
+{
+    // the last row ends after row_bytes, not after a whole pitch
+    int64_t bytes = rows <= 0 ? 0 : (rows - 1) * pitch + row_bytes;
+    const uint32_t n = bytes > 0xffffffffll ? 0xffffffffu : (uint32_t)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+
+template <int MODE>
+__device__ inline void store_out(const GemmParams &p, int64_t m, int64_t n, int acc)
+{
+#pragma clang fp contract(off) // delta * scale is rounded before it is added, as in the reference's two statements
+    if (MODE == TSATTN_MM_I32) {
+        ((int32_t *)p.out)[m * p.out_pitch + n] = acc;
+    } else if (MODE == TSATTN_MM_F32) {
+        ((float *)p.out)[m * p.out_pitch + n] = (float)acc * p.scale;
+    } else {
+        float *o = (float *)p.out + m * p.out_pitch + n;
+        *o += (float)acc * p.scale; // (*pRes)[k] += delta[k] * scale
+    }
+}
+
+// ---- many rows --------------------------------------------------------------------------------------------------
+template <int MODE>
+__global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(GemmParams p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[2][GT_BM * GT_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t w_lds[2][GT_BN * GT_PITCH];
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid / WAVE;
+    const int wm = wave >> 1, wn = wave & 1; // 2 x 2 waves of 64 x 64
+    const int li = lane & 31, g = lane >> 5;
+
+    // Consecutive workgroups walk along a row of output tiles: they share one tile of activations, which is then
+    // read from HBM once; the 8 XCDs take workgroups round-robin, so each keeps every eighth tile of weights in its
+    // own L2 for the whole launch.
+    const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN;
+    const int64_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const int64_t m0 = tile_m * GT_BM, n0 = tile_n * GT_BN;
+
+    const __amdgpu_buffer_rsrc_t ar = rows_rsrc(p.a + m0 * p.a_pitch, p.m - m0 < GT_BM ? p.m - m0 : GT_BM, p.a_pitch, p.k);
+    const __amdgpu_buffer_rsrc_t wr = rows_rsrc(p.w + n0 * p.w_pitch, p.n - n0 < GT_BN ? p.n - n0 : GT_BN, p.w_pitch, p.k);
+    // staging: 128 rows x 64 bytes = 512 chunks of 16 bytes per operand, two per thread
+    int a_off[2], w_off[2], lds_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int ch = tid + i * GT_THREADS;
+        const int r = ch >> 2, c = ch & 3;
+        a_off[i] = r * (int)p.a_pitch + c * 16;
+        w_off[i] = r * (int)p.w_pitch + c * 16;
+        lds_off[i] = r * GT_PITCH + c * 16;
+    }
+    v4i ra[2], rw[2];
+    auto load = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            ra[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[i], kb, 0));
+            rw[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, w_off[i], kb, 0));
+        }
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *(v4i *)(a_lds[buf] + lds_off[i]) = ra[i];
+            *(v4i *)(w_lds[buf] + lds_off[i]) = rw[i];
+        }
+    };
+
+    v16i acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = v16i{0};
+
+    const int n_steps = (int)(p.k / GT_BK);
+    load(0);
+    stage(0);
+    if (n_steps > 1) load(GT_BK);
+    __syncthreads();
+    for (int s = 0; s < n_steps; ++s) {
+        const int buf = s & 1;
+        const uint8_t *ab = a_lds[buf] + (wm * 64 + li) * GT_PITCH + 16 * g;
+        const uint8_t *wb = w_lds[buf] + (wn * 64 + li) * GT_PITCH + 16 * g;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const v4i a0 = *(const v4i *)(ab + 32 * ks), a1 = *(const v4i *)(ab + 32 * GT_PITCH + 32 * ks);
+            const v4i w0 = *(const v4i *)(wb + 32 * ks), w1 = *(const v4i *)(wb + 32 * GT_PITCH + 32 * ks);
+            acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w1, acc[1][1], 0, 0, 0);
+        }
+        if (s + 1 < n_steps) stage(buf ^ 1);
+        if (s + 2 < n_steps) load((s + 2) * GT_BK);
+        __syncthreads();
+    }
+
+    // accumulator register r of tile (i, j): row m0 + wm*64 + i*32 + 8*(r/4) + 4*g + r%4, column n0 + wn*64 + j*32 + li
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int64_t n = n0 + wn * 64 + j * 32 + li;
+            if (n >= p.n) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = m0 + wm * 64 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                if (m < p.m) store_out<MODE>(p, m, n, acc[i][j][r]);
+            }
+        }
+}
+
+// ---- few rows ---------------------------------------------------------------------------------------------------
+// One workgroup per 32 weight rows and part of K.  K is walked in slabs of 1024 bytes: every wave instruction asks
+// for 1 KiB of consecutive memory of one row (the weights are read once, so what matters is that HBM sees long
+// consecutive requests and that many are in flight), the slab goes through LDS, and there the rows are read back the
+// way the MFMA wants them (32 bytes of a row per lane and step).  The four waves each take a quarter of the slab
+// and add their sums up in LDS.
+constexpr int GS_THREADS = 256;
+constexpr int GS_WAVES = GS_THREADS / WAVE;
+constexpr int GS_BN = 32;      // weight rows per workgroup
+constexpr int GS_MB = 4;       // blocks of 32 activation rows handled by this kernel
+constexpr int GS_SLAB = 1024;  // bytes of K per slab
+constexpr int GS_PITCH = GS_SLAB + 16;
+constexpr int GS_LD = 32 * GS_SLAB / 16 / GS_THREADS; // 16-byte chunks per thread and slab: 8
+
+template <int MODE>
+__global__ __launch_bounds__(GS_THREADS) void gemm_skinny_kernel(GemmParams p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t w_lds[32 * GS_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t x_lds[32 * GS_PITCH];
+    static_assert(GS_MB * 16 * WAVE * 4 <= 32 * GS_PITCH, "the waves' sums are added up in the activations' slab");
+    int(*red)[16 * WAVE] = (int(*)[16 * WAVE]) x_lds;
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid / WAVE;
+    const int li = lane & 31, g = lane >> 5;
+    const int64_t n0 = (int64_t)blockIdx.x * GS_BN;
+
+    // this workgroup's part of K (blockIdx.y of gridDim.y parts, in whole steps of 64 bytes); with more than one
+    // part the sums go to this part's plane of the workspace
+    const int all_steps = (int)(p.k / 64);
+    const int split_steps = (all_steps + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int k_begin = (int)blockIdx.y * split_steps * 64, k_end = min(all_steps, ((int)blockIdx.y + 1) * split_steps) * 64;
+    p.out = (uint8_t *)p.out + (int64_t)blockIdx.y * p.split_stride * 4;
+
+    const int n_mb = (int)((p.m + 31) / 32);
+    const __amdgpu_buffer_rsrc_t wr = rows_rsrc(p.w + n0 * p.w_pitch, p.n - n0 < GS_BN ? p.n - n0 : GS_BN, p.w_pitch, p.k);
+    const __amdgpu_buffer_rsrc_t ar = rows_rsrc(p.a, p.m, p.a_pitch, p.k);
+    // chunk i of this thread: row 4*i + wave, bytes 16*lane.. of the slab: one wave instruction = one row's KiB
+    v16i acc[GS_MB];
+#pragma unroll
+    for (int j = 0; j < GS_MB; ++j) acc[j] = v16i{0};
+
+    for (int kb = k_begin; kb < k_end; kb += GS_SLAB) {
+        const int slab = min(GS_SLAB, k_end - kb); // bytes of K in this slab, a multiple of 64
+        const bool in_slab = 16 * lane < slab;
+        v4i rw[GS_LD];
+#pragma unroll
+        for (int i = 0; i < GS_LD; ++i) {
+            const int row = 4 * i + wave;
+            rw[i] = in_slab ? __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, row * (int)p.w_pitch + 16 * lane, kb, 0)) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < GS_MB; ++j) {
+            if (j < n_mb) { // uniform
+                v4i rx[GS_LD];
+#pragma unroll
+                for (int i = 0; i < GS_LD; ++i) {
+                    const int row = 32 * j + 4 * i + wave;
+                    rx[i] = in_slab ? __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, row * (int)p.a_pitch + 16 * lane, kb, 0)) : v4i{0, 0, 0, 0};
+                }
+                __syncthreads(); // the previous block's reads of x_lds (and, for j == 0, of w_lds) are done
+                if (j == 0) {
+#pragma unroll
+                    for (int i = 0; i < GS_LD; ++i) *(v4i *)(w_lds + (4 * i + wave) * GS_PITCH + 16 * lane) = rw[i];
+                }
+#pragma unroll
+                for (int i = 0; i < GS_LD; ++i) *(v4i *)(x_lds + (4 * i + wave) * GS_PITCH + 16 * lane) = rx[i];
+                __syncthreads();
+                // this wave's quarter of the slab: steps 4*wave .. 4*wave+3 (those inside the slab)
+                const uint8_t *wb = w_lds + li * GS_PITCH + 32 * g, *xb = x_lds + li * GS_PITCH + 32 * g;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int off = (4 * wave + u) * 64;
+                    if (off < slab) { // uniform
+                        const v4i w0 = *(const v4i *)(wb + off), w1 = *(const v4i *)(wb + off + 16);
+                        const v4i x0 = *(const v4i *)(xb + off), x1 = *(const v4i *)(xb + off + 16);
+                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w0, x0, acc[j], 0, 0, 0);
+                        acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w1, x1, acc[j], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+    // sum the waves' shares in LDS; register r of block j: weight row n0 + 8*(r/4) + 4*g + r%4, activation row 32*j + li
+    __syncthreads(); // the slab has been read
+    for (int i = tid; i < GS_MB * 16 * WAVE; i += GS_THREADS) (&red[0][0])[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < GS_MB; ++j) {
+        if (j < n_mb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) atomicAdd(&red[j][r * WAVE + lane], acc[j][r]);
+        }
+    }
+    __syncthreads();
+    for (int r = wave; r < 16; r += GS_WAVES) {
+        const int64_t n = n0 + 8 * (r / 4) + 4 * g + (r & 3);
+        for (int j = 0; j < n_mb; ++j) {
+            const int64_t m = 32 * j + li;
+            if (n < p.n && m < p.m) store_out<MODE>(p, m, n, red[j][r * WAVE + lane]);
+        }
+    }
+}
+
+// sums the planes of the workspace and applies the epilogue: one thread per output element
+template <int MODE>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(GemmParams p, const int32_t *ws, int n_split)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= p.m * p.n) return;
+    int sum = 0;
+    for (int s = 0; s < n_split; ++s) sum += ws[s * p.split_stride + i];
+    store_out<MODE>(p, i / p.n, i % p.n, sum);
+}
+
+template <int MODE>
+void launch_mode(const GemmParams &p, hipStream_t st)
+{
+    if (p.m > 32 * GS_MB) {
+        const int64_t tiles = ((p.m + GT_BM - 1) / GT_BM) * ((p.n + GT_BN - 1) / GT_BN);
+        hipLaunchKernelGGL((gemm_tiled_kernel<MODE>), dim3((unsigned)tiles), dim3(GT_THREADS), 0, st, p);
+        return;
+    }
+    // Few rows: the weights are streamed once and every compute unit has to help.  With 32 weight rows per
+    // workgroup there are too few workgroups unless K is split as well, which needs room for the parts' sums.
+    const int64_t n_tiles = (p.n + GS_BN - 1) / GS_BN;
+    int split = 1;
+    while (split < 16 && n_tiles * split < 512 && p.k / (split * 2) >= GS_SLAB &&
+           (int64_t)(split * 2) * p.m * p.n * 4 <= p.workspace_bytes)
+        split *= 2;
+    if (split == 1) {
+        hipLaunchKernelGGL((gemm_skinny_kernel<MODE>), dim3((unsigned)n_tiles, 1), dim3(GS_THREADS), 0, st, p);
+        return;
+    }
+    GemmParams q = p;
+    q.out = p.workspace;
+    q.out_pitch = p.n;
+    q.split_stride = p.m * p.n;
+    hipLaunchKernelGGL((gemm_skinny_kernel<TSATTN_MM_I32>), dim3((unsigned)n_tiles, (unsigned)split), dim3(GS_THREADS), 0, st, q);
+    GemmParams r = p;
+    r.split_stride = p.m * p.n;
+    hipLaunchKernelGGL((gemm_reduce_kernel<MODE>), dim3((unsigned)((p.m * p.n + 255) / 256)), dim3(256), 0, st, r,
+                       (const int32_t *)p.workspace, split);
+}
+
+} // namespace
+
+hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st)
+{
+    if (p.m <= 0 || p.n <= 0) return hipSuccess;
+    if (p.mode == TSATTN_MM_I32) launch_mode<TSATTN_MM_I32>(p, st);
+    else if (p.mode == TSATTN_MM_F32) launch_mode<TSATTN_MM_F32>(p, st);
+    else if (p.mode == TSATTN_MM_ADD_SCALED) launch_mode<TSATTN_MM_ADD_SCALED>(p, st);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+} // namespace tsattn

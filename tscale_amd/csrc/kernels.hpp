@@ -105,7 +105,8 @@ struct ProduceParams {
     uint8_t *dst;
     int64_t dst_pitch;
     float *scale;
-    int64_t scale_pitch;
+    int64_t scale_pitch, scale_row_stride;
+    int relu;
 };
 
 hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head_dim, bool src_i32, hipStream_t st);
@@ -124,6 +125,21 @@ struct KvProductParams {
 };
 
 hipError_t launch_kv_product(const KvProductParams &p, bool val_f16, hipStream_t st);
+
+struct GemmParams {
+    const uint8_t *a, *w;
+    int64_t a_pitch, w_pitch; // bytes
+    int64_t m, n, k;
+    int mode;                 // tsattn_mm_mode
+    float scale;
+    void *out;
+    int64_t out_pitch;        // elements
+    void *workspace;          // optional room for split-K partial sums (few rows)
+    int64_t workspace_bytes;
+    int64_t split_stride;     // set by the launcher: elements between the parts' planes
+};
+
+hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st);
 
 struct FillParams {
     const int32_t *seq_offset;

@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
             mult = 1.0f / discr;
         }
         mults[tid] = mult;
-        if (p.scale) p.scale[s_head[tid] * p.scale_pitch + s_row[tid]] = discr * p.scale_mult;
+        if (p.scale) p.scale[s_head[tid] * p.scale_pitch + s_row[tid] * p.scale_row_stride] = discr * p.scale_mult;
     }
     __syncthreads();
 
@@ -126,7 +126,8 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
             for (int i = 0; i < 4; ++i) {
                 const float y = vals[pr * PITCH + x + 4 * k + i] * mult;
                 // a head of zeros is written as zero bytes whatever the signs of its (rotated) zeros
-                const uint32_t b = mult == 0.0f ? 0u : ((DST == TSATTN_I8) ? (uint8_t)float_to_i8(y) : float_to_e4m3(y));
+                uint32_t b = mult == 0.0f ? 0u : ((DST == TSATTN_I8) ? (uint8_t)float_to_i8(y) : float_to_e4m3(y));
+                if (DST == TSATTN_I8 && p.relu && (b & 0x80u)) b = 0u; // x = max(0, x)
                 w[k] |= b << (8 * i);
             }
         }

@@ -1,6 +1,7 @@
 #include "att_compute.h"
 
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 
@@ -209,6 +210,120 @@ void ComputeValLookup(int width, float alibiSlope, const TAttentionVecHistory &h
     a.alibi_slope = alibiSlope;
     a.out = valLookup;
     Check(tsattn_decode(h.Handle, &a, stream), "tsattn_decode");
+}
+
+// ---- one layer of the int8 inference path ----------------------------------------------------------------------
+
+TLayerComputer::TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, int seqCount)
+    : Handle(handle), Dims(dims), SeqCount(seqCount)
+{
+    TS_VERIFY(dims.QDim == dims.TTDim && (dims.QDim == 64 || dims.QDim == 128), "QDim %d TTDim %d: equal, 64 or 128", dims.QDim, dims.TTDim);
+    TS_VERIFY(dims.Dim % STATE_NORM_TILE == 0, "Dim %d is not a multiple of %d", dims.Dim, STATE_NORM_TILE);
+    ReluDim = dims.HeadCount * dims.QDim;
+    const size_t n = (size_t)seqCount, qsum = (size_t)dims.GetQSum();
+    auto alloc = [](void **p, size_t bytes) { CheckHip(hipMalloc(p, bytes), "hipMalloc(layer buffers)"); };
+    alloc((void **)&NormState, n * dims.Dim);
+    alloc((void **)&Qk, n * qsum); alloc((void **)&Qv, n * qsum); alloc((void **)&K, n * qsum); alloc((void **)&V, n * qsum);
+    alloc((void **)&Kv, n * qsum * COMBINER_REP);
+    alloc((void **)&Relu, n * ReluDim);
+    alloc((void **)&QkSrc, n * qsum * 4); alloc((void **)&QvSrc, n * qsum * 4);
+    alloc((void **)&KSrc, n * qsum * 4); alloc((void **)&VSrc, n * qsum * 4);
+    alloc((void **)&ReluSrc, n * ReluDim * 4);
+    alloc((void **)&QvHeadScale, n * dims.HeadCount * 4); alloc((void **)&VHeadScale, n * dims.HeadCount * 4);
+    alloc((void **)&ValLookup, n * qsum * 4);
+    // room for the matrix products to split K (few rows): 16 planes of the widest result
+    size_t widest = qsum > (size_t)dims.Dim ? qsum : (size_t)dims.Dim;
+    if ((size_t)ReluDim > widest) widest = ReluDim;
+    WorkspaceBytes = (int64_t)(16 * 4 * n * widest);
+    alloc(&Workspace, (size_t)WorkspaceBytes);
+    // values carry the constant VEC_SCALE (cpu_infer.cpp:454)
+    std::vector<float> vs(n * dims.HeadCount, VEC_SCALE);
+    CheckHip(hipMemcpy(VHeadScale, vs.data(), vs.size() * sizeof(float), hipMemcpyHostToDevice), "hipMemcpy(value scales)");
+}
+
+TLayerComputer::~TLayerComputer()
+{
+    void *all[] = {NormState, Qk, Qv, K, V, Kv, Relu, QkSrc, QvSrc, KSrc, VSrc, ReluSrc, QvHeadScale, VHeadScale, ValLookup, Workspace};
+    for (void *p : all) (void)hipFree(p);
+}
+
+void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
+                                      TAttentionVecHistory *pKVCache, float *state, void *stream)
+{
+    TAttentionVecHistory &kvCache = *pKVCache;
+    const int dim = Dims.Dim, headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
+    TS_VERIFY(kvCache.SeqCount == SeqCount && kvCache.HeadCount == headCount && kvCache.HeadDim == headDim && kvCache.DType == TSATTN_I8,
+              "the KV cache does not match the layer (%d sequences, %d heads of %d, int8)", SeqCount, headCount, headDim);
+
+    // NormalizeState: per group of `groupDim` values, to int8; optionally rope first, the groups' scales, ReLU
+    auto normalize = [&](const void *src, bool srcI32, int groups, int groupDim, const int32_t *pos, uint8_t *dst, float *headScale,
+                         float scaleMult, bool relu) {
+        tsattn_produce_args a = {};
+        a.src_dtype = srcI32 ? TSATTN_SRC_I32 : TSATTN_SRC_F32;
+        a.dst_dtype = TSATTN_I8;
+        a.n_rows = SeqCount; a.n_heads = groups; a.head_dim = groupDim;
+        a.src = src; a.src_pitch = (int64_t)groups * groupDim;
+        a.pos = pos; a.rope = pos ? ropeBuf : nullptr; a.rope_len = pos ? ropeLen : 0;
+        a.rotate_dir = 1; a.vec_scale = VEC_SCALE; a.scale_mult = scaleMult;
+        a.dst = dst; a.dst_pitch = (int64_t)groups * groupDim;
+        a.scale = headScale; a.scale_pitch = 1; a.scale_row_stride = groups; // [seq][head], what the cache append reads
+        a.relu = relu ? 1 : 0;
+        Check(tsattn_rope_normalize_rows(Handle, &a, stream), "tsattn_rope_normalize_rows");
+    };
+    // MulForward / AddScaled
+    auto mulForward = [&](const uint8_t *vec, int k, const int8_t *matr, int n, int mode, float scale, void *res) {
+        tsattn_matmul_args a = {};
+        a.m = SeqCount; a.n = n; a.k = k;
+        a.a = vec; a.a_pitch = k; a.w = matr; a.w_pitch = k;
+        a.mode = mode; a.scale = scale; a.out = res; a.out_pitch = n;
+        a.workspace = Workspace; a.workspace_bytes = WorkspaceBytes;
+        Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
+    };
+
+    normalize(state, false, dim / STATE_NORM_TILE, STATE_NORM_TILE, nullptr, NormState, nullptr, 1, false);
+    mulForward(NormState, dim, att.QK, qsum, TSATTN_MM_F32, 1, QkSrc);
+    mulForward(NormState, dim, att.QV, qsum, TSATTN_MM_F32, 1, QvSrc);
+    mulForward(NormState, dim, att.K, qsum, TSATTN_MM_I32, 1, KSrc);
+    mulForward(NormState, dim, att.V, qsum, TSATTN_MM_I32, 1, VSrc);
+    normalize(QkSrc, false, headCount, headDim, t, Qk, nullptr, 1, false);
+    // the cached key scale takes the matrix scale: qvMult *= att.QVScale * VEC_SCALE * CalcDotScale(dim)
+    normalize(QvSrc, false, headCount, headDim, t, Qv, QvHeadScale, att.QVScale * VEC_SCALE * sqrtf(1.0f / (float)dim), false);
+    normalize(KSrc, true, headCount, headDim, nullptr, K, nullptr, 1, false);
+    normalize(VSrc, true, headCount, headDim, nullptr, V, nullptr, 1, false);
+
+    // kvCache.AddVectors(qv, qvHeadScale, v) and ComputeValLookup(width, slope, dims, kvCache, qk, &valLookup) in one call
+    // (width 0 would make the token attend to the row being written: two calls then)
+    if (att.AttentionWidth == 0) {
+        kvCache.AddVectors(Qv, QvHeadScale, V, VHeadScale, stream);
+        ComputeValLookup(att.AttentionWidth, att.AlibiSlope, kvCache, Qk, nullptr, VEC_SCALE, ValLookup, stream);
+    } else {
+        tsattn_decode_args a = {};
+        a.dtype = TSATTN_I8; a.q_dtype = TSATTN_Q_8BIT;
+        a.n_seqs = SeqCount; a.n_heads = headCount; a.head_dim = headDim;
+        a.q = Qk; a.q_pitch = qsum; a.q_scale = nullptr; a.q_scale_const = VEC_SCALE;
+        a.k_cache = kvCache.QVState; a.v_cache = kvCache.VState;
+        a.seq_stride = (int64_t)headCount * kvCache.MaxLen * headDim;
+        a.head_stride = (int64_t)kvCache.MaxLen * headDim;
+        a.tok_stride = headDim;
+        a.k_scale = kvCache.QVStateScale; a.v_scale = kvCache.VStateScale;
+        a.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; a.s_head_stride = kvCache.MaxLen;
+        a.cache_len = kvCache.Length; a.max_len = kvCache.MaxLen;
+        a.window = att.AttentionWidth; a.alibi_slope = att.AlibiSlope;
+        a.out = ValLookup;
+        a.k_new = Qv; a.v_new = V; a.new_pitch = qsum; a.k_scale_new = QvHeadScale; a.v_scale_new = VHeadScale;
+        Check(tsattn_decode(Handle, &a, stream), "tsattn_decode");
+    }
+
+    Check(tsattn_kv_product(Handle, SeqCount, headCount, headDim, COMBINER_REP, K, qsum, TSATTN_OUT_F32, ValLookup, qsum, 1.0f, Kv,
+                            (int64_t)qsum * COMBINER_REP, stream), "tsattn_kv_product");
+    const int kvDim = qsum * COMBINER_REP;
+    mulForward(Kv, kvDim, att.Combiner, dim, TSATTN_MM_ADD_SCALED, att.CombinerScale * VEC_SCALE * sqrtf(1.0f / (float)kvDim), state);
+
+    // relu
+    normalize(state, false, dim / STATE_NORM_TILE, STATE_NORM_TILE, nullptr, NormState, nullptr, 1, false);
+    mulForward(NormState, dim, att.Expand, ReluDim, TSATTN_MM_I32, 1, ReluSrc);
+    normalize(ReluSrc, true, headCount, ReluDim / headCount, nullptr, Relu, nullptr, 1, true);
+    mulForward(Relu, ReluDim, att.Contract, dim, TSATTN_MM_ADD_SCALED, att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim), state);
 }
 
 } // namespace NTsAttn

@@ -8,6 +8,8 @@
 //   CudaCall(c, Fp8Att)...                 gpt/compute/gpt_cuda.cu:503-507            TAttentionComputer::ComputeValLookup
 //   TAttentionVecHistory::AddVectors       gpt/train/cpu_infer.cpp:397-410            TAttentionVecHistory::AddVectors
 //   ComputeValLookup (KV cache)            gpt/train/cpu_infer.cpp:413-460 (call :509) NTsAttn::ComputeValLookup
+//   TCPUModelParams::TAttentionMatrices    gpt/train/cpu_infer.cpp:60-77              NTsAttn::TAttentionMatrices
+//   AddLookupProduct                       gpt/train/cpu_infer.cpp:465-527            TLayerComputer::AddLookupProduct
 //
 // All arithmetic runs in libtsattn.so through the C ABI of include/tsattn.h; this layer owns the
 // per-context device buffers (allocated once, like TAttentionComputeCtx::AllocateCuda,
@@ -127,5 +129,48 @@ struct TAttentionVecHistory {
 // [seqCount][headCount] (nullptr = qkConstScale).  valLookup: device [seqCount][headCount*headDim] fp32.
 void ComputeValLookup(int width, float alibiSlope, const TAttentionVecHistory &history, const void *qk,
                       const float *qkScale, float qkConstScale, float *valLookup, void *stream);
+
+// One layer's matrices of the int8 inference path, on the device: int8, one row per output (the layout MulForward
+// reads), with the scales ConvertMatrix returned.
+struct TAttentionMatrices {
+    const int8_t *QK = nullptr, *QV = nullptr, *K = nullptr, *V = nullptr; // [HeadCount*QDim][Dim]
+    const int8_t *Combiner = nullptr;                                       // [Dim][HeadCount*TTDim*COMBINER_REP]
+    const int8_t *Expand = nullptr;                                         // [ReluDim][Dim]
+    const int8_t *Contract = nullptr;                                       // [Dim][ReluDim]
+    float QVScale = 0, CombinerScale = 0, ContractScale = 0;
+    int AttentionWidth = 0;
+    float AlibiSlope = 0;
+};
+
+constexpr float VEC_SCALE = 1.0f / 24; // gpt/train/cpu_infer.cpp:16
+constexpr int STATE_NORM_TILE = 128;   // gpt/model_params/model_dim.h:22
+constexpr int COMBINER_REP = 4;        // gpt/model_params/model_dim.h:12
+
+// AddLookupProduct for a batch: one new token per sequence, every sequence with its own state row and KV cache.
+// Owns the intermediate vectors (allocated once for seqCount sequences).  QDim == TTDim == 64 or 128; the feed-forward
+// width is reluDim = HeadCount * QDim (ReluMult 1 at QDim 128).
+class TLayerComputer
+{
+    tsattn_handle_t Handle = nullptr;
+    TModelDims Dims;
+    int SeqCount = 0, ReluDim = 0;
+    uint8_t *NormState = nullptr, *Qk = nullptr, *Qv = nullptr, *K = nullptr, *V = nullptr, *Kv = nullptr, *Relu = nullptr;
+    float *QkSrc = nullptr, *QvSrc = nullptr, *QvHeadScale = nullptr, *VHeadScale = nullptr, *ValLookup = nullptr;
+    int32_t *KSrc = nullptr, *VSrc = nullptr, *ReluSrc = nullptr;
+    void *Workspace = nullptr;
+    int64_t WorkspaceBytes = 0;
+
+  public:
+    TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, int seqCount);
+    ~TLayerComputer();
+    TLayerComputer(const TLayerComputer &) = delete;
+    TLayerComputer &operator=(const TLayerComputer &) = delete;
+
+    // t: device int32 [seqCount], the new tokens' positions; ropeBuf: device table of FillRopeBuf with ropeLen rows;
+    // state: device [seqCount][Dim] fp32, updated in place; the cache gets the new rows and its lengths grow by one.
+    void AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
+                          TAttentionVecHistory *pKVCache, float *state, void *stream);
+    const float *GetValLookup() const { return ValLookup; } // [seqCount][HeadCount*TTDim] of the last call
+};
 
 } // namespace NTsAttn
