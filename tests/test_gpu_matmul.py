@@ -29,6 +29,7 @@ dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
 @pytest.mark.parametrize("m,n,k", [
     (1, 32, 64), (32, 2048, 2048), (31, 100, 192), (33, 33, 64), (64, 40, 1024), (128, 96, 320),     # few rows
     (129, 128, 64), (300, 257, 192), (1000, 130, 2048), (256, 256, 4096), (131, 1, 128),             # many rows
+    (8192, 4096, 128), (8000, 4100, 64),                                                             # many rows, tall output tiles
 ])
 def test_matmul_int32_bit_exact(ctx, m, n, k):
     rng = np.random.default_rng(m + 7 * n + k)

@@ -15,7 +15,7 @@ namespace tsattn {
 namespace {
 
 constexpr int GT_THREADS = 256;
-constexpr int GT_BM = 128, GT_BN = 128, GT_BK = 64;
+constexpr int GT_BN = 128, GT_BK = 64;
 constexpr int GT_PITCH = GT_BK + 16; // LDS row pitch: 16-lane phases of a 16-byte read hit distinct banks
 
 __device__ inline __amdgpu_buffer_rsrc_t rows_rsrc(const void *base, int64_t rows, int64_t pitch, int64_t row_bytes)
@@ -41,91 +41,234 @@ __device__ inline void store_out(const GemmParams &p, int64_t m, int64_t n, int 
 }
 
 // ---- many rows --------------------------------------------------------------------------------------------------
-template <int MODE>
-__global__ __launch_bounds__(GT_THREADS) void gemm_tiled_kernel(GemmParams p)
+// Output tiles of GT_BM x 128, K in steps of 64 bytes through LDS (two buffers), four waves as 2 x 2, each wave
+// (GT_BM / 2) x 64 = MT x 2 MFMA tiles.  What limits an int8 product here is LDS bandwidth: one 32x32x32 MFMA takes 32
+// cycles and two KiB of operands, so operands have to be used several times from registers: MT = 4 reads 6 KiB per 8
+// MFMAs.
+template <int MODE, int MT>
+__global__ __launch_bounds__(GT_THREADS, 2) void gemm_tiled_kernel(GemmParams p)
 {
-    __shared__ __attribute__((aligned(16))) uint8_t a_lds[2][GT_BM * GT_PITCH];
+    constexpr int BM = 64 * MT;
+    constexpr int A_CH = BM * GT_BK / 16 / GT_THREADS, W_CH = GT_BN * GT_BK / 16 / GT_THREADS; // 16-byte chunks per thread
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[2][BM * GT_PITCH];
     __shared__ __attribute__((aligned(16))) uint8_t w_lds[2][GT_BN * GT_PITCH];
     const int tid = threadIdx.x;
     const int lane = tid & (WAVE - 1);
     const int wave = tid / WAVE;
-    const int wm = wave >> 1, wn = wave & 1; // 2 x 2 waves of 64 x 64
+    const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 31, g = lane >> 5;
 
-    // Consecutive workgroups walk along a row of output tiles: they share one tile of activations, which is then
-    // read from HBM once; the 8 XCDs take workgroups round-robin, so each keeps every eighth tile of weights in its
-    // own L2 for the whole launch.
-    const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN;
-    const int64_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
-    const int64_t m0 = tile_m * GT_BM, n0 = tile_n * GT_BN;
-
-    const __amdgpu_buffer_rsrc_t ar = rows_rsrc(p.a + m0 * p.a_pitch, p.m - m0 < GT_BM ? p.m - m0 : GT_BM, p.a_pitch, p.k);
-    const __amdgpu_buffer_rsrc_t wr = rows_rsrc(p.w + n0 * p.w_pitch, p.n - n0 < GT_BN ? p.n - n0 : GT_BN, p.w_pitch, p.k);
-    // staging: 128 rows x 64 bytes = 512 chunks of 16 bytes per operand, two per thread
-    int a_off[2], w_off[2], lds_off[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int ch = tid + i * GT_THREADS;
-        const int r = ch >> 2, c = ch & 3;
-        a_off[i] = r * (int)p.a_pitch + c * 16;
-        w_off[i] = r * (int)p.w_pitch + c * 16;
-        lds_off[i] = r * GT_PITCH + c * 16;
+    // Which output tile.  The 8 XCDs take workgroups round-robin and each has its own L2; the 64 or so workgroups an
+    // XCD runs at a time walk through K at about the same pace, so its L2 only has to hold the current slices of the
+    // rows they use.  Give those 64 an 8 x 8 block of tiles: 8 tiles of activations and 8 of weights cross the fabric
+    // per 64 output tiles instead of up to 64 + 8.  Shapes that do not divide that way walk along rows of tiles.
+    const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN, tiles_m = (p.m + BM - 1) / BM;
+    int64_t tile_m, tile_n;
+    if (tiles_n % 8 == 0 && tiles_m % 8 == 0 && ((tiles_n >> 3) * (tiles_m >> 3)) % 8 == 0) { // whole blocks, eight at a time
+        const int64_t x = blockIdx.x & 7, l = blockIdx.x >> 3;
+        const int64_t sb = (l >> 6) * 8 + x, within = l & 63; // super-block of 8 x 8 tiles, tile inside it
+        const int64_t sb_per_row = tiles_n >> 3;
+        tile_m = (sb / sb_per_row) * 8 + (within >> 3);
+        tile_n = (sb % sb_per_row) * 8 + (within & 7);
+    } else {
+        tile_m = blockIdx.x / tiles_n;
+        tile_n = blockIdx.x % tiles_n;
     }
-    v4i ra[2], rw[2];
-    auto load = [&](int kb) __attribute__((always_inline)) {
+    const int64_t m0 = tile_m * BM, n0 = tile_n * GT_BN;
+
+    const __amdgpu_buffer_rsrc_t ar = rows_rsrc(p.a + m0 * p.a_pitch, p.m - m0 < BM ? p.m - m0 : BM, p.a_pitch, p.k);
+    const __amdgpu_buffer_rsrc_t wr = rows_rsrc(p.w + n0 * p.w_pitch, p.n - n0 < GT_BN ? p.n - n0 : GT_BN, p.w_pitch, p.k);
+    // staging: a row of 64 bytes is four chunks of 16
+    int a_off[A_CH], w_off[W_CH], a_dst[A_CH], w_dst[W_CH];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            ra[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[i], kb, 0));
-            rw[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, w_off[i], kb, 0));
-        }
+    for (int i = 0; i < A_CH; ++i) {
+        const int ch = tid + i * GT_THREADS, r = ch >> 2, c = ch & 3;
+        a_off[i] = r * (int)p.a_pitch + c * 16;
+        a_dst[i] = r * GT_PITCH + c * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < W_CH; ++i) {
+        const int ch = tid + i * GT_THREADS, r = ch >> 2, c = ch & 3;
+        w_off[i] = r * (int)p.w_pitch + c * 16;
+        w_dst[i] = r * GT_PITCH + c * 16;
+    }
+    // two sets of staging registers: what is requested at the end of step s is the tile of step s + 3 and has two
+    // whole steps to arrive before it is written to LDS
+    v4i ra[2][A_CH], rw[2][W_CH];
+    auto load = [&](int set, int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < A_CH; ++i) ra[set][i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[i], kb, 0));
+#pragma unroll
+        for (int i = 0; i < W_CH; ++i) rw[set][i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, w_off[i], kb, 0));
     };
-    auto stage = [&](int buf) __attribute__((always_inline)) {
+    auto stage = [&](int set, int buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            *(v4i *)(a_lds[buf] + lds_off[i]) = ra[i];
-            *(v4i *)(w_lds[buf] + lds_off[i]) = rw[i];
-        }
+        for (int i = 0; i < A_CH; ++i) *(v4i *)(a_lds[buf] + a_dst[i]) = ra[set][i];
+#pragma unroll
+        for (int i = 0; i < W_CH; ++i) *(v4i *)(w_lds[buf] + w_dst[i]) = rw[set][i];
     };
 
-    v16i acc[2][2];
+    v16i acc[MT][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = v16i{0};
 
     const int n_steps = (int)(p.k / GT_BK);
-    load(0);
-    stage(0);
-    if (n_steps > 1) load(GT_BK);
-    __syncthreads();
-    for (int s = 0; s < n_steps; ++s) {
-        const int buf = s & 1;
-        const uint8_t *ab = a_lds[buf] + (wm * 64 + li) * GT_PITCH + 16 * g;
+    auto compute = [&](int buf) __attribute__((always_inline)) {
+        const uint8_t *ab = a_lds[buf] + (wm * (BM / 2) + li) * GT_PITCH + 16 * g;
         const uint8_t *wb = w_lds[buf] + (wn * 64 + li) * GT_PITCH + 16 * g;
+        // all of the step's operands are asked for before the first MFMA: the LDS latency is paid once per step
+        v4i a[2][MT], w[2][2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            const v4i a0 = *(const v4i *)(ab + 32 * ks), a1 = *(const v4i *)(ab + 32 * GT_PITCH + 32 * ks);
-            const v4i w0 = *(const v4i *)(wb + 32 * ks), w1 = *(const v4i *)(wb + 32 * GT_PITCH + 32 * ks);
-            acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w1, acc[1][1], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) w[ks][j] = *(const v4i *)(wb + j * 32 * GT_PITCH + 32 * ks);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) a[ks][i] = *(const v4i *)(ab + i * 32 * GT_PITCH + 32 * ks);
         }
-        if (s + 1 < n_steps) stage(buf ^ 1);
-        if (s + 2 < n_steps) load((s + 2) * GT_BK);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks][i], w[ks][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // step s computes from LDS buffer s & 1, then writes the tile of step s + 1 (register set (s + 1) & 1) to the
+    // other buffer and asks for the tile of step s + 3 into the set just emptied
+    // (Requests and LDS writes are unconditional: past K a request reads zeros or other rows of the tile, never
+    // outside it, and nobody computes from what it leaves in LDS.  With branches around them the compiler loses track
+    // of which request is which and waits for all of them before every write.)
+    load(0, 0);
+    stage(0, 0);
+    load(1, GT_BK);
+    load(0, 2 * GT_BK);
+    __syncthreads();
+    for (int s = 0; s < n_steps; s += 2) {
+        compute(0);
+        stage(1, 1);
+        load(1, (s + 3) * GT_BK);
+        __syncthreads();
+        if (s + 1 < n_steps) compute(1);
+        stage(0, 0);
+        load(0, (s + 4) * GT_BK);
         __syncthreads();
     }
 
-    // accumulator register r of tile (i, j): row m0 + wm*64 + i*32 + 8*(r/4) + 4*g + r%4, column n0 + wn*64 + j*32 + li
+    // accumulator register r of tile (i, j): row m0 + wm*(BM/2) + i*32 + 8*(r/4) + 4*g + r%4, column n0 + wn*64 + j*32 + li
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int64_t n = n0 + wn * 64 + j * 32 + li;
             if (n >= p.n) continue;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int64_t m = m0 + wm * 64 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                const int64_t m = m0 + wm * (BM / 2) + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                if (m < p.m) store_out<MODE>(p, m, n, acc[i][j][r]);
+            }
+        }
+}
+
+// Tall tiles for large products: 256 x 128 outputs, K in steps of 128 bytes (a row's whole cache line per request),
+// one LDS buffer and one step of requests held in registers while the previous step is computed from LDS; waves of
+// 128 x 64.  K must be a multiple of 128.
+constexpr int GL_BK = 128, GL_PITCH = GL_BK + 16, GL_BM = 256;
+
+template <int MODE>
+__global__ __launch_bounds__(GT_THREADS, 2) void gemm_tall_kernel(GemmParams p)
+{
+    constexpr int MT = 4;
+    constexpr int A_CH = GL_BM * GL_BK / 16 / GT_THREADS, W_CH = GT_BN * GL_BK / 16 / GT_THREADS; // 8 and 4
+    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GL_BM * GL_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t w_lds[GT_BN * GL_PITCH];
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid / WAVE;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, g = lane >> 5;
+
+    // 8 x 8 blocks of tiles per XCD where the shape allows (see gemm_tiled_kernel)
+    const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN, tiles_m = (p.m + GL_BM - 1) / GL_BM;
+    int64_t tile_m, tile_n;
+    if (tiles_n % 8 == 0 && tiles_m % 8 == 0 && ((tiles_n >> 3) * (tiles_m >> 3)) % 8 == 0) {
+        const int64_t x = blockIdx.x & 7, l = blockIdx.x >> 3;
+        const int64_t sb = (l >> 6) * 8 + x, within = l & 63;
+        const int64_t sb_per_row = tiles_n >> 3;
+        tile_m = (sb / sb_per_row) * 8 + (within >> 3);
+        tile_n = (sb % sb_per_row) * 8 + (within & 7);
+    } else {
+        tile_m = blockIdx.x / tiles_n;
+        tile_n = blockIdx.x % tiles_n;
+    }
+    const int64_t m0 = tile_m * GL_BM, n0 = tile_n * GT_BN;
+    const __amdgpu_buffer_rsrc_t ar = rows_rsrc(p.a + m0 * p.a_pitch, p.m - m0 < GL_BM ? p.m - m0 : GL_BM, p.a_pitch, p.k);
+    const __amdgpu_buffer_rsrc_t wr = rows_rsrc(p.w + n0 * p.w_pitch, p.n - n0 < GT_BN ? p.n - n0 : GT_BN, p.w_pitch, p.k);
+    int a_off[A_CH], w_off[W_CH], a_dst[A_CH], w_dst[W_CH];
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+        const int ch = tid + i * GT_THREADS, r = ch >> 3, c = ch & 7; // eight lanes per row: its whole 128 bytes
+        a_off[i] = r * (int)p.a_pitch + c * 16;
+        a_dst[i] = r * GL_PITCH + c * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < W_CH; ++i) {
+        const int ch = tid + i * GT_THREADS, r = ch >> 3, c = ch & 7;
+        w_off[i] = r * (int)p.w_pitch + c * 16;
+        w_dst[i] = r * GL_PITCH + c * 16;
+    }
+    v4i ra[A_CH], rw[W_CH];
+    auto load = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < A_CH; ++i) ra[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[i], kb, 0));
+#pragma unroll
+        for (int i = 0; i < W_CH; ++i) rw[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, w_off[i], kb, 0));
+    };
+    auto stage = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < A_CH; ++i) *(v4i *)(a_lds + a_dst[i]) = ra[i];
+#pragma unroll
+        for (int i = 0; i < W_CH; ++i) *(v4i *)(w_lds + w_dst[i]) = rw[i];
+    };
+    v16i acc[MT][2];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = v16i{0};
+
+    const int n_steps = (int)(p.k / GL_BK);
+    const uint8_t *ab = a_lds + (wm * 128 + li) * GL_PITCH + 16 * g;
+    const uint8_t *wb = w_lds + (wn * 64 + li) * GL_PITCH + 16 * g;
+    load(0);
+    for (int s = 0; s < n_steps; ++s) {
+        stage();
+        load((s + 1) * GL_BK); // past K: zeros or other bytes of the tile, never computed with
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            v4i a[MT], w[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) w[j] = *(const v4i *)(wb + j * 32 * GL_PITCH + 32 * ks);
+#pragma unroll
+            for (int i = 0; i < MT; ++i) a[i] = *(const v4i *)(ab + i * 32 * GL_PITCH + 32 * ks);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], w[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads(); // everybody has read the step before it is overwritten
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int64_t n = n0 + wn * 64 + j * 32 + li;
+            if (n >= p.n) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
                 if (m < p.m) store_out<MODE>(p, m, n, acc[i][j][r]);
             }
         }
@@ -250,8 +393,14 @@ template <int MODE>
 void launch_mode(const GemmParams &p, hipStream_t st)
 {
     if (p.m > 32 * GS_MB) {
-        const int64_t tiles = ((p.m + GT_BM - 1) / GT_BM) * ((p.n + GT_BN - 1) / GT_BN);
-        hipLaunchKernelGGL((gemm_tiled_kernel<MODE>), dim3((unsigned)tiles), dim3(GT_THREADS), 0, st, p);
+        // tall output tiles when there are enough rows to fill the chip with them
+        const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN;
+        if (((p.m + 255) / 256) * tiles_n >= 1024) {
+            if (p.k % GL_BK == 0) hipLaunchKernelGGL((gemm_tall_kernel<MODE>), dim3((unsigned)(((p.m + 255) / 256) * tiles_n)), dim3(GT_THREADS), 0, st, p);
+            else hipLaunchKernelGGL((gemm_tiled_kernel<MODE, 4>), dim3((unsigned)(((p.m + 255) / 256) * tiles_n)), dim3(GT_THREADS), 0, st, p);
+        } else {
+            hipLaunchKernelGGL((gemm_tiled_kernel<MODE, 2>), dim3((unsigned)(((p.m + 127) / 128) * tiles_n)), dim3(GT_THREADS), 0, st, p);
+        }
         return;
     }
     // Few rows: the weights are streamed once and every compute unit has to help.  With 32 weight rows per
