@@ -289,6 +289,15 @@ def bench_matmul(ctx, steps):
     ops = 2.0 * m * n * k
     res["prompt"] = {"rows": m, "ms": round(ms, 4), "TOP/s": round(ops / ms / 1e9, 2), "frac_of_int8_peak": round(ops / ms / 1e9 / PEAK_I8_TOPS, 4)}
     del a, state
+    # a square product with an int32 result: the kernel without the state update
+    m2 = 8192
+    a = torch.randint(0, 256, (m2, k), dtype=torch.uint8, device="cuda", generator=g)
+    w2 = torch.randint(0, 256, (m2, k), dtype=torch.uint8, device="cuda", generator=g)
+    out = torch.empty((m2, m2), dtype=torch.int32, device="cuda")
+    ms = gpu_time_ms(lambda: ctx.matmul_i8(a, w2, out=out), max(3, steps // 10), 2)
+    res["square_8192"] = {"ms": round(ms, 4), "TOP/s": round(2.0 * m2 * m2 * k / ms / 1e9, 2),
+                          "frac_of_int8_peak": round(2.0 * m2 * m2 * k / ms / 1e9 / PEAK_I8_TOPS, 4)}
+    del a, w2, out
     m = 32
     a = torch.randint(0, 256, (m, k), dtype=torch.uint8, device="cuda", generator=g)
     state = torch.zeros((m, n), dtype=torch.float32, device="cuda")
