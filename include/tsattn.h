@@ -237,6 +237,22 @@ typedef struct tsattn_produce_args {
     /* Non-zero: negative results become 0 after the conversion, the ReLU of the reference's int8 feed-forward
      * block (gpt/train/cpu_infer.cpp:520-524).  int8 only. */
     int relu;
+    /* Options that let one call take the place of several (all 0 / NULL = not used):
+     * src_planes > 1 (int32 source only): the source is the sum of that many int32 arrays src_plane_stride elements
+     *   apart: the parts of a matrix product whose K was split (tsattn_matmul_i8, TSATTN_MM_I32_PLANES);
+     * rope_heads > 0: only heads below it are rotated (a row that holds the qk and qv heads first, then k and v);
+     * scale_head_count > 0: scales are written only for heads scale_head_begin .. +scale_head_count, at index
+     *   head - scale_head_begin, with scale_row_stride >= scale_head_count in the [row][head] layout;
+     * resid (f32 [n_rows][resid_pitch], n_heads*head_dim wide): the residual update that precedes the normalisation,
+     *   resid += source * resid_scale (AddScaled, cpu_infer.cpp:308-316, calls :514, :526), written back, and
+     *   the updated rows are what is normalised. */
+    int src_planes;
+    int64_t src_plane_stride;
+    int rope_heads;
+    int scale_head_begin, scale_head_count;
+    float *resid;
+    int64_t resid_pitch;
+    float resid_scale;
 } tsattn_produce_args;
 
 int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, void *stream);
@@ -261,6 +277,11 @@ enum tsattn_mm_mode {
     TSATTN_MM_I32 = 0,        /* out (int32) = sum */
     TSATTN_MM_F32 = 1,        /* out (f32) = (float)sum * scale   (MulForward into TVector<float>: scale 1) */
     TSATTN_MM_ADD_SCALED = 2, /* out (f32) += (float)sum * scale  (AddScaled) */
+    /* out (int32 [planes][m][n], n = out_pitch) = partial sums whose total over the planes is the product; *planes_out
+     * (host memory) receives their number, at most 16, 1 unless K was split (few rows, out holds 16 * m * n ints).
+     * For a consumer that adds the planes up itself (tsattn_rope_normalize_rows with src_planes) and so saves the
+     * launch that would. */
+    TSATTN_MM_I32_PLANES = 3,
 };
 
 typedef struct tsattn_matmul_args {
@@ -278,6 +299,7 @@ typedef struct tsattn_matmul_args {
      * is never exceeded).  The result is the same with and without it. */
     void *workspace;
     int64_t workspace_bytes;
+    int *planes_out;           /* TSATTN_MM_I32_PLANES: host int that receives the number of planes */
 } tsattn_matmul_args;
 
 int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *stream);

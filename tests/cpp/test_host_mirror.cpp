@@ -174,7 +174,7 @@ static int RunCase(int dtype, int window, float slope)
 // holds, so each step is checked on identical inputs: the rows appended to the two KV caches must then be identical
 // bytes (normalisation and integer products are exact on both sides), the attention output and the new state agree
 // within the attention tolerance.
-static int RunLayerCase(int width, float slope, int headDim)
+static int RunLayerCase(int width, float slope, int headDim, bool oneProjectionMatrix)
 {
     const int B = 5, H = 4, d = headDim, dim = 512, steps = 7, maxLen = 16;
     const int qsum = H * d, kvDim = qsum * 4, reluDim = H * d;
@@ -195,7 +195,16 @@ static int RunLayerCase(int width, float slope, int headDim)
     L.qv_scale = 0.031f; L.combiner_scale = 0.027f; L.contract_scale = 0.035f;
     L.attention_width = width; L.alibi_slope = slope;
     TAttentionMatrices att;
-    att.QK = ToDevice(QK); att.QV = ToDevice(QV); att.K = ToDevice(K); att.V = ToDevice(V);
+    int8_t *proj = nullptr;
+    if (oneProjectionMatrix) {
+        // QK, QV, K, V one after the other in memory: the layer makes one product of them
+        std::vector<int8_t> all;
+        for (const auto *m : {&QK, &QV, &K, &V}) all.insert(all.end(), m->begin(), m->end());
+        proj = ToDevice(all);
+        att.QK = proj; att.QV = proj + QK.size(); att.K = proj + 2 * QK.size(); att.V = proj + 3 * QK.size();
+    } else {
+        att.QK = ToDevice(QK); att.QV = ToDevice(QV); att.K = ToDevice(K); att.V = ToDevice(V);
+    }
     att.Combiner = ToDevice(Comb); att.Expand = ToDevice(Expand); att.Contract = ToDevice(Contract);
     att.QVScale = L.qv_scale; att.CombinerScale = L.combiner_scale; att.ContractScale = L.contract_scale;
     att.AttentionWidth = width; att.AlibiSlope = slope;
@@ -268,11 +277,13 @@ static int RunLayerCase(int width, float slope, int headDim)
         // can a few of the int8 values the feed-forward block derives from the state: steps of single int8 units, far
         // below the state's scale (most steps come out bit-identical)
         if (maxVal > 2e-5 || maxState > 2e-2) ++fails;
-        printf("layer width %4d slope %.2f d %3d: %d tokens x %d sequences, max |valLookup diff| %.2e, max |state diff| / rms %.2e  %s\n", width,
-               slope, d, steps, B, maxVal, maxState, fails ? "FAIL" : "ok");
+        printf("layer width %4d slope %.2f d %3d %s: %d tokens x %d sequences, max |valLookup diff| %.2e, max |state diff| / rms %.2e  %s\n", width,
+               slope, d, oneProjectionMatrix ? "(one projection product)" : "(four)", steps, B, maxVal, maxState, fails ? "FAIL" : "ok");
         HIP_OK(hipFree(ropeDev)); HIP_OK(hipFree(stateDev)); HIP_OK(hipFree(tDev));
     }
-    for (const int8_t *p : {att.QK, att.QV, att.K, att.V, att.Combiner, att.Expand, att.Contract}) HIP_OK(hipFree((void *)p));
+    if (proj) HIP_OK(hipFree(proj));
+    else for (const int8_t *p : {att.QK, att.QV, att.K, att.V}) HIP_OK(hipFree((void *)p));
+    for (const int8_t *p : {att.Combiner, att.Expand, att.Contract}) HIP_OK(hipFree((void *)p));
     tsattn_destroy(handle);
     return fails;
 }
@@ -280,10 +291,11 @@ static int RunLayerCase(int width, float slope, int headDim)
 int main()
 {
     int fails = 0;
-    fails += RunLayerCase(1000, 0.0f, 128);
-    fails += RunLayerCase(4, 0.5f, 128);
-    fails += RunLayerCase(1, 0.0f, 64);
-    fails += RunLayerCase(0, 0.0f, 128);
+    fails += RunLayerCase(1000, 0.0f, 128, true);
+    fails += RunLayerCase(1000, 0.0f, 128, false);
+    fails += RunLayerCase(4, 0.5f, 128, true);
+    fails += RunLayerCase(1, 0.0f, 64, false);
+    fails += RunLayerCase(0, 0.0f, 128, true);
     for (int dtype : {TSATTN_I8, TSATTN_E4M3}) {
         fails += RunCase(dtype, 64, 0.5f);
         fails += RunCase(dtype, 1000, 0.0f);

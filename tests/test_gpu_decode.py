@@ -119,7 +119,7 @@ def test_decode_constant_scales_and_reference_polynomial(ctx):
 
 
 def test_decode_full_size_properties(ctx):
-    """BASELINE decode shape (B64, L4096, H16, d128, int8, bf16 query): size-independent properties.
+    """The benchmark's decode shape (B64, L4096, H16, d128, int8, bf16 query): size-independent properties.
     (a) V = ones with scale 1 -> every output element equals 1 - 2^-swl >= 0 and is identical across d;
     (b) the result does not depend on the number of KV splits beyond fp32 re-association."""
     from tscale_amd import KVCache

@@ -1,0 +1,69 @@
+"""GPU: one layer of the int8 inference path, token by token (tscale_amd.attention.add_lookup_product: a chain of
+library calls through the C ABI) against the oracle's AddLookupProduct (gpt/train/cpu_infer.cpp:465-527).  Each step
+starts from the state the GPU path holds, so inputs are identical: appended cache rows and key scales must be the same
+bytes, the attention output agrees to a few ulps, the new state is the same up to flips of single int8 roundings."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import pyoracle as orc
+from tscale_amd import KVCache, capi
+from tscale_amd.attention import VEC_SCALE, add_lookup_product
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from tscale_amd import AttentionContext
+    c = AttentionContext(0, max_seqs=8, max_heads=4, max_head_dim=128)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("H,d,dim,width,slope", [(2, 128, 256, 1000, 0.0), (4, 64, 512, 3, 0.5), (2, 128, 384, 0, 0.0)])
+def test_layer_steps_match_the_oracle(ctx, H, d, dim, width, slope):
+    B, max_len, steps = 4, 12, 6
+    qsum = H * d
+    rng = np.random.default_rng(H * d + width)
+    mat = lambda n, k: np.clip(np.rint(rng.standard_normal((n, k)) * 32), -127, 127).astype(np.int8)
+    mats = {"qk": mat(qsum, dim), "qv": mat(qsum, dim), "k": mat(qsum, dim), "v": mat(qsum, dim),
+            "combiner": mat(dim, qsum * 4), "expand": mat(qsum, dim), "contract": mat(dim, qsum)}
+    scales = (0.031, 0.027, 0.035)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    layer = {"proj": dev(np.concatenate([mats[n] for n in ("qk", "qv", "k", "v")]).view(np.uint8)),
+             "combiner": dev(mats["combiner"].view(np.uint8)), "expand": dev(mats["expand"].view(np.uint8)),
+             "contract": dev(mats["contract"].view(np.uint8)), "qv_scale": scales[0], "combiner_scale": scales[1],
+             "contract_scale": scales[2], "width": width, "slope": slope}
+    # caches with some history; sequence 3 runs into the end of its cache
+    # (values in [-127, 127] as the reference's conversion leaves them: its vpdpbusd dot product, which the oracle
+    # follows, is not defined for -128, cpu_infer.cpp:88-92)
+    kc = rng.integers(-127, 128, (B, H, max_len, d)).astype(np.int8).view(np.uint8)
+    vc = rng.integers(-127, 128, (B, H, max_len, d)).astype(np.int8).view(np.uint8)
+    ksc = ((rng.random((B, H, max_len)) + 0.5) * 1e-3).astype(np.float32)
+    lens = np.array([0, 2, 7, 9], dtype=np.int32)
+    cache = KVCache(ctx, capi.I8, B, H, max_len, d)
+    cache.k.copy_(dev(kc)); cache.v.copy_(dev(vc)); cache.k_scale.copy_(dev(ksc)); cache.v_scale.fill_(VEC_SCALE)
+    cache.cache_len.copy_(dev(lens))
+    rope_np = orc.fill_rope(d, 64)
+    rope = dev(rope_np)
+    state = dev(rng.standard_normal((B, dim)).astype(np.float32) * 2)
+    room = torch.empty(16 * 4 * B * dim, dtype=torch.uint8, device="cuda")
+    keep = {}
+    exact_steps = 0
+    for step in range(steps):
+        t = (lens + 3).astype(np.int32)
+        st_in = state.cpu().numpy()
+        want, want_val = orc.add_lookup_product(mats, scales, width, slope, H, d, t, rope_np, st_in, kc, vc, ksc, lens)
+        val = add_lookup_product(ctx, layer, cache, dev(t), rope, state, workspace=room, scratch=keep)
+        torch.cuda.synchronize()
+        assert cache.cache_len.cpu().numpy().tolist() == lens.tolist()
+        assert np.array_equal(cache.k.cpu().numpy(), kc) and np.array_equal(cache.v.cpu().numpy(), vc), f"step {step}: cache rows"
+        assert np.array_equal(cache.k_scale.cpu().numpy(), ksc), f"step {step}: cached key scales"
+        assert np.abs(val.cpu().numpy() - want_val).max() < 2e-5
+        got = state.cpu().numpy()
+        rms = np.sqrt((want.astype(np.float64) ** 2).mean())
+        assert np.abs(got - want).max() / rms < 2e-2, f"step {step}"
+        exact_steps += int(np.array_equal(got, want))
+    assert lens.tolist() == [min(max_len, l + steps) for l in (0, 2, 7, 9)]
+    assert exact_steps >= steps // 2, "most steps come out bit-identical"

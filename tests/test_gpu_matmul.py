@@ -94,3 +94,16 @@ def test_matmul_split_k_with_a_workspace_gives_the_same_bits(ctx, m, n, k, mode)
         got = ctx.matmul_i8(dev(a.view(np.uint8)), dev(w.view(np.uint8)), mode=mode, scale=0.002, out=out, workspace=ws)
         torch.cuda.synchronize()
         assert np.array_equal(got.cpu().numpy(), want), f"workspace {ws_bytes} bytes"
+
+
+@pytest.mark.parametrize("m,n,k", [(32, 2048, 8192), (5, 96, 128), (300, 130, 256)])
+def test_matmul_planes_sum_to_the_product(ctx, m, n, k):
+    """TSATTN_MM_I32_PLANES: the parts of a split-K product left as int32 planes for a consumer that adds them up."""
+    rng = np.random.default_rng(m * n)
+    a, w = rand_i8(rng, (m, k)), rand_i8(rng, (n, k))
+    planes = ctx.matmul_i8(dev(a.view(np.uint8)), dev(w.view(np.uint8)), mode=capi.MM_I32_PLANES)
+    torch.cuda.synchronize()
+    assert 1 <= planes.shape[0] <= 16 and planes.shape[1:] == (m, n)
+    if (m, n, k) == (32, 2048, 8192):
+        assert planes.shape[0] > 1, "this shape is meant to split K"
+    assert np.array_equal(planes.sum(dim=0, dtype=torch.int32).cpu().numpy(), orc.matmul_i8(a, w))

@@ -119,3 +119,43 @@ def test_producer_relu_and_row_major_scales(ctx):
     assert s.shape == (n, H) and np.array_equal(s.cpu().numpy(), want_s.T)
     with pytest.raises(capi.TsattnError):
         ctx.rope_normalize_rows(xd, H, capi.E4M3, relu=True)
+
+
+def test_producer_fused_forms_equal_the_separate_calls(ctx):
+    """One producer call standing in for several: the parts of a split-K product summed on the fly, rotation for the
+    leading heads only, scales for a range of heads, the residual update before the normalisation.  Each against the
+    oracle's separate steps, bit for bit."""
+    rng = np.random.default_rng(33)
+    n, H, d = 19, 2, 128
+    hd4 = 4 * H * d     # a row holding the qk, qv, k and v heads
+    parts = (rng.standard_normal((3, n, hd4)) * 3000).astype(np.int32)
+    total = parts.sum(axis=0).astype(np.int32)
+    pos = rng.integers(0, 50, n).astype(np.int32)
+    rope = orc.fill_rope(d, 64)
+    # the oracle's four separate calls on the summed product
+    seg = lambda i: np.ascontiguousarray(total[:, i * H * d:(i + 1) * H * d])
+    want = [orc.rope_normalize_rows(capi.I8, seg(0), H, pos=pos, rope=rope),
+            orc.rope_normalize_rows(capi.I8, seg(1), H, pos=pos, rope=rope, scale_mult=0.37),
+            orc.rope_normalize_rows(capi.I8, seg(2), H),
+            orc.rope_normalize_rows(capi.I8, seg(3), H)]
+    q, s = ctx.rope_normalize_rows(torch.from_numpy(parts).cuda(), 4 * H, capi.I8, pos=torch.from_numpy(pos).cuda(),
+                                   rope=torch.from_numpy(rope).cuda(), scale_mult=0.37, row_major_scale=True,
+                                   rope_heads=2 * H, scale_heads=(H, H))
+    torch.cuda.synchronize()
+    got = q.cpu().numpy()
+    for i in range(4):
+        assert np.array_equal(got[:, i * H * d:(i + 1) * H * d], want[i][0]), f"segment {i}"
+    assert s.shape == (n, H) and np.array_equal(s.cpu().numpy(), want[1][1].T)
+
+    # residual update, then normalisation of the updated state (AddScaled + NormalizeState)
+    dim = 4 * d
+    state = rng.standard_normal((n, dim)).astype(np.float32)
+    delta = (rng.standard_normal((2, n, dim)) * 50000).astype(np.int32)
+    scale = np.float32(3.1e-5)
+    new_state = state + delta.sum(axis=0).astype(np.float32) * scale       # one rounding per operation, as in AddScaled
+    want_q, _ = orc.rope_normalize_rows(capi.I8, new_state, dim // 128)
+    st = torch.from_numpy(state).cuda()
+    q, _ = ctx.rope_normalize_rows(torch.from_numpy(delta).cuda(), dim // 128, capi.I8, resid=st, resid_scale=float(scale))
+    torch.cuda.synchronize()
+    assert np.array_equal(st.cpu().numpy(), new_state)
+    assert np.array_equal(q.cpu().numpy(), want_q)

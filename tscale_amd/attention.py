@@ -92,36 +92,52 @@ class AttentionContext:
         return host.to(self.device)
 
     def rope_normalize_rows(self, x, n_heads, dtype, pos=None, rope=None, rotate_dir=1.0, vec_scale=1.0 / 24,
-                            scale_mult=1.0, row_major_scale=False, relu=False):
+                            scale_mult=1.0, row_major_scale=False, relu=False, rope_heads=0, scale_heads=None,
+                            resid=None, resid_scale=1.0):
         """ApplyRope + NormalizeState of the reference's inference path (cpu_infer.cpp:486-499): x [n_rows, H*d]
         float32 or int32 -> (uint8 [n_rows, H*d], f32 scale [H, n_rows], or [n_rows, H] with row_major_scale: what
-        the cache append reads); pos int32 [n_rows] or None (no rotation); relu: negative results become 0 (:520-524)."""
-        assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.dtype in (torch.float32, torch.int32)
-        n_rows, hd = x.shape
+        the cache append reads); pos int32 [n_rows] or None (no rotation); relu: negative results become 0 (:520-524).
+        x may be int32 [planes, n_rows, H*d]: the parts of a split-K product, summed on the fly.  rope_heads: only the
+        heads below it are rotated.  scale_heads = (begin, count): scales only for those heads.  resid (f32
+        [n_rows, H*d]): resid += x * resid_scale first, in place, and the updated rows are normalised."""
+        assert x.is_cuda and x.is_contiguous() and x.dtype in (torch.float32, torch.int32)
+        planes = 1
+        if x.dim() == 3:
+            assert x.dtype == torch.int32
+            planes = x.shape[0]
+        n_rows, hd = x.shape[-2:]
         q = torch.empty((n_rows, hd), dtype=torch.uint8, device=x.device)
-        scale = torch.empty((n_rows, n_heads) if row_major_scale else (n_heads, n_rows), dtype=torch.float32, device=x.device)
+        n_scale = n_heads if scale_heads is None else scale_heads[1]
+        scale = torch.empty((n_rows, n_scale) if row_major_scale else (n_scale, n_rows), dtype=torch.float32, device=x.device)
         a = capi.ProduceArgs()
         a.src_dtype = capi.SRC_F32 if x.dtype == torch.float32 else capi.SRC_I32
         a.dst_dtype = dtype
         a.n_rows, a.n_heads, a.head_dim = n_rows, n_heads, hd // n_heads
         a.src, a.src_pitch = _ptr(x), hd
+        a.src_planes, a.src_plane_stride = planes, n_rows * hd
         a.pos, a.rope = _ptr(pos), _ptr(rope)
         a.rope_len = 0 if rope is None else rope.shape[0]
+        a.rope_heads = int(rope_heads)
         a.rotate_dir, a.vec_scale, a.scale_mult = float(rotate_dir), float(vec_scale), float(scale_mult)
         a.dst, a.dst_pitch = _ptr(q), hd
         a.scale, a.scale_pitch = _ptr(scale), (1 if row_major_scale else n_rows)
-        a.scale_row_stride = n_heads if row_major_scale else 1
+        a.scale_row_stride = n_scale if row_major_scale else 1
+        if scale_heads is not None:
+            a.scale_head_begin, a.scale_head_count = int(scale_heads[0]), int(scale_heads[1])
         a.relu = int(bool(relu))
+        if resid is not None:
+            assert resid.dtype == torch.float32 and resid.shape == (n_rows, hd) and resid.stride(1) == 1
+            a.resid, a.resid_pitch, a.resid_scale = _ptr(resid), resid.stride(0), float(resid_scale)
         capi.check(self.lib.tsattn_rope_normalize_rows(self.handle, ctypes.byref(a), _stream_ptr()))
         return q, scale
 
     def kv_product(self, k, value, n_heads, rep=4, mult=1.0):
         """KVProduct (cpu_infer.cpp:320-337): k uint8 (int8 bytes) [n, H*d], value f32/f16 [n, H*d] -> uint8 [n, H*d*rep]."""
         n, hd = k.shape
-        assert value.shape == k.shape and value.is_contiguous() and k.is_contiguous()
+        assert value.shape == k.shape and value.is_contiguous() and k.stride(1) == 1
         kv = torch.empty((n, hd * rep), dtype=torch.uint8, device=k.device)
         vdt = capi.OUT_F16 if value.dtype == torch.float16 else capi.OUT_F32
-        capi.check(self.lib.tsattn_kv_product(self.handle, n, n_heads, hd // n_heads, rep, _ptr(k), hd, vdt, _ptr(value), hd,
+        capi.check(self.lib.tsattn_kv_product(self.handle, n, n_heads, hd // n_heads, rep, _ptr(k), k.stride(0), vdt, _ptr(value), hd,
                                               float(mult), _ptr(kv), hd * rep, _stream_ptr()))
         return kv
 
@@ -132,6 +148,21 @@ class AttentionContext:
         m, k = a.shape
         n = w.shape[0]
         assert w.shape[1] == k and a.stride(1) == 1 and w.stride(1) == 1
+        if mode == capi.MM_I32_PLANES:
+            # partial sums [planes, m, n] for a consumer that adds them up (rope_normalize_rows); returns the planes in use
+            if out is None:
+                out = torch.empty((16, m, n), dtype=torch.int32, device=a.device)
+            assert out.is_contiguous() and out.dtype == torch.int32 and out.numel() >= 16 * m * n
+            args = capi.MatmulArgs()
+            args.m, args.n, args.k = m, n, k
+            args.a, args.a_pitch = _ptr(a), a.stride(0)
+            args.w, args.w_pitch = _ptr(w), w.stride(0)
+            args.mode, args.scale = mode, 1.0
+            args.out, args.out_pitch = _ptr(out), n
+            planes = ctypes.c_int(0)
+            args.planes_out = ctypes.pointer(planes)
+            capi.check(self.lib.tsattn_matmul_i8(self.handle, ctypes.byref(args), _stream_ptr()))
+            return out.view(-1)[:planes.value * m * n].view(planes.value, m, n)
         if out is None:
             assert mode != capi.MM_ADD_SCALED
             out = torch.empty((m, n), dtype=torch.int32 if mode == capi.MM_I32 else torch.float32, device=a.device)
@@ -239,41 +270,44 @@ STATE_NORM_TILE = 128     # gpt/model_params/model_dim.h:22
 COMBINER_REP = 4          # gpt/model_params/model_dim.h:12
 
 
-def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None):
+def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None, scratch=None):
     """One layer of the int8 inference path for one new token per sequence: AddLookupProduct,
-    gpt/train/cpu_infer.cpp:465-527, as a chain of library calls (the C++ form is NTsAttn::TLayerComputer).
-    layer: dict with uint8 (int8 bytes) matrices qk, qv, k, v [H*d, dim], combiner [dim, 4*H*d], expand [H*d, dim],
-    contract [dim, H*d], floats qv_scale, combiner_scale, contract_scale, and width, slope.  cache: KVCache whose value
-    scales are VEC_SCALE; t: int32 [B] positions; rope: table of fill_rope_table; state: f32 [B, dim], updated in place.
+    gpt/train/cpu_infer.cpp:465-527, as a chain of 11-12 library calls (the C++ form is NTsAttn::TLayerComputer).
+    layer: dict with uint8 (int8 bytes) matrices proj [4*H*d, dim] (the QK, QV, K and V matrices one after the other),
+    combiner [dim, 4*H*d], expand [H*d, dim], contract [dim, H*d], floats qv_scale, combiner_scale, contract_scale, and
+    width, slope.  cache: KVCache whose value scales are VEC_SCALE; t: int32 [B] positions; rope: table of
+    fill_rope_table; state: f32 [B, dim], updated in place.  scratch: dict for buffers kept between calls.
     Returns the attention output [B, H*d]."""
     B, dim = state.shape
     H, d = cache.n_heads, cache.head_dim
     qsum = H * d
     groups = dim // STATE_NORM_TILE
+    f32 = np.float32
+    sc = scratch if scratch is not None else {}
+    if "planes" not in sc:
+        sc["planes"] = torch.empty((16, B, max(4 * qsum, dim)), dtype=torch.int32, device=state.device)
+        sc["v_scale"] = torch.full((B, H), VEC_SCALE, dtype=torch.float32, device=state.device)
+    planes_buf, v_scale = sc["planes"], sc["v_scale"]
     norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
-    qk_src = ctx.matmul_i8(norm, layer["qk"], mode=capi.MM_F32, workspace=workspace)
-    qv_src = ctx.matmul_i8(norm, layer["qv"], mode=capi.MM_F32, workspace=workspace)
-    k_src = ctx.matmul_i8(norm, layer["k"], workspace=workspace)
-    v_src = ctx.matmul_i8(norm, layer["v"], workspace=workspace)
-    qk, _ = ctx.rope_normalize_rows(qk_src, H, capi.I8, pos=t, rope=rope)
-    key_mult = float(np.float32(layer["qv_scale"]) * np.float32(VEC_SCALE) * np.float32(np.sqrt(np.float32(1.0) / np.float32(dim))))
-    qv, qv_scale = ctx.rope_normalize_rows(qv_src, H, capi.I8, pos=t, rope=rope, scale_mult=key_mult, row_major_scale=True)
-    k, _ = ctx.rope_normalize_rows(k_src, H, capi.I8)
-    v, _ = ctx.rope_normalize_rows(v_src, H, capi.I8)
-    v_scale = torch.full((B, H), VEC_SCALE, dtype=torch.float32, device=state.device)
+    # the four projections as one product; RoPE on the qk and qv heads, per-head normalisation of all four in one call
+    proj = ctx.matmul_i8(norm, layer["proj"], mode=capi.MM_I32_PLANES, out=planes_buf)
+    key_mult = float(f32(layer["qv_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(dim))))
+    q4, qv_scale = ctx.rope_normalize_rows(proj, 4 * H, capi.I8, pos=t, rope=rope, scale_mult=key_mult, row_major_scale=True,
+                                           rope_heads=2 * H, scale_heads=(H, H))
+    qk, qv, k, v = q4[:, :qsum], q4[:, qsum:2 * qsum], q4[:, 2 * qsum:3 * qsum], q4[:, 3 * qsum:]
     if layer["width"] == 0:   # the token attends to the row being written: append first
         cache.add_vectors(qv, qv_scale, v, v_scale)
         val = ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, 0, layer["slope"])
     else:
         val = ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, layer["width"], layer["slope"], append=(qv, qv_scale, v, v_scale))
     kv = ctx.kv_product(k, val, H, COMBINER_REP)
-    f32 = np.float32
-    ctx.matmul_i8(kv, layer["combiner"], mode=capi.MM_ADD_SCALED, out=state, workspace=workspace,
-                  scale=float(f32(layer["combiner_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(qsum * COMBINER_REP)))))
-    norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
-    relu_src = ctx.matmul_i8(norm, layer["expand"], workspace=workspace)
+    # combiner; its AddScaled is done by the normalisation that follows
+    delta = ctx.matmul_i8(kv, layer["combiner"], mode=capi.MM_I32_PLANES, out=planes_buf)
+    norm, _ = ctx.rope_normalize_rows(delta, groups, capi.I8, resid=state,
+                                      resid_scale=float(f32(layer["combiner_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(qsum * COMBINER_REP)))))
+    relu_src = ctx.matmul_i8(norm, layer["expand"], mode=capi.MM_I32_PLANES, out=planes_buf)
     relu, _ = ctx.rope_normalize_rows(relu_src, H, capi.I8, relu=True)
-    relu_dim = relu_src.shape[1]
+    relu_dim = relu_src.shape[-1]
     ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state, workspace=workspace,
                   scale=float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim)))))
     return val

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libtsattn.so")
 I8, E4M3 = 0, 1
 OUT_F32, OUT_F16 = 0, 1
 SRC_F32, SRC_BF16, SRC_I32 = 0, 1, 2
-MM_I32, MM_F32, MM_ADD_SCALED = 0, 1, 2
+MM_I32, MM_F32, MM_ADD_SCALED, MM_I32_PLANES = 0, 1, 2, 3
 Q_8BIT, Q_BF16 = 0, 1
 SPAN_TILE_INTS = 32
 
@@ -78,6 +78,8 @@ class ProduceArgs(_c.Structure):
         ("rope", _c.c_void_p), ("rope_len", _c.c_int64), ("rotate_dir", _c.c_float), ("vec_scale", _c.c_float),
         ("scale_mult", _c.c_float), ("dst", _c.c_void_p), ("dst_pitch", _c.c_int64), ("scale", _c.c_void_p),
         ("scale_pitch", _c.c_int64), ("scale_row_stride", _c.c_int64), ("relu", _c.c_int),
+        ("src_planes", _c.c_int), ("src_plane_stride", _c.c_int64), ("rope_heads", _c.c_int), ("scale_head_begin", _c.c_int),
+        ("scale_head_count", _c.c_int), ("resid", _c.c_void_p), ("resid_pitch", _c.c_int64), ("resid_scale", _c.c_float),
     ]
 
 
@@ -85,7 +87,7 @@ class MatmulArgs(_c.Structure):
     _fields_ = [
         ("m", _c.c_int64), ("n", _c.c_int64), ("k", _c.c_int64), ("a", _c.c_void_p), ("a_pitch", _c.c_int64),
         ("w", _c.c_void_p), ("w_pitch", _c.c_int64), ("mode", _c.c_int), ("scale", _c.c_float), ("out", _c.c_void_p),
-        ("out_pitch", _c.c_int64), ("workspace", _c.c_void_p), ("workspace_bytes", _c.c_int64),
+        ("out_pitch", _c.c_int64), ("workspace", _c.c_void_p), ("workspace_bytes", _c.c_int64), ("planes_out", _c.POINTER(_c.c_int)),
     ]
 
 

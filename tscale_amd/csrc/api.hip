@@ -299,9 +299,18 @@ int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, 
         (a->rope && !aligned16(a->rope)))
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: pitches must cover a row; src, dst and rope 16-byte aligned, pitches multiples of 16 bytes");
     const int64_t row_stride = a->scale_row_stride ? a->scale_row_stride : 1;
+    if (a->scale_head_count < 0 || a->scale_head_begin < 0 || a->scale_head_begin + a->scale_head_count > a->n_heads)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale head range outside the heads");
+    const int scale_heads = a->scale_head_count > 0 ? a->scale_head_count : a->n_heads;
     if (a->scale && (row_stride < 0 || a->scale_pitch <= 0 ||
-                     !((row_stride == 1 && a->scale_pitch >= a->n_rows) || (a->scale_pitch == 1 && row_stride >= a->n_heads))))
-        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale layout must be [n_heads][scale_pitch >= n_rows] or [n_rows][scale_row_stride >= n_heads]");
+                     !((row_stride == 1 && a->scale_pitch >= a->n_rows) || (a->scale_pitch == 1 && row_stride >= scale_heads))))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale layout must be [heads][scale_pitch >= n_rows] or [n_rows][scale_row_stride >= heads]");
+    if (a->src_planes < 0 || a->src_planes > 16 || (a->src_planes > 1 && (a->src_dtype != TSATTN_SRC_I32 || a->src_plane_stride < a->n_rows * a->src_pitch ||
+                                                                           a->src_plane_stride % 4)))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: up to 16 int32 source planes, at least n_rows * src_pitch elements apart, 16-byte aligned");
+    if (a->rope_heads < 0 || a->rope_heads > a->n_heads) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: rope_heads outside the heads");
+    if (a->resid && (a->resid_pitch < row || a->resid_pitch % 4 || !aligned16(a->resid)))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: resid must be 16-byte aligned with a pitch that covers a row");
     if (a->relu && a->dst_dtype != TSATTN_I8) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_rope_normalize_rows: relu with an int8 result only");
     tsattn::ProduceParams p;
     p.src = a->src; p.src_pitch = a->src_pitch; p.n_rows = a->n_rows; p.n_heads = a->n_heads;
@@ -309,6 +318,10 @@ int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, 
     p.rotate_dir = a->rotate_dir; p.vec_scale = a->vec_scale; p.scale_mult = a->scale_mult;
     p.dst = (uint8_t *)a->dst; p.dst_pitch = a->dst_pitch; p.scale = a->scale; p.scale_pitch = a->scale_pitch;
     p.scale_row_stride = row_stride; p.relu = a->relu;
+    p.src_planes = a->src_planes > 1 ? a->src_planes : 1; p.src_plane_stride = a->src_plane_stride;
+    p.rope_heads = a->rope_heads > 0 ? a->rope_heads : a->n_heads;
+    p.scale_head_begin = a->scale_head_count > 0 ? a->scale_head_begin : 0; p.scale_head_count = scale_heads;
+    p.resid = a->resid; p.resid_pitch = a->resid_pitch; p.resid_scale = a->resid_scale;
     hipError_t e = tsattn::launch_rope_normalize(p, a->dst_dtype, a->head_dim, a->src_dtype == TSATTN_SRC_I32, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "rope normalize launch");
     return TSATTN_OK;
@@ -341,8 +354,10 @@ int tsattn_kv_product(tsattn_handle_t h, int64_t n_rows, int n_heads, int head_d
 int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *stream)
 {
     if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: null argument");
-    if (a->mode != TSATTN_MM_I32 && a->mode != TSATTN_MM_F32 && a->mode != TSATTN_MM_ADD_SCALED)
+    if (a->mode != TSATTN_MM_I32 && a->mode != TSATTN_MM_F32 && a->mode != TSATTN_MM_ADD_SCALED && a->mode != TSATTN_MM_I32_PLANES)
         return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: mode %d", a->mode);
+    if (a->mode == TSATTN_MM_I32_PLANES && !a->planes_out) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: planes_out is needed for the planes mode");
+    if (a->mode == TSATTN_MM_I32_PLANES && a->out_pitch != a->n) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: the planes are dense: out_pitch must equal n");
     if (a->m < 0 || a->n < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: negative size");
     if (a->k <= 0 || a->k % 64) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: k %lld (a positive multiple of 64)", (long long)a->k);
     if (a->m == 0 || a->n == 0) return TSATTN_OK;
@@ -356,7 +371,7 @@ int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *strea
     p.m = a->m; p.n = a->n; p.k = a->k; p.mode = a->mode; p.scale = a->scale; p.out = a->out; p.out_pitch = a->out_pitch;
     const bool ws_ok = a->workspace && a->workspace_bytes > 0 && aligned16(a->workspace);
     p.workspace = ws_ok ? a->workspace : nullptr; p.workspace_bytes = ws_ok ? a->workspace_bytes : 0; p.split_stride = 0;
-    hipError_t e = tsattn::launch_matmul_i8(p, (hipStream_t)stream);
+    hipError_t e = tsattn::launch_matmul_i8(p, (hipStream_t)stream, a->planes_out);
     if (e != hipSuccess) return hip_fail(e, "matmul launch");
     return TSATTN_OK;
 }

@@ -403,33 +403,53 @@ void launch_mode(const GemmParams &p, hipStream_t st)
         }
         return;
     }
-    // Few rows: the weights are streamed once and every compute unit has to help.  With 32 weight rows per
-    // workgroup there are too few workgroups unless K is split as well, which needs room for the parts' sums.
+    hipLaunchKernelGGL((gemm_skinny_kernel<MODE>), dim3((unsigned)((p.n + GS_BN - 1) / GS_BN), 1), dim3(GS_THREADS), 0, st, p);
+}
+
+// Few rows: the weights are streamed once and every compute unit has to help.  With 32 weight rows per workgroup
+// there are too few workgroups unless K is split as well, which needs room for the parts' sums.
+int split_for(const GemmParams &p, int64_t room_bytes)
+{
+    if (p.m > 32 * GS_MB) return 1;
     const int64_t n_tiles = (p.n + GS_BN - 1) / GS_BN;
     int split = 1;
-    while (split < 16 && n_tiles * split < 512 && p.k / (split * 2) >= GS_SLAB &&
-           (int64_t)(split * 2) * p.m * p.n * 4 <= p.workspace_bytes)
-        split *= 2;
-    if (split == 1) {
-        hipLaunchKernelGGL((gemm_skinny_kernel<MODE>), dim3((unsigned)n_tiles, 1), dim3(GS_THREADS), 0, st, p);
-        return;
-    }
-    GemmParams q = p;
-    q.out = p.workspace;
-    q.out_pitch = p.n;
-    q.split_stride = p.m * p.n;
-    hipLaunchKernelGGL((gemm_skinny_kernel<TSATTN_MM_I32>), dim3((unsigned)n_tiles, (unsigned)split), dim3(GS_THREADS), 0, st, q);
-    GemmParams r = p;
-    r.split_stride = p.m * p.n;
-    hipLaunchKernelGGL((gemm_reduce_kernel<MODE>), dim3((unsigned)((p.m * p.n + 255) / 256)), dim3(256), 0, st, r,
-                       (const int32_t *)p.workspace, split);
+    while (split < 16 && n_tiles * split < 512 && p.k / (split * 2) >= GS_SLAB && (int64_t)(split * 2) * p.m * p.n * 4 <= room_bytes) split *= 2;
+    return split;
 }
 
 } // namespace
 
-hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st)
+hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out)
 {
-    if (p.m <= 0 || p.n <= 0) return hipSuccess;
+    if (p.m <= 0 || p.n <= 0) {
+        if (planes_out) *planes_out = 1;
+        return hipSuccess;
+    }
+    if (p.mode == TSATTN_MM_I32_PLANES) {
+        // the parts' sums straight into the caller's planes (16 * m * n ints of room by contract)
+        const int split = split_for(p, (int64_t)16 * p.m * p.n * 4);
+        GemmParams q = p;
+        q.split_stride = p.m * p.n;
+        if (split == 1) launch_mode<TSATTN_MM_I32>(q, st);
+        else hipLaunchKernelGGL((gemm_skinny_kernel<TSATTN_MM_I32>), dim3((unsigned)((p.n + GS_BN - 1) / GS_BN), (unsigned)split), dim3(GS_THREADS), 0, st, q);
+        *planes_out = split;
+        return hipGetLastError();
+    }
+    const int split = split_for(p, p.workspace ? p.workspace_bytes : 0);
+    if (split > 1) {
+        GemmParams q = p;
+        q.out = p.workspace;
+        q.out_pitch = p.n;
+        q.split_stride = p.m * p.n;
+        hipLaunchKernelGGL((gemm_skinny_kernel<TSATTN_MM_I32>), dim3((unsigned)((p.n + GS_BN - 1) / GS_BN), (unsigned)split), dim3(GS_THREADS), 0, st, q);
+        GemmParams r = p;
+        r.split_stride = p.m * p.n;
+        const dim3 grid((unsigned)((p.m * p.n + 255) / 256));
+        if (p.mode == TSATTN_MM_I32) hipLaunchKernelGGL((gemm_reduce_kernel<TSATTN_MM_I32>), grid, dim3(256), 0, st, r, (const int32_t *)p.workspace, split);
+        else if (p.mode == TSATTN_MM_F32) hipLaunchKernelGGL((gemm_reduce_kernel<TSATTN_MM_F32>), grid, dim3(256), 0, st, r, (const int32_t *)p.workspace, split);
+        else hipLaunchKernelGGL((gemm_reduce_kernel<TSATTN_MM_ADD_SCALED>), grid, dim3(256), 0, st, r, (const int32_t *)p.workspace, split);
+        return hipGetLastError();
+    }
     if (p.mode == TSATTN_MM_I32) launch_mode<TSATTN_MM_I32>(p, st);
     else if (p.mode == TSATTN_MM_F32) launch_mode<TSATTN_MM_F32>(p, st);
     else if (p.mode == TSATTN_MM_ADD_SCALED) launch_mode<TSATTN_MM_ADD_SCALED>(p, st);

@@ -107,6 +107,13 @@ struct ProduceParams {
     float *scale;
     int64_t scale_pitch, scale_row_stride;
     int relu;
+    int src_planes;
+    int64_t src_plane_stride;
+    int rope_heads;       // heads below it are rotated (set to n_heads when all are)
+    int scale_head_begin, scale_head_count;
+    float *resid;
+    int64_t resid_pitch;
+    float resid_scale;
 };
 
 hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head_dim, bool src_i32, hipStream_t st);
@@ -139,7 +146,7 @@ struct GemmParams {
     int64_t split_stride;     // set by the launcher: elements between the parts' planes
 };
 
-hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st);
+hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out);
 
 struct FillParams {
     const int32_t *seq_offset;

@@ -56,14 +56,27 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
         const int x0 = (c / 8) * 64 + (c % 8) * 4, x1 = x0 + 32;
         const int64_t e = s_row[pr] * p.src_pitch + (int64_t)s_head[pr] * D;
         if (SRC_I32) {
-            const v4i a = *(const v4i *)((const int32_t *)p.src + e + x0), b = *(const v4i *)((const int32_t *)p.src + e + x1);
+            v4i a = *(const v4i *)((const int32_t *)p.src + e + x0), b = *(const v4i *)((const int32_t *)p.src + e + x1);
+            for (int pl = 1; pl < p.src_planes; ++pl) { // the parts of a product whose K was split: exact integer sums
+                a += *(const v4i *)((const int32_t *)p.src + pl * p.src_plane_stride + e + x0);
+                b += *(const v4i *)((const int32_t *)p.src + pl * p.src_plane_stride + e + x1);
+            }
             v0[st] = v4f{(float)a.x, (float)a.y, (float)a.z, (float)a.w};
             v1[st] = v4f{(float)b.x, (float)b.y, (float)b.z, (float)b.w};
         } else {
             v0[st] = *(const v4f *)((const float *)p.src + e + x0);
             v1[st] = *(const v4f *)((const float *)p.src + e + x1);
         }
-        if (p.pos) {
+        if (p.resid) {
+            // state += delta * scale, written back; the updated state is what gets normalised
+            float *r0 = p.resid + s_row[pr] * p.resid_pitch + (int64_t)s_head[pr] * D + x0, *r1 = r0 + 32;
+            const v4f u0 = *(const v4f *)r0 + v0[st] * p.resid_scale, u1 = *(const v4f *)r1 + v1[st] * p.resid_scale;
+            *(v4f *)r0 = u0;
+            *(v4f *)r1 = u1;
+            v0[st] = u0;
+            v1[st] = u1;
+        }
+        if (p.pos && s_head[pr] < p.rope_heads) {
             const float *rr = p.rope + (int64_t)s_pos[pr] * D;
             cs[st] = *(const v4f *)(rr + x0);
             sn[st] = *(const v4f *)(rr + x1);
@@ -75,7 +88,7 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
         const int pr = j / PER_PAIR, c = j % PER_PAIR;
         if (pr >= n_here) continue;
         const int x0 = (c / 8) * 64 + (c % 8) * 4, x1 = x0 + 32;
-        if (p.pos) {
+        if (p.pos && s_head[pr] < p.rope_heads) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float cos_value = cs[st][i];
@@ -109,7 +122,8 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
             mult = 1.0f / discr;
         }
         mults[tid] = mult;
-        if (p.scale) p.scale[s_head[tid] * p.scale_pitch + s_row[tid] * p.scale_row_stride] = discr * p.scale_mult;
+        const int sh = s_head[tid] - p.scale_head_begin;
+        if (p.scale && sh >= 0 && sh < p.scale_head_count) p.scale[sh * p.scale_pitch + s_row[tid] * p.scale_row_stride] = discr * p.scale_mult;
     }
     __syncthreads();
 

@@ -223,18 +223,18 @@ TLayerComputer::TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, i
     const size_t n = (size_t)seqCount, qsum = (size_t)dims.GetQSum();
     auto alloc = [](void **p, size_t bytes) { CheckHip(hipMalloc(p, bytes), "hipMalloc(layer buffers)"); };
     alloc((void **)&NormState, n * dims.Dim);
-    alloc((void **)&Qk, n * qsum); alloc((void **)&Qv, n * qsum); alloc((void **)&K, n * qsum); alloc((void **)&V, n * qsum);
+    alloc((void **)&Q4, n * qsum * 4);
     alloc((void **)&Kv, n * qsum * COMBINER_REP);
     alloc((void **)&Relu, n * ReluDim);
-    alloc((void **)&QkSrc, n * qsum * 4); alloc((void **)&QvSrc, n * qsum * 4);
-    alloc((void **)&KSrc, n * qsum * 4); alloc((void **)&VSrc, n * qsum * 4);
-    alloc((void **)&ReluSrc, n * ReluDim * 4);
-    alloc((void **)&QvHeadScale, n * dims.HeadCount * 4); alloc((void **)&VHeadScale, n * dims.HeadCount * 4);
+    alloc((void **)&QvHeadScale, n * dims.HeadCount * 4);
+    alloc((void **)&VHeadScale, n * dims.HeadCount * 4);
     alloc((void **)&ValLookup, n * qsum * 4);
-    // room for the matrix products to split K (few rows): 16 planes of the widest result
-    size_t widest = qsum > (size_t)dims.Dim ? qsum : (size_t)dims.Dim;
+    // the int32 results of the matrix products: up to 16 planes (K split over workgroups) of the widest one
+    size_t widest = 4 * qsum > (size_t)dims.Dim ? 4 * qsum : (size_t)dims.Dim;
     if ((size_t)ReluDim > widest) widest = ReluDim;
-    WorkspaceBytes = (int64_t)(16 * 4 * n * widest);
+    PlaneElems = (int64_t)(n * widest);
+    alloc((void **)&Planes, (size_t)PlaneElems * 16 * 4);
+    WorkspaceBytes = (int64_t)(16 * 4 * n * dims.Dim);
     alloc(&Workspace, (size_t)WorkspaceBytes);
     // values carry the constant VEC_SCALE (cpu_infer.cpp:454)
     std::vector<float> vs(n * dims.HeadCount, VEC_SCALE);
@@ -243,7 +243,7 @@ TLayerComputer::TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, i
 
 TLayerComputer::~TLayerComputer()
 {
-    void *all[] = {NormState, Qk, Qv, K, V, Kv, Relu, QkSrc, QvSrc, KSrc, VSrc, ReluSrc, QvHeadScale, VHeadScale, ValLookup, Workspace};
+    void *all[] = {NormState, Q4, Kv, Relu, QvHeadScale, VHeadScale, ValLookup, Planes, Workspace};
     for (void *p : all) (void)hipFree(p);
 }
 
@@ -255,75 +255,114 @@ void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, in
     TS_VERIFY(kvCache.SeqCount == SeqCount && kvCache.HeadCount == headCount && kvCache.HeadDim == headDim && kvCache.DType == TSATTN_I8,
               "the KV cache does not match the layer (%d sequences, %d heads of %d, int8)", SeqCount, headCount, headDim);
 
-    // NormalizeState: per group of `groupDim` values, to int8; optionally rope first, the groups' scales, ReLU
-    auto normalize = [&](const void *src, bool srcI32, int groups, int groupDim, const int32_t *pos, uint8_t *dst, float *headScale,
-                         float scaleMult, bool relu) {
-        tsattn_produce_args a = {};
+    // MulForward, result left as int32 planes in Planes (their sum is the product); returns the number of planes
+    auto mulForward = [&](const uint8_t *vec, int k, const int8_t *matr, int n) {
+        tsattn_matmul_args a = {};
+        int planes = 0;
+        a.m = SeqCount; a.n = n; a.k = k;
+        a.a = vec; a.a_pitch = k; a.w = matr; a.w_pitch = k;
+        a.mode = TSATTN_MM_I32_PLANES; a.out = Planes; a.out_pitch = n; a.planes_out = &planes;
+        Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
+        return planes;
+    };
+    // NormalizeState on Planes or on a float array: per group of groupDim values, to int8
+    auto normalize = [&](tsattn_produce_args a, const void *src, bool srcI32, int planes, int groups, int groupDim, uint8_t *dst) {
         a.src_dtype = srcI32 ? TSATTN_SRC_I32 : TSATTN_SRC_F32;
         a.dst_dtype = TSATTN_I8;
         a.n_rows = SeqCount; a.n_heads = groups; a.head_dim = groupDim;
         a.src = src; a.src_pitch = (int64_t)groups * groupDim;
-        a.pos = pos; a.rope = pos ? ropeBuf : nullptr; a.rope_len = pos ? ropeLen : 0;
-        a.rotate_dir = 1; a.vec_scale = VEC_SCALE; a.scale_mult = scaleMult;
+        a.src_planes = planes; a.src_plane_stride = (int64_t)SeqCount * groups * groupDim;
+        a.rotate_dir = 1; a.vec_scale = VEC_SCALE;
+        if (a.scale_mult == 0) a.scale_mult = 1;
         a.dst = dst; a.dst_pitch = (int64_t)groups * groupDim;
-        a.scale = headScale; a.scale_pitch = 1; a.scale_row_stride = groups; // [seq][head], what the cache append reads
-        a.relu = relu ? 1 : 0;
         Check(tsattn_rope_normalize_rows(Handle, &a, stream), "tsattn_rope_normalize_rows");
     };
-    // MulForward / AddScaled
-    auto mulForward = [&](const uint8_t *vec, int k, const int8_t *matr, int n, int mode, float scale, void *res) {
-        tsattn_matmul_args a = {};
-        a.m = SeqCount; a.n = n; a.k = k;
-        a.a = vec; a.a_pitch = k; a.w = matr; a.w_pitch = k;
-        a.mode = mode; a.scale = scale; a.out = res; a.out_pitch = n;
-        a.workspace = Workspace; a.workspace_bytes = WorkspaceBytes;
-        Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
-    };
 
-    normalize(state, false, dim / STATE_NORM_TILE, STATE_NORM_TILE, nullptr, NormState, nullptr, 1, false);
-    mulForward(NormState, dim, att.QK, qsum, TSATTN_MM_F32, 1, QkSrc);
-    mulForward(NormState, dim, att.QV, qsum, TSATTN_MM_F32, 1, QvSrc);
-    mulForward(NormState, dim, att.K, qsum, TSATTN_MM_I32, 1, KSrc);
-    mulForward(NormState, dim, att.V, qsum, TSATTN_MM_I32, 1, VSrc);
-    normalize(QkSrc, false, headCount, headDim, t, Qk, nullptr, 1, false);
-    // the cached key scale takes the matrix scale: qvMult *= att.QVScale * VEC_SCALE * CalcDotScale(dim)
-    normalize(QvSrc, false, headCount, headDim, t, Qv, QvHeadScale, att.QVScale * VEC_SCALE * sqrtf(1.0f / (float)dim), false);
-    normalize(KSrc, true, headCount, headDim, nullptr, K, nullptr, 1, false);
-    normalize(VSrc, true, headCount, headDim, nullptr, V, nullptr, 1, false);
+    normalize({}, state, false, 1, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState);
 
-    // kvCache.AddVectors(qv, qvHeadScale, v) and ComputeValLookup(width, slope, dims, kvCache, qk, &valLookup) in one call
-    // (width 0 would make the token attend to the row being written: two calls then)
-    if (att.AttentionWidth == 0) {
-        kvCache.AddVectors(Qv, QvHeadScale, V, VHeadScale, stream);
-        ComputeValLookup(att.AttentionWidth, att.AlibiSlope, kvCache, Qk, nullptr, VEC_SCALE, ValLookup, stream);
+    // The four projections.  Matrices that lie one after the other in memory (QK, QV, K, V) are one product; the
+    // result rows hold the qk, qv, k and v heads in that order either way.
+    const size_t matBytes = (size_t)qsum * dim;
+    int planes = 1;
+    if ((const int8_t *)att.QV == att.QK + matBytes && att.K == att.QV + matBytes && att.V == att.K + matBytes) {
+        planes = mulForward(NormState, dim, att.QK, 4 * qsum);
     } else {
-        tsattn_decode_args a = {};
-        a.dtype = TSATTN_I8; a.q_dtype = TSATTN_Q_8BIT;
-        a.n_seqs = SeqCount; a.n_heads = headCount; a.head_dim = headDim;
-        a.q = Qk; a.q_pitch = qsum; a.q_scale = nullptr; a.q_scale_const = VEC_SCALE;
-        a.k_cache = kvCache.QVState; a.v_cache = kvCache.VState;
-        a.seq_stride = (int64_t)headCount * kvCache.MaxLen * headDim;
-        a.head_stride = (int64_t)kvCache.MaxLen * headDim;
-        a.tok_stride = headDim;
-        a.k_scale = kvCache.QVStateScale; a.v_scale = kvCache.VStateScale;
-        a.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; a.s_head_stride = kvCache.MaxLen;
-        a.cache_len = kvCache.Length; a.max_len = kvCache.MaxLen;
-        a.window = att.AttentionWidth; a.alibi_slope = att.AlibiSlope;
-        a.out = ValLookup;
-        a.k_new = Qv; a.v_new = V; a.new_pitch = qsum; a.k_scale_new = QvHeadScale; a.v_scale_new = VHeadScale;
-        Check(tsattn_decode(Handle, &a, stream), "tsattn_decode");
+        const int8_t *mats[4] = {att.QK, att.QV, att.K, att.V};
+        for (int i = 0; i < 4; ++i) {
+            tsattn_matmul_args a = {};
+            a.m = SeqCount; a.n = qsum; a.k = dim;
+            a.a = NormState; a.a_pitch = dim; a.w = mats[i]; a.w_pitch = dim;
+            a.mode = TSATTN_MM_I32; a.out = Planes + (size_t)i * qsum; a.out_pitch = 4 * qsum;
+            a.workspace = Workspace; a.workspace_bytes = WorkspaceBytes;
+            Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
+        }
     }
+    // ApplyRope on qk and qv, NormalizeState per head on all four, in one call; the cached key scale takes the matrix
+    // scale: qvMult *= att.QVScale * VEC_SCALE * CalcDotScale(dim)
+    {
+        tsattn_produce_args a = {};
+        a.pos = t; a.rope = ropeBuf; a.rope_len = ropeLen; a.rope_heads = 2 * headCount;
+        a.scale = QvHeadScale; a.scale_pitch = 1; a.scale_row_stride = headCount; // [seq][head], what the cache append reads
+        a.scale_head_begin = headCount; a.scale_head_count = headCount;
+        a.scale_mult = att.QVScale * VEC_SCALE * sqrtf(1.0f / (float)dim);
+        normalize(a, Planes, true, planes, 4 * headCount, headDim, Q4);
+    }
+    const uint8_t *qk = Q4, *qv = Q4 + qsum, *k = Q4 + 2 * (size_t)qsum, *v = Q4 + 3 * (size_t)qsum;
+    const int64_t pitch4 = 4 * (int64_t)qsum;
 
-    Check(tsattn_kv_product(Handle, SeqCount, headCount, headDim, COMBINER_REP, K, qsum, TSATTN_OUT_F32, ValLookup, qsum, 1.0f, Kv,
+    // kvCache.AddVectors(qv, qvHeadScale, v) and ComputeValLookup(width, slope, dims, kvCache, qk, &valLookup)
+    tsattn_decode_args da = {};
+    da.dtype = TSATTN_I8; da.q_dtype = TSATTN_Q_8BIT;
+    da.n_seqs = SeqCount; da.n_heads = headCount; da.head_dim = headDim;
+    da.q = qk; da.q_pitch = pitch4; da.q_scale = nullptr; da.q_scale_const = VEC_SCALE;
+    da.k_cache = kvCache.QVState; da.v_cache = kvCache.VState;
+    da.seq_stride = (int64_t)headCount * kvCache.MaxLen * headDim;
+    da.head_stride = (int64_t)kvCache.MaxLen * headDim;
+    da.tok_stride = headDim;
+    da.k_scale = kvCache.QVStateScale; da.v_scale = kvCache.VStateScale;
+    da.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; da.s_head_stride = kvCache.MaxLen;
+    da.cache_len = kvCache.Length; da.max_len = kvCache.MaxLen;
+    da.window = att.AttentionWidth; da.alibi_slope = att.AlibiSlope;
+    da.out = ValLookup;
+    if (att.AttentionWidth == 0) {
+        // the token attends to the row being written: append first, in its own call
+        tsattn_append_args aa = {};
+        aa.n_seqs = SeqCount; aa.n_heads = headCount; aa.head_dim = headDim;
+        aa.k_new = qv; aa.v_new = v; aa.new_pitch = pitch4; aa.k_scale_new = QvHeadScale; aa.v_scale_new = VHeadScale;
+        aa.k_cache = kvCache.QVState; aa.v_cache = kvCache.VState;
+        aa.seq_stride = da.seq_stride; aa.head_stride = da.head_stride; aa.tok_stride = da.tok_stride;
+        aa.k_scale = kvCache.QVStateScale; aa.v_scale = kvCache.VStateScale;
+        aa.s_seq_stride = da.s_seq_stride; aa.s_head_stride = da.s_head_stride;
+        aa.cache_len = kvCache.Length; aa.max_len = kvCache.MaxLen;
+        Check(tsattn_cache_append(Handle, &aa, stream), "tsattn_cache_append");
+    } else {
+        da.k_new = qv; da.v_new = v; da.new_pitch = pitch4; da.k_scale_new = QvHeadScale; da.v_scale_new = VHeadScale;
+    }
+    Check(tsattn_decode(Handle, &da, stream), "tsattn_decode");
+
+    Check(tsattn_kv_product(Handle, SeqCount, headCount, headDim, COMBINER_REP, k, pitch4, TSATTN_OUT_F32, ValLookup, qsum, 1.0f, Kv,
                             (int64_t)qsum * COMBINER_REP, stream), "tsattn_kv_product");
+    // combiner; its AddScaled is done by the normalisation that follows (state += delta * scale, then normalise)
     const int kvDim = qsum * COMBINER_REP;
-    mulForward(Kv, kvDim, att.Combiner, dim, TSATTN_MM_ADD_SCALED, att.CombinerScale * VEC_SCALE * sqrtf(1.0f / (float)kvDim), state);
-
+    planes = mulForward(Kv, kvDim, att.Combiner, dim);
+    {
+        tsattn_produce_args a = {};
+        a.resid = state; a.resid_pitch = dim; a.resid_scale = att.CombinerScale * VEC_SCALE * sqrtf(1.0f / (float)kvDim);
+        normalize(a, Planes, true, planes, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState);
+    }
     // relu
-    normalize(state, false, dim / STATE_NORM_TILE, STATE_NORM_TILE, nullptr, NormState, nullptr, 1, false);
-    mulForward(NormState, dim, att.Expand, ReluDim, TSATTN_MM_I32, 1, ReluSrc);
-    normalize(ReluSrc, true, headCount, ReluDim / headCount, nullptr, Relu, nullptr, 1, true);
-    mulForward(Relu, ReluDim, att.Contract, dim, TSATTN_MM_ADD_SCALED, att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim), state);
+    planes = mulForward(NormState, dim, att.Expand, ReluDim);
+    {
+        tsattn_produce_args a = {};
+        a.relu = 1;
+        normalize(a, Planes, true, planes, headCount, ReluDim / headCount, Relu);
+    }
+    tsattn_matmul_args ca = {};
+    ca.m = SeqCount; ca.n = dim; ca.k = ReluDim;
+    ca.a = Relu; ca.a_pitch = ReluDim; ca.w = att.Contract; ca.w_pitch = ReluDim;
+    ca.mode = TSATTN_MM_ADD_SCALED; ca.scale = att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim);
+    ca.out = state; ca.out_pitch = dim; ca.workspace = Workspace; ca.workspace_bytes = WorkspaceBytes;
+    Check(tsattn_matmul_i8(Handle, &ca, stream), "tsattn_matmul_i8");
 }
 
 } // namespace NTsAttn

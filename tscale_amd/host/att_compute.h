@@ -114,7 +114,6 @@ struct TAttentionVecHistory {
     float *QVStateScale = nullptr;
     float *VStateScale = nullptr;
     int32_t *Length = nullptr;         // device [seqCount]
-    float *SplitAcc = nullptr;
 
     TAttentionVecHistory(tsattn_handle_t handle, int dtype, int seqCount, int headCount, int maxLen, int headDim);
     ~TAttentionVecHistory();
@@ -147,16 +146,20 @@ constexpr int STATE_NORM_TILE = 128;   // gpt/model_params/model_dim.h:22
 constexpr int COMBINER_REP = 4;        // gpt/model_params/model_dim.h:12
 
 // AddLookupProduct for a batch: one new token per sequence, every sequence with its own state row and KV cache.
-// Owns the intermediate vectors (allocated once for seqCount sequences).  QDim == TTDim == 64 or 128; the feed-forward
+// Owns the intermediate vectors (allocated once for seqCount sequences).  11 or 12 launches per call: the four
+// projections are one product when QK, QV, K and V lie one after the other in memory, the normalisations that follow
+// them are one call, K-split products leave their parts for the consumer to add up, and the combiner's AddScaled is
+// done by the normalisation after it.  QDim == TTDim == 64 or 128; the feed-forward
 // width is reluDim = HeadCount * QDim (ReluMult 1 at QDim 128).
 class TLayerComputer
 {
     tsattn_handle_t Handle = nullptr;
     TModelDims Dims;
     int SeqCount = 0, ReluDim = 0;
-    uint8_t *NormState = nullptr, *Qk = nullptr, *Qv = nullptr, *K = nullptr, *V = nullptr, *Kv = nullptr, *Relu = nullptr;
-    float *QkSrc = nullptr, *QvSrc = nullptr, *QvHeadScale = nullptr, *VHeadScale = nullptr, *ValLookup = nullptr;
-    int32_t *KSrc = nullptr, *VSrc = nullptr, *ReluSrc = nullptr;
+    uint8_t *NormState = nullptr, *Q4 = nullptr, *Kv = nullptr, *Relu = nullptr; // Q4: rows of qk, qv, k, v heads
+    float *QvHeadScale = nullptr, *VHeadScale = nullptr, *ValLookup = nullptr;
+    int32_t *Planes = nullptr; // int32 results of the matrix products, up to 16 planes
+    int64_t PlaneElems = 0;
     void *Workspace = nullptr;
     int64_t WorkspaceBytes = 0;
 
