@@ -322,41 +322,59 @@ def bench_matmul(ctx, steps):
     return res
 
 
+class Int8Layers:
+    """24 layers of the int8 inference path (AddLookupProduct, gpt/train/cpu_infer.cpp:465-527) at the 1.5B-style
+    attention shape: model width 2048, 16 heads x 128, feed-forward width 2048, per-layer attention width and slope
+    from InitAlibi's schedule, random int8 weights of rms 32 (what the reference's matrix conversion leaves,
+    MODEL_DISCR_SCALE = 1/32), one KV cache per layer for B = 32 sequences.  Embedding, final layer and sampling are
+    not part of it."""
+
+    def __init__(self, ctx, cache_len, seed):
+        import torch
+        from tscale_amd import KVCache, capi
+        from tscale_amd.attention import alibi_layer_schedule, VEC_SCALE
+        self.ctx = ctx
+        self.B, self.H, self.d, self.dim, self.depth, self.prompt, self.n_new = 32, 16, 128, 2048, 24, 2048, 64
+        self.L = self.prompt + self.n_new
+        qsum = self.H * self.d
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        self.g = g
+        def matrix(n, k):
+            return (torch.randn((n, k), device="cuda", generator=g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
+        self.sched = alibi_layer_schedule(self.depth, self.L)
+        self.layers, self.caches = [], []
+        for w, slope in self.sched:
+            self.layers.append({"proj": matrix(4 * qsum, self.dim), "combiner": matrix(self.dim, qsum * 4),
+                                "expand": matrix(qsum, self.dim), "contract": matrix(self.dim, qsum),
+                                "qv_scale": 0.03, "combiner_scale": 0.03, "contract_scale": 0.03, "width": w, "slope": slope})
+            c = KVCache(ctx, capi.I8, self.B, self.H, self.L, self.d)
+            if cache_len > 0:   # a cache that already holds a prompt: random rows
+                c.k.copy_((torch.randn(c.k.shape, device="cuda", generator=g) * 24).round().clamp(-127, 127).to(torch.int8).view(torch.uint8))
+                c.v.copy_((torch.randn(c.v.shape, device="cuda", generator=g) * 24).round().clamp(-127, 127).to(torch.int8).view(torch.uint8))
+                c.k_scale.copy_((torch.rand(c.k_scale.shape, device="cuda", generator=g) + 0.5) * 1e-4)
+            c.v_scale.fill_(VEC_SCALE)
+            c.cache_len.fill_(cache_len)
+            self.caches.append(c)
+        self.rope = ctx.fill_rope_table(self.d, self.L)
+        self.weight_bytes = sum(sum(v.numel() for v in layer.values() if isinstance(v, torch.Tensor)) for layer in self.layers)
+        self.matmul_ops_per_token = 2.0 * sum(sum(v.numel() for v in layer.values() if isinstance(v, torch.Tensor)) for layer in self.layers)
+
+
 def bench_token_step(ctx, steps):
-    """One generated token per sequence through all 24 layers of the int8 inference path (AddLookupProduct,
-    gpt/train/cpu_infer.cpp:465-527, per layer: state normalisation, four projections, RoPE + per-head normalisation,
-    cache append + attention over the cache, KVProduct, combiner, feed-forward; 11-12 library calls), B32 at cache length 2048+, model width
-    2048, 16 heads x 128, random int8 weights.  Embedding, final layer and sampling are not part of it."""
+    """One generated token per sequence through all 24 layers (per layer: state normalisation, four projections,
+    RoPE + per-head normalisation, cache append + attention over the cache, KVProduct, combiner, feed-forward; 11-12
+    library calls), B32 at cache length 2048+."""
     import torch
-    from tscale_amd import KVCache, capi
-    from tscale_amd.attention import add_lookup_product, alibi_layer_schedule, VEC_SCALE
-    B, H, d, dim, depth, prompt, n_new = 32, 16, 128, 2048, 24, 2048, 64
-    L = prompt + n_new
-    qsum = H * d
-    g = torch.Generator(device="cuda").manual_seed(1313 + 9)
-    def matrix(n, k):   # int8 of rms 32, what the reference's matrix conversion leaves (MODEL_DISCR_SCALE = 1/32)
-        return (torch.randn((n, k), device="cuda", generator=g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
-    sched = alibi_layer_schedule(depth, L)
-    layers, caches = [], []
-    for w, slope in sched:
-        layers.append({"proj": matrix(4 * qsum, dim),
-                       "combiner": matrix(dim, qsum * 4), "expand": matrix(qsum, dim), "contract": matrix(dim, qsum),
-                       "qv_scale": 0.03, "combiner_scale": 0.03, "contract_scale": 0.03, "width": w, "slope": slope})
-        c = KVCache(ctx, capi.I8, B, H, L, d)
-        c.k.copy_(torch.randint(0, 256, c.k.shape, dtype=torch.uint8, device="cuda", generator=g))
-        c.v.copy_(torch.randint(0, 256, c.v.shape, dtype=torch.uint8, device="cuda", generator=g))
-        c.k_scale.copy_((torch.rand(c.k_scale.shape, device="cuda", generator=g) + 0.5) * 1e-4)
-        c.v_scale.fill_(VEC_SCALE)
-        c.cache_len.fill_(prompt)
-        caches.append(c)
-    rope = ctx.fill_rope_table(d, L)
-    state = torch.randn((B, dim), device="cuda", generator=g)
-    t = torch.full((B,), prompt, dtype=torch.int32, device="cuda")
+    from tscale_amd.attention import add_lookup_product
+    m = Int8Layers(ctx, cache_len=2048, seed=1313 + 9)
+    B, H, d, dim, qsum = m.B, m.H, m.d, m.dim, m.H * m.d
+    state = torch.randn((B, dim), device="cuda", generator=m.g)
+    t = torch.full((B,), m.prompt, dtype=torch.int32, device="cuda")
     room = torch.empty(16 * 4 * B * max(dim, qsum), dtype=torch.uint8, device="cuda")
     keep = {}
     def step():
-        for layer, c in zip(layers, caches):
-            add_lookup_product(ctx, layer, c, t, rope, state, workspace=room, scratch=keep)
+        for layer, c in zip(m.layers, m.caches):
+            add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep)
         t.add_(1)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -368,18 +386,48 @@ def bench_token_step(ctx, steps):
     with torch.cuda.graph(graph):
         step()
     torch.cuda.synchronize()
-    reps = min(n_new - 2, max(10, steps))
+    reps = min(m.n_new - 2, max(10, steps))
     ms = gpu_time_ms(graph.replay, reps, 0)
     assert bool(torch.isfinite(state).all())
-    weight_bytes = sum(sum(v.numel() for v in layer.values() if isinstance(v, torch.Tensor)) for layer in layers)
-    n = prompt + 1 + reps // 2
-    cache_bytes = sum(B * H * min(n - 1, w) * (2 * d + 8) for w, _ in sched)
+    n = m.prompt + 1 + reps // 2
+    cache_bytes = sum(B * H * min(n - 1, w) * (2 * d + 8) for w, _ in m.sched)
     return {"config": "24 layers, B32, cache length ~2048+, model width 2048, 16 heads x 128, int8 weights and KV cache; "
                       "11-12 library calls per layer in one HIP graph per token",
             "ms_per_token_step": round(ms, 4), "tokens_per_s": round(B / ms * 1e3, 1),
-            "weight_bytes": weight_bytes, "cache_bytes_per_step": cache_bytes,
-            "GB/s": round((weight_bytes + cache_bytes) / ms / 1e6, 1),
-            "frac_of_hbm_peak": round((weight_bytes + cache_bytes) / ms / 1e6 / PEAK_HBM_GBPS, 4)}
+            "weight_bytes": m.weight_bytes, "cache_bytes_per_step": cache_bytes,
+            "GB/s": round((m.weight_bytes + cache_bytes) / ms / 1e6, 1),
+            "frac_of_hbm_peak": round((m.weight_bytes + cache_bytes) / ms / 1e6 / PEAK_HBM_GBPS, 4)}
+
+
+def bench_prompt_pass(ctx, steps):
+    """The prompt of the same configuration through the same 24 layers in batch form (add_lookup_product_prompt):
+    32 x 2048 tokens, per layer one prefill attention launch, one cache fill, seven matrix products in four calls."""
+    import torch
+    from tscale_amd.attention import add_lookup_product_prompt
+    m = Int8Layers(ctx, cache_len=0, seed=1313 + 10)
+    B, H, d, dim = m.B, m.H, m.d, m.dim
+    n = B * m.prompt
+    off = torch.arange(0, n + 1, m.prompt, dtype=torch.int32, device="cuda")
+    pos = torch.arange(m.prompt, dtype=torch.int32, device="cuda").repeat(B)
+    spans = {w: ctx.build_spans(off, n, w) for w in {w for w, _ in m.sched}}
+    tiles = {w: ctx.build_span_tiles(*sp) for w, sp in spans.items()}
+    state0 = torch.randn((n, dim), device="cuda", generator=m.g)
+    state = torch.empty_like(state0)
+    def run():
+        state.copy_(state0)
+        for layer, c in zip(m.layers, m.caches):
+            c.cache_len.zero_()
+            w = layer["width"]
+            add_lookup_product_prompt(ctx, layer, c, off, pos, m.rope, state, *spans[w], span_tiles=tiles[w],
+                                      causal_period=m.prompt if w >= m.prompt else 0)
+    ms = gpu_time_ms(run, 2, 1)
+    assert bool(torch.isfinite(state).all()) and int(m.caches[0].cache_len[0]) == m.prompt
+    att_flops = sum(prefill_flops(B, m.prompt, H, d, w) for w, _ in m.sched)
+    mm_ops = m.matmul_ops_per_token * n
+    return {"config": "24 layers, B32 x 2048 prompt tokens, model width 2048, 16 heads x 128, int8; batch form of the layer",
+            "ms": round(ms, 3), "tokens_per_s": round(n / ms * 1e3, 1),
+            "matmul_TOP": round(mm_ops / 1e12, 2), "attention_TOP": round(att_flops / 1e12, 2),
+            "TOP/s": round((mm_ops + att_flops) / ms / 1e9, 1), "frac_of_int8_peak": round((mm_ops + att_flops) / ms / 1e9 / PEAK_I8_TOPS, 4)}
 
 
 def cpu_baseline_prefill(wl, n_seq_sample):
@@ -457,6 +505,9 @@ def run_only(ctx, args):
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
+    if name == "prompt-pass":
+        print(json.dumps({"only": name, **bench_prompt_pass(ctx, args.steps)}))
+        return
     if name == "token-step":
         print(json.dumps({"only": name, **bench_token_step(ctx, args.steps)}))
         return
@@ -494,7 +545,7 @@ def main():
     ap.add_argument("--extra", action="store_true",
                     help="also time the 1.5B-style prefill shapes and the attention share of the 1.5B-style generation run")
     ap.add_argument("--only", default=None,
-                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step"],
+                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step", "prompt-pass"],
                     help="profiling aid: run just this launch --steps times and print its timing")
     ap.add_argument("--calibrate", action="store_true",
                     help="with --only: first run three 256 MiB device copies (counter calibration)")
@@ -581,6 +632,7 @@ def main():
         result["kv_product"] = bench_kv_product(ctx, args.steps)
         result["combiner_matmul"] = bench_matmul(ctx, args.steps)
         result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
+        result["prompt_pass_24_layers"] = bench_prompt_pass(ctx, args.steps)
     print(json.dumps(result))
 
 

@@ -278,7 +278,8 @@ enum tsattn_mm_mode {
     TSATTN_MM_F32 = 1,        /* out (f32) = (float)sum * scale   (MulForward into TVector<float>: scale 1) */
     TSATTN_MM_ADD_SCALED = 2, /* out (f32) += (float)sum * scale  (AddScaled) */
     /* out (int32 [planes][m][n], n = out_pitch) = partial sums whose total over the planes is the product; *planes_out
-     * (host memory) receives their number, at most 16, 1 unless K was split (few rows, out holds 16 * m * n ints).
+     * (host memory) receives their number: 1 with more than 128 rows (out holds m * n ints), up to 16 with fewer (K may
+     * be split; out holds 16 * m * n ints).
      * For a consumer that adds the planes up itself (tsattn_rope_normalize_rows with src_planes) and so saves the
      * launch that would. */
     TSATTN_MM_I32_PLANES = 3,

@@ -67,3 +67,57 @@ def test_layer_steps_match_the_oracle(ctx, H, d, dim, width, slope):
         exact_steps += int(np.array_equal(got, want))
     assert lens.tolist() == [min(max_len, l + steps) for l in (0, 2, 7, 9)]
     assert exact_steps >= steps // 2, "most steps come out bit-identical"
+
+
+@pytest.mark.parametrize("width,slope", [(1000, 0.0), (16, 0.5)])
+def test_prompt_layer_equals_the_oracle_token_by_token(ctx, width, slope):
+    """A batch of prompt tokens through add_lookup_product_prompt (one prefill launch, one cache fill) against the oracle
+    fed one token at a time: same cache bytes and key scales, attention output within the prefill tolerance, states the
+    same up to flips of int8 roundings."""
+    from tscale_amd.attention import add_lookup_product_prompt
+    H, d, dim, max_len = 2, 128, 256, 64
+    seq_lens = [37, 50, 1]
+    B, n = len(seq_lens), sum(seq_lens)
+    qsum = H * d
+    rng = np.random.default_rng(width)
+    mat = lambda r, k: np.clip(np.rint(rng.standard_normal((r, k)) * 32), -127, 127).astype(np.int8)
+    mats = {"qk": mat(qsum, dim), "qv": mat(qsum, dim), "k": mat(qsum, dim), "v": mat(qsum, dim),
+            "combiner": mat(dim, qsum * 4), "expand": mat(qsum, dim), "contract": mat(dim, qsum)}
+    scales = (0.031, 0.027, 0.035)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    layer = {"proj": dev(np.concatenate([mats[m] for m in ("qk", "qv", "k", "v")]).view(np.uint8)),
+             "combiner": dev(mats["combiner"].view(np.uint8)), "expand": dev(mats["expand"].view(np.uint8)),
+             "contract": dev(mats["contract"].view(np.uint8)), "qv_scale": scales[0], "combiner_scale": scales[1],
+             "contract_scale": scales[2], "width": width, "slope": slope}
+    rope_np = orc.fill_rope(d, max_len)
+    state0 = rng.standard_normal((n, dim)).astype(np.float32) * 2
+    # oracle: every sequence on its own, token after token
+    kc = np.zeros((B, H, max_len, d), dtype=np.uint8); vc = np.zeros_like(kc)
+    ksc = np.zeros((B, H, max_len), dtype=np.float32)
+    want = np.empty_like(state0); want_val = np.empty((n, qsum), dtype=np.float32)
+    off = np.concatenate([[0], np.cumsum(seq_lens)])
+    for b in range(B):
+        lens = np.zeros(1, dtype=np.int32)
+        for p_ in range(seq_lens[b]):
+            tok = off[b] + p_
+            o, v_ = orc.add_lookup_product(mats, scales, width, slope, H, d, np.array([p_], dtype=np.int32), rope_np,
+                                           state0[tok:tok + 1], kc[b:b + 1], vc[b:b + 1], ksc[b:b + 1], lens)
+            want[tok], want_val[tok] = o[0], v_[0]
+    # GPU: the whole batch at once
+    cache = KVCache(ctx, capi.I8, B, H, max_len, d)
+    cache.v_scale.fill_(VEC_SCALE)
+    seq_offset = dev(off.astype(np.int32))
+    pos = dev(np.concatenate([np.arange(l) for l in seq_lens]).astype(np.int32))
+    st, fi = ctx.build_spans(seq_offset, n, width)
+    state = dev(state0)
+    val = add_lookup_product_prompt(ctx, layer, cache, seq_offset, pos, dev(rope_np), state, st, fi)
+    torch.cuda.synchronize()
+    assert cache.cache_len.cpu().numpy().tolist() == seq_lens
+    assert np.array_equal(cache.k.cpu().numpy(), kc) and np.array_equal(cache.v.cpu().numpy(), vc)
+    assert np.array_equal(cache.k_scale.cpu().numpy(), ksc)
+    from tests.common import assert_within_tolerance
+    assert_within_tolerance(val.cpu().numpy(), want_val, "attention output of the prompt")
+    got = state.cpu().numpy()
+    rms = np.sqrt((want.astype(np.float64) ** 2).mean())
+    assert np.abs(got - want).max() / rms < 5e-2
+    assert np.sqrt(((got - want).astype(np.float64) ** 2).mean()) / rms < 5e-3

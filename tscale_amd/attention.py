@@ -150,9 +150,10 @@ class AttentionContext:
         assert w.shape[1] == k and a.stride(1) == 1 and w.stride(1) == 1
         if mode == capi.MM_I32_PLANES:
             # partial sums [planes, m, n] for a consumer that adds them up (rope_normalize_rows); returns the planes in use
+            room = (16 if m <= 128 else 1) * m * n    # K is split only for few rows
             if out is None:
-                out = torch.empty((16, m, n), dtype=torch.int32, device=a.device)
-            assert out.is_contiguous() and out.dtype == torch.int32 and out.numel() >= 16 * m * n
+                out = torch.empty(room, dtype=torch.int32, device=a.device)
+            assert out.is_contiguous() and out.dtype == torch.int32 and out.numel() >= room
             args = capi.MatmulArgs()
             args.m, args.n, args.k = m, n, k
             args.a, args.a_pitch = _ptr(a), a.stride(0)
@@ -309,6 +310,43 @@ def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None, scratc
     relu, _ = ctx.rope_normalize_rows(relu_src, H, capi.I8, relu=True)
     relu_dim = relu_src.shape[-1]
     ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state, workspace=workspace,
+                  scale=float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim)))))
+    return val
+
+
+def add_lookup_product_prompt(ctx, layer, cache, seq_offset, pos, rope, state, span_start, span_finish, span_tiles=None,
+                              causal_period=0):
+    """The same layer for a whole batch of prompt tokens at once (sequences concatenated, seq_offset int32 [B+1], pos
+    int32 [n_tokens] = each token's position in its sequence): every token's attention over the earlier tokens of its
+    sequence is one tsattn_prefill launch, and the tokens' key and value rows go into the cache in one
+    tsattn_cache_fill.  Token by token through add_lookup_product gives the same cache and the same states (a token's
+    layer input does not depend on other tokens' outputs of the same layer).  state: f32 [n_tokens, dim], updated in
+    place; the spans are those of the layer's width (build_spans).  Returns the attention output."""
+    n, dim = state.shape
+    H, d = cache.n_heads, cache.head_dim
+    qsum = H * d
+    groups = dim // STATE_NORM_TILE
+    f32 = np.float32
+    norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
+    proj = ctx.matmul_i8(norm, layer["proj"], mode=capi.MM_I32_PLANES)
+    key_mult = float(f32(layer["qv_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(dim))))
+    q4, qv_scale = ctx.rope_normalize_rows(proj, 4 * H, capi.I8, pos=pos, rope=rope, scale_mult=key_mult,
+                                           rope_heads=2 * H, scale_heads=(H, H))      # scales as [head][token] planes
+    del proj
+    qk, qv, k, v = q4[:, :qsum], q4[:, qsum:2 * qsum], q4[:, 2 * qsum:3 * qsum], q4[:, 3 * qsum:]
+    val = ctx.compute_val_lookup(capi.I8, H, qk, qv, v, VEC_SCALE, qv_scale, VEC_SCALE, span_start, span_finish, layer["slope"],
+                                 span_tiles=span_tiles, causal_period=causal_period)
+    cache.fill_from_prefill(seq_offset, qv, qv_scale, v)       # value scales: the cache's constant VEC_SCALE
+    kv = ctx.kv_product(k, val, H, COMBINER_REP)
+    delta = ctx.matmul_i8(kv, layer["combiner"], mode=capi.MM_I32_PLANES)
+    norm, _ = ctx.rope_normalize_rows(delta, groups, capi.I8, resid=state,
+                                      resid_scale=float(f32(layer["combiner_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(qsum * COMBINER_REP)))))
+    del delta, kv
+    relu_src = ctx.matmul_i8(norm, layer["expand"], mode=capi.MM_I32_PLANES)
+    relu, _ = ctx.rope_normalize_rows(relu_src, H, capi.I8, relu=True)
+    relu_dim = relu_src.shape[-1]
+    del relu_src
+    ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state,
                   scale=float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim)))))
     return val
 
