@@ -399,6 +399,58 @@ def bench_token_step(ctx, steps):
             "frac_of_hbm_peak": round((m.weight_bytes + cache_bytes) / ms / 1e6 / PEAK_HBM_GBPS, 4)}
 
 
+def bench_generate_model(ctx, steps):
+    """Greedy generation with the whole int8 model on the device (ComputePrediction, gpt/train/cpu_infer.cpp:552-582):
+    embedding of the previous choice -> 24 layers -> final normalisation, final-layer product (50257 x 2048), softmax
+    and greedy choice, which is the next step's label; one HIP graph per token, B32 at cache length 2048+."""
+    import numpy as np
+    import torch
+    from tscale_amd import capi
+    from tscale_amd.attention import add_lookup_product, VEC_SCALE, STATE_NORM_TILE
+    m = Int8Layers(ctx, cache_len=2048, seed=1313 + 11)
+    B, H, d, dim, qsum = m.B, m.H, m.d, m.dim, m.H * m.d
+    vocab = 50257
+    def matrix(n, k):
+        return (torch.randn((n, k), device="cuda", generator=m.g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
+    embed, final = matrix(vocab, dim), matrix(vocab, dim)
+    bias = torch.randn(vocab, device="cuda", generator=m.g) * 0.1
+    f32 = np.float32
+    final_scale = float(f32(np.sqrt(f32(1.0) / f32(dim))) * (f32(1.0) / f32(0.693147)) * f32(0.03) * f32(VEC_SCALE))
+    labels = torch.randint(0, vocab, (B,), dtype=torch.int32, device="cuda", generator=m.g)
+    state = torch.empty((B, dim), dtype=torch.float32, device="cuda")
+    t = torch.full((B,), m.prompt, dtype=torch.int32, device="cuda")
+    room = torch.empty(16 * 4 * B * max(dim, qsum), dtype=torch.uint8, device="cuda")
+    planes = torch.empty(16 * B * vocab, dtype=torch.int32, device="cuda")
+    keep = {}
+    def step():
+        ctx.embed_rows(labels, embed, 0.03, out=state)
+        for layer, c in zip(m.layers, m.caches):
+            add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep)
+        norm, _ = ctx.rope_normalize_rows(state, dim // STATE_NORM_TILE, capi.I8)
+        logits = ctx.matmul_i8(norm, final, mode=capi.MM_I32_PLANES, out=planes)
+        ctx.softmax_rows(logits, final_scale, bias, want_prob=False, argmax=labels)
+        t.add_(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    torch.cuda.synchronize()
+    reps = min(m.n_new - 2, max(10, steps))
+    first = labels.clone()
+    ms = gpu_time_ms(graph.replay, reps, 0)
+    assert bool(torch.isfinite(state).all()) and int(labels.min()) >= 0 and int(labels.max()) < vocab
+    head_bytes = final.numel() + B * dim
+    return {"config": "greedy generation, whole int8 model on the device: embedding, 24 layers, final layer 50257 x 2048, softmax, "
+                      "argmax fed back; B32, cache length ~2048+; one HIP graph per token",
+            "ms_per_token_step": round(ms, 4), "tokens_per_s": round(B / ms * 1e3, 1),
+            "weight_bytes": m.weight_bytes + head_bytes, "choices_changed": bool((labels != first).any())}
+
+
 def bench_prompt_pass(ctx, steps):
     """The prompt of the same configuration through the same 24 layers in batch form (add_lookup_product_prompt):
     32 x 2048 tokens, per layer one prefill attention launch, one cache fill, seven matrix products in four calls."""
@@ -505,6 +557,9 @@ def run_only(ctx, args):
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
+    if name == "generate-model":
+        print(json.dumps({"only": name, **bench_generate_model(ctx, args.steps)}))
+        return
     if name == "prompt-pass":
         print(json.dumps({"only": name, **bench_prompt_pass(ctx, args.steps)}))
         return
@@ -545,7 +600,7 @@ def main():
     ap.add_argument("--extra", action="store_true",
                     help="also time the 1.5B-style prefill shapes and the attention share of the 1.5B-style generation run")
     ap.add_argument("--only", default=None,
-                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step", "prompt-pass"],
+                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step", "prompt-pass", "generate-model"],
                     help="profiling aid: run just this launch --steps times and print its timing")
     ap.add_argument("--calibrate", action="store_true",
                     help="with --only: first run three 256 MiB device copies (counter calibration)")
@@ -633,6 +688,7 @@ def main():
         result["combiner_matmul"] = bench_matmul(ctx, args.steps)
         result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
         result["prompt_pass_24_layers"] = bench_prompt_pass(ctx, args.steps)
+        result["generate_whole_model"] = bench_generate_model(ctx, args.steps)
     print(json.dumps(result))
 
 

@@ -305,6 +305,22 @@ typedef struct tsattn_matmul_args {
 
 int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *stream);
 
+/* The two ends of ComputePrediction (gpt/train/cpu_infer.cpp:552-582) around the layers.
+ *
+ * tsattn_embed_rows: state[row][x] = sum over the row's labels of embed[label][x] * embed_scale, added in label order
+ * (:559-565).  labels: int32 [n_rows][labels_per_row], entries outside [0, n_labels) are empty slots; embed: int8
+ * [n_labels][embed_pitch bytes]; dim a multiple of 16; state f32 [n_rows][state_pitch], 16-byte aligned.
+ *
+ * tsattn_softmax_rows: the final SoftMax (:340-355 with TSoftMaxBuf :220-281, base 2): w[k] = vec[k] * scale + bias[k],
+ * prob[k] = 2^(w[k] - M) / sum, M = max(0, max w); argmax[row] = the first k of the largest w (the greedy choice).
+ * vec: int32 [n_rows][src_pitch], optionally the sum of src_planes arrays src_plane_stride elements apart
+ * (TSATTN_MM_I32_PLANES); bias f32 [n] or NULL; prob f32 [n_rows][prob_pitch] or NULL; argmax int32 [n_rows] or NULL. */
+int tsattn_embed_rows(tsattn_handle_t h, int64_t n_rows, int dim, const int32_t *labels, int labels_per_row, const void *embed,
+                      int64_t embed_pitch, int64_t n_labels, float embed_scale, float *state, int64_t state_pitch, void *stream);
+int tsattn_softmax_rows(tsattn_handle_t h, int64_t n_rows, int64_t n, const int32_t *src, int src_planes, int64_t src_plane_stride,
+                        int64_t src_pitch, float scale, const float *bias, float *prob, int64_t prob_pitch, int32_t *argmax,
+                        void *stream);
+
 /* The table ApplyRope reads: FillRopeBuf, gpt/att/rope.cpp:4-24.  Host function, host memory:
  * table[t * head_dim + x], t < max_len; copy it to the device once. */
 void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table);

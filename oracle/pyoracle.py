@@ -246,6 +246,30 @@ def add_lookup_product(mats, scales, width, slope, head_count, head_dim, t, rope
     return out, val
 
 
+def embed_rows(labels, embed, scale):
+    """labels int32 [n_rows] or [n_rows, L]; embed int8 [n_labels, dim] -> float32 [n_rows, dim]."""
+    L = lib()
+    labels = _c_arr(np.asarray(labels).reshape(len(labels), -1), np.int32)
+    embed = _c_arr(np.asarray(embed).view(np.int8), np.int8)
+    n_rows, per_row = labels.shape
+    n_labels, dim = embed.shape
+    out = np.empty((n_rows, dim), dtype=np.float32)
+    L.tso_embed_rows(ctypes.c_int64(n_rows), int(dim), _p(labels), int(per_row), _p(embed), ctypes.c_int64(n_labels), ctypes.c_float(scale), _p(out))
+    return out
+
+
+def softmax_rows(vec, scale, bias=None, exp2_mode=0):
+    """vec int32 [n_rows, n] -> (prob float32 [n_rows, n], argmax int32 [n_rows])."""
+    L = lib()
+    vec = _c_arr(vec, np.int32)
+    n_rows, n = vec.shape
+    b = None if bias is None else _c_arr(bias, np.float32)
+    prob = np.empty((n_rows, n), dtype=np.float32)
+    arg = np.empty(n_rows, dtype=np.int32)
+    L.tso_softmax_rows(ctypes.c_int64(n_rows), ctypes.c_int64(n), _p(vec), ctypes.c_float(scale), _p(b), int(exp2_mode), _p(prob), _p(arg))
+    return prob, arg
+
+
 def make_spans(seq_lens, window, doc_start_flag=None):
     L = lib()
     off = np.zeros(len(seq_lens) + 1, dtype=np.int64)

@@ -52,6 +52,10 @@
  *                                                         update is linear in the two matrix scales): the order of
  *                                                         the steps and which scale goes where were checked by
  *                                                         reading -- parity unpinned beyond its parts
+ *   tso_embed_rows         train/cpu_infer.cpp:559-565   pinned: numpy gather and sum
+ *   tso_softmax_rows       train/cpu_infer.cpp:340-355   pinned: scipy's softmax on ln 2 * w (a library routine), rows
+ *                                                         sum to 1, adding a constant to the bias changes nothing
+ *                                                         while the largest w stays above 0
  *
  * The reference holds no golden vectors or known-answer tests for this path, and the two files
  * that contain it (gpt_cpu.cpp, cpu_infer.cpp) cannot be compiled without the CUDA SDK, so the
@@ -941,4 +945,49 @@ void tso_add_lookup_product(const tso_layer_params *L, int64_t n_seq, const int3
 
     free(norm); free(qk_src); free(qv_src); free(k_src); free(v_src); free(qk); free(qv); free(k); free(v);
     free(qv_head_scale); free(val); free(kv); free(relu_src); free(relu);
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* embedding and final softmax (train/cpu_infer.cpp:552-582)                                  */
+
+void tso_embed_rows(int64_t n_rows, int dim, const int32_t *labels, int labels_per_row, const int8_t *embed, int64_t n_labels,
+                    float scale, float *state)
+{
+    for (int64_t r = 0; r < n_rows; ++r) {
+        float *st = state + r * dim;
+        for (int x = 0; x < dim; ++x) st[x] = 0; /* ClearPodArray(&state, dim) */
+        for (int l = 0; l < labels_per_row; ++l) {
+            int32_t label = labels[r * labels_per_row + l];
+            if (label < 0 || label >= n_labels) continue;
+            for (int x = 0; x < dim; ++x) {
+                st[x] += embed[(int64_t)label * dim + x] * scale; /* state[x] += LabelEmbed[label][x] * LabelEmbedScale */
+            }
+        }
+    }
+}
+
+void tso_softmax_rows(int64_t n_rows, int64_t n, const int32_t *vec, float scale, const float *bias, int exp2_mode, float *prob,
+                      int32_t *argmax)
+{
+    int64_t cap = ((n + 7) / 8) * 8;
+    if (cap < 8) cap = 8;
+    float *buf = (float *)malloc(sizeof(float) * (size_t)cap);
+    for (int64_t r = 0; r < n_rows; ++r) {
+        float max_value = 0; /* a fresh TSoftMaxBuf: MaxValue = 0 */
+        float best = -INFINITY;
+        int32_t arg = 0;
+        for (int64_t i = n; i < cap; ++i) buf[i] = -1e38f;
+        for (int64_t k = 0; k < n; ++k) {
+            float w = vec[r * n + k] * scale + (bias ? bias[k] : 0.0f); /* vec[k] * vecScale + bias[k] */
+            buf[k] = w;
+            max_value = (max_value > w) ? max_value : w;
+            if (w > best) { best = w; arg = (int32_t)k; }
+        }
+        if (argmax) argmax[r] = arg;
+        if (prob) {
+            float sc = softmax_buf_inplace(buf, (int)n, max_value, exp2_mode);
+            for (int64_t k = 0; k < n; ++k) prob[r * n + k] = buf[k] * sc;
+        }
+    }
+    free(buf);
 }

@@ -139,6 +139,16 @@ void tso_add_lookup_product(const tso_layer_params *L, int64_t n_seq, const int3
                             float *k_scale_cache, int64_t s_seq_stride, int64_t s_head_stride, int32_t *cache_len, int max_len,
                             float *val_lookup, int n_threads);
 
+/* ---- the two ends of ComputePrediction around the layers (train/cpu_infer.cpp:552-582) ----
+ * tso_embed_rows: state[row][x] = sum over the row's labels of embed[label][x] * scale, in label order (:559-565);
+ * labels outside [0, n_labels) are empty slots.
+ * tso_softmax_rows: SoftMax (:340-355): w[k] = vec[k] * scale + bias[k] through the softmax buffer (exp2_mode as in
+ * tso_decode), prob[k] = Buf[k] * Scale; argmax = the first index of the largest w.  bias, prob, argmax nullable. */
+void tso_embed_rows(int64_t n_rows, int dim, const int32_t *labels, int labels_per_row, const int8_t *embed, int64_t n_labels,
+                    float scale, float *state);
+void tso_softmax_rows(int64_t n_rows, int64_t n, const int32_t *vec, float scale, const float *bias, int exp2_mode, float *prob,
+                      int32_t *argmax);
+
 /* softmax buffer of cpu_infer.cpp:220-281 on its own (for bounding the polynomial):
  * in: n logits (the caller includes the leading 0 if wanted); out: n weights already multiplied by
  * Scale.  Returns Scale. */

@@ -179,6 +179,33 @@ class AttentionContext:
         capi.check(self.lib.tsattn_matmul_i8(self.handle, ctypes.byref(args), _stream_ptr()))
         return out
 
+    def embed_rows(self, labels, embed, embed_scale, out=None):
+        """The embedding sum of ComputePrediction (cpu_infer.cpp:559-565): labels int32 [n_rows] or [n_rows, L], embed uint8
+        (int8 bytes) [n_labels, dim] -> f32 [n_rows, dim]."""
+        if labels.dim() == 1:
+            labels = labels.view(-1, 1)
+        n_rows, per_row = labels.shape
+        n_labels, dim = embed.shape
+        if out is None:
+            out = torch.empty((n_rows, dim), dtype=torch.float32, device=embed.device)
+        assert labels.dtype == torch.int32 and labels.is_contiguous() and embed.stride(1) == 1 and out.stride(1) == 1
+        capi.check(self.lib.tsattn_embed_rows(self.handle, n_rows, dim, _ptr(labels), per_row, _ptr(embed), embed.stride(0), n_labels,
+                                              float(embed_scale), _ptr(out), out.stride(0), _stream_ptr()))
+        return out
+
+    def softmax_rows(self, vec, scale, bias=None, want_prob=True, argmax=None):
+        """The final SoftMax of ComputePrediction (cpu_infer.cpp:340-355, base 2) and the greedy choice: vec int32 [n_rows, n]
+        or [planes, n_rows, n] (parts of a split-K product) -> (prob f32 [n_rows, n] or None, argmax int32 [n_rows])."""
+        planes = vec.shape[0] if vec.dim() == 3 else 1
+        n_rows, n = vec.shape[-2:]
+        assert vec.dtype == torch.int32 and vec.is_contiguous()
+        prob = torch.empty((n_rows, n), dtype=torch.float32, device=vec.device) if want_prob else None
+        if argmax is None:
+            argmax = torch.empty(n_rows, dtype=torch.int32, device=vec.device)
+        capi.check(self.lib.tsattn_softmax_rows(self.handle, n_rows, n, _ptr(vec), planes, n_rows * n, n, float(scale), _ptr(bias),
+                                                _ptr(prob), n, _ptr(argmax), _stream_ptr()))
+        return prob, argmax
+
     def build_spans(self, seq_offset, n_tokens, window, doc_start_flag=None):
         """seq_offset: int32 [n_seqs+1] on the device.  Returns (span_start, span_finish) int32 [n_tokens]."""
         st = torch.empty(n_tokens, dtype=torch.int32, device=self.device)

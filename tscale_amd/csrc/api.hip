@@ -376,6 +376,42 @@ int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *strea
     return TSATTN_OK;
 }
 
+int tsattn_embed_rows(tsattn_handle_t h, int64_t n_rows, int dim, const int32_t *labels, int labels_per_row, const void *embed,
+                      int64_t embed_pitch, int64_t n_labels, float embed_scale, float *state, int64_t state_pitch, void *stream)
+{
+    if (!h) return fail(TSATTN_ERR_BAD_ARG, "tsattn_embed_rows: null handle");
+    if (n_rows < 0 || dim <= 0 || dim % 16 || labels_per_row <= 0 || n_labels <= 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_embed_rows: sizes (dim a multiple of 16)");
+    if (n_rows == 0) return TSATTN_OK;
+    if (!labels || !embed || !state) return fail(TSATTN_ERR_BAD_ARG, "tsattn_embed_rows: null data pointer");
+    if (embed_pitch < dim || embed_pitch % 16 || state_pitch < dim || state_pitch % 4 || !aligned16(embed) || !aligned16(state))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_embed_rows: pitches must cover a row; embed, state and their pitches multiples of 16 bytes");
+    tsattn::HeadParams p = {};
+    p.n_rows = n_rows; p.dim = dim; p.labels = labels; p.labels_per_row = labels_per_row; p.embed = (const uint8_t *)embed;
+    p.embed_pitch = embed_pitch; p.n_labels = n_labels; p.embed_scale = embed_scale; p.state = state; p.state_pitch = state_pitch;
+    hipError_t e = tsattn::launch_embed_rows(p, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "embed launch");
+    return TSATTN_OK;
+}
+
+int tsattn_softmax_rows(tsattn_handle_t h, int64_t n_rows, int64_t n, const int32_t *src, int src_planes, int64_t src_plane_stride,
+                        int64_t src_pitch, float scale, const float *bias, float *prob, int64_t prob_pitch, int32_t *argmax,
+                        void *stream)
+{
+    if (!h) return fail(TSATTN_ERR_BAD_ARG, "tsattn_softmax_rows: null handle");
+    if (n_rows < 0 || n < 0 || n > 0x7fffffff) return fail(TSATTN_ERR_BAD_ARG, "tsattn_softmax_rows: sizes");
+    if (n_rows == 0 || n == 0) return TSATTN_OK;
+    if (!src || (!prob && !argmax)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_softmax_rows: null data pointer");
+    if (src_pitch < n || (prob && prob_pitch < n)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_softmax_rows: pitches must cover a row");
+    if (src_planes < 0 || src_planes > 16 || (src_planes > 1 && src_plane_stride < n_rows * src_pitch))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_softmax_rows: up to 16 source planes, at least n_rows * src_pitch elements apart");
+    tsattn::HeadParams p = {};
+    p.n_rows = n_rows; p.n = n; p.src = src; p.src_planes = src_planes > 1 ? src_planes : 1; p.src_plane_stride = src_plane_stride;
+    p.src_pitch = src_pitch; p.scale = scale; p.bias = bias; p.prob = prob; p.prob_pitch = prob_pitch; p.argmax = argmax;
+    hipError_t e = tsattn::launch_softmax_rows(p, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "softmax launch");
+    return TSATTN_OK;
+}
+
 void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table)
 {
     if (!table || head_dim <= 0 || head_dim % 64 || max_len <= 0) return;

@@ -148,6 +148,32 @@ struct GemmParams {
 
 hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out);
 
+struct HeadParams {
+    int64_t n_rows;
+    // embedding
+    int dim;
+    const int32_t *labels;
+    int labels_per_row;
+    const uint8_t *embed;
+    int64_t embed_pitch, n_labels;
+    float embed_scale;
+    float *state;
+    int64_t state_pitch;
+    // softmax
+    int64_t n;
+    const int32_t *src;
+    int src_planes;
+    int64_t src_plane_stride, src_pitch;
+    float scale;
+    const float *bias;
+    float *prob;
+    int64_t prob_pitch;
+    int32_t *argmax;
+};
+
+hipError_t launch_embed_rows(const HeadParams &p, hipStream_t st);
+hipError_t launch_softmax_rows(const HeadParams &p, hipStream_t st);
+
 struct FillParams {
     const int32_t *seq_offset;
     const uint8_t *k_src, *v_src;
