@@ -63,6 +63,24 @@ def gpu_time_ms(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
+def graph_time_ms(fn, calls, replays):
+    """Average GPU time of one call of fn, from a HIP graph of `calls` calls replayed `replays` times: for launches short
+    enough that the host's call overhead would otherwise be what is timed."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(calls):
+            fn()
+    torch.cuda.synchronize()
+    return gpu_time_ms(graph.replay, replays, 1) / calls
+
+
 class PrefillWorkload:
     def __init__(self, ctx, dtype, B, S, H, d, n_layers, seed, short=64):
         import torch
@@ -251,7 +269,7 @@ def bench_producer(ctx, steps):
     x = torch.randn((n, H * d), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1313 + 6))
     pos = (torch.arange(n, device="cuda", dtype=torch.int32) % 2048).contiguous()
     rope = ctx.fill_rope_table(d, 2048)
-    ms = gpu_time_ms(lambda: ctx.rope_normalize_rows(x, H, capi.I8, pos=pos, rope=rope), max(5, steps // 5), 2)
+    ms = graph_time_ms(lambda: ctx.rope_normalize_rows(x, H, capi.I8, pos=pos, rope=rope), 10, max(3, steps // 10))
     nbytes = n * H * d * 5 + n * H * 4 + n * 4 + n * d * 4
     return {"config": "rope_normalize_rows: 65536 rows x 16 heads x 128, f32 -> int8 + f32 scale per (row, head), with RoPE",
             "ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4),
@@ -265,7 +283,7 @@ def bench_kv_product(ctx, steps):
     g = torch.Generator(device="cuda").manual_seed(1313 + 7)
     k = torch.randint(0, 256, (n, H * d), dtype=torch.uint8, device="cuda", generator=g)
     val = torch.randn((n, H * d), device="cuda", generator=g) * 0.3
-    ms = gpu_time_ms(lambda: ctx.kv_product(k, val, H), max(5, steps // 5), 2)
+    ms = graph_time_ms(lambda: ctx.kv_product(k, val, H), 10, max(3, steps // 10))
     nbytes = n * H * d * (1 + 4 + 4)
     return {"config": "kv_product: 65536 rows x 16 heads x 128, int8 k x f32 value -> 4 x int8", "ms": round(ms, 4),
             "GB/s": round(nbytes / ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBPS, 4), "bytes": nbytes}

@@ -67,19 +67,37 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
             v0[st] = *(const v4f *)((const float *)p.src + e + x0);
             v1[st] = *(const v4f *)((const float *)p.src + e + x1);
         }
-        if (p.resid) {
-            // state += delta * scale, written back; the updated state is what gets normalised
-            float *r0 = p.resid + s_row[pr] * p.resid_pitch + (int64_t)s_head[pr] * D + x0, *r1 = r0 + 32;
-            const v4f u0 = *(const v4f *)r0 + v0[st] * p.resid_scale, u1 = *(const v4f *)r1 + v1[st] * p.resid_scale;
-            *(v4f *)r0 = u0;
-            *(v4f *)r1 = u1;
-            v0[st] = u0;
-            v1[st] = u1;
-        }
-        if (p.pos && s_head[pr] < p.rope_heads) {
+        if (p.pos) { // heads that are not rotated read their row too and then turn by the identity: no divergent branch
             const float *rr = p.rope + (int64_t)s_pos[pr] * D;
             cs[st] = *(const v4f *)(rr + x0);
             sn[st] = *(const v4f *)(rr + x1);
+        }
+    }
+    if (p.resid) {
+        // state += delta * scale, written back; the updated state is what gets normalised.  (In loops of their own, after
+        // every request above has been issued: a store in between would keep the compiler from issuing them together.)
+        v4f u0[STEPS], u1[STEPS];
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st) {
+            const int j = tid + st * 256;
+            const int pr = j / PER_PAIR, c = j % PER_PAIR;
+            if (pr >= n_here) continue;
+            const int x0 = (c / 8) * 64 + (c % 8) * 4;
+            const float *r0 = p.resid + s_row[pr] * p.resid_pitch + (int64_t)s_head[pr] * D + x0;
+            u0[st] = *(const v4f *)r0;
+            u1[st] = *(const v4f *)(r0 + 32);
+        }
+#pragma unroll
+        for (int st = 0; st < STEPS; ++st) {
+            const int j = tid + st * 256;
+            const int pr = j / PER_PAIR, c = j % PER_PAIR;
+            if (pr >= n_here) continue;
+            const int x0 = (c / 8) * 64 + (c % 8) * 4;
+            float *r0 = p.resid + s_row[pr] * p.resid_pitch + (int64_t)s_head[pr] * D + x0;
+            v0[st] = u0[st] + v0[st] * p.resid_scale;
+            v1[st] = u1[st] + v1[st] * p.resid_scale;
+            *(v4f *)r0 = v0[st];
+            *(v4f *)(r0 + 32) = v1[st];
         }
     }
 #pragma unroll
@@ -88,11 +106,12 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
         const int pr = j / PER_PAIR, c = j % PER_PAIR;
         if (pr >= n_here) continue;
         const int x0 = (c / 8) * 64 + (c % 8) * 4, x1 = x0 + 32;
-        if (p.pos && s_head[pr] < p.rope_heads) {
+        if (p.pos) {
+            const bool turn = s_head[pr] < p.rope_heads;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float cos_value = cs[st][i];
-                const float sin_value = sn[st][i] * p.rotate_dir;
+                const float cos_value = turn ? cs[st][i] : 1.0f;
+                const float sin_value = turn ? sn[st][i] * p.rotate_dir : 0.0f;
                 const float r0 = v0[st][i] * cos_value - v1[st][i] * sin_value;
                 const float r1 = v0[st][i] * sin_value + v1[st][i] * cos_value;
                 v0[st][i] = r0;
