@@ -142,3 +142,48 @@ def test_decode_full_size_properties(ctx):
     q8, qs = orc.quantize_rows(orc.I8, bits, 1)
     want = orc.decode(orc.I8, q8, qs.T.copy(), kq, vq, ksn, 1.0, np.array([L], np.int32), 10 ** 6, 0.0)
     assert np.abs(outs[1][3, 5 * d:6 * d] - want[0]).max() < 1e-5
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_decode_randomised_shapes(ctx, seed):
+    """Seeded random decode launches: batch, heads, cache capacity and lengths (empty, one row, full), windows, slopes,
+    split counts (auto, 1, several), with and without the fused append; always against the oracle."""
+    rng = np.random.default_rng(2000 + seed)
+    dtype = [capi.I8, capi.E4M3][seed % 2]
+    d = [128, 64][(seed // 2) % 2]
+    B, H = int(rng.integers(1, 9)), int(rng.choice([1, 2, 3, 5, 8, 16]))
+    L = int(rng.choice([8, 100, 513, 2000]))
+    lens = [int(x) for x in rng.integers(0, L + 1, B)]
+    lens[0] = L                      # one full cache
+    if B > 1:
+        lens[1] = 0                  # one empty
+    window = int(rng.choice([1, 2, 64, 100, 10 ** 6])) if seed % 4 else 0
+    slope = float(rng.choice([0.0, 0.3]))
+    splits = int(rng.choice([0, 1, 2, 5]))
+    k, v, ks, vs = make_cache(300 + seed, dtype, B, H, L, d, lens)
+    q, qs = orc.quantize_rows(dtype, rng.standard_normal((B, H * d)).astype(np.float32), H)
+    qs = np.ascontiguousarray(qs.T)
+    cache = gpu_cache(ctx, dtype, k, v, ks, vs, lens)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    what = f"seed {seed}: dtype {dtype} d {d} B {B} H {H} L {L} lens {lens} window {window} slope {slope} splits {splits}"
+    if window == 0 or seed % 2 == 0:
+        want = orc.decode(dtype, q, qs, k, v, ks, vs, np.array(lens, np.int32), window, slope)
+        out = ctx.compute_val_lookup_decode(cache, dev(q), dev(qs), window, slope, n_splits=splits).cpu().numpy()
+    else:
+        # fused append of one new row per sequence; the oracle appends to its own copy first
+        kq, kss = orc.quantize_rows(dtype, rng.standard_normal((B, H * d)).astype(np.float32), H)
+        vq, vss = orc.quantize_rows(dtype, rng.standard_normal((B, H * d)).astype(np.float32), H)
+        new_lens = []
+        for b in range(B):
+            n = lens[b]
+            if n < L:
+                k[b, :, n] = kq[b].reshape(H, d); v[b, :, n] = vq[b].reshape(H, d)
+                ks[b, :, n] = kss[:, b]; vs[b, :, n] = vss[:, b]
+                n += 1
+            new_lens.append(n)
+        want = orc.decode(dtype, q, qs, k, v, ks, vs, np.array(new_lens, np.int32), window, slope)
+        out = ctx.compute_val_lookup_decode(cache, dev(q), dev(qs), window, slope, n_splits=splits,
+                                            append=(dev(kq), dev(kss.T), dev(vq), dev(vss.T))).cpu().numpy()
+        assert cache.cache_len.cpu().numpy().tolist() == new_lens, what
+        assert np.array_equal(cache.k.cpu().numpy(), k) and np.array_equal(cache.k_scale.cpu().numpy(), ks), what
+    assert np.abs(out - want).max() < 1e-4 * max(1.0, np.abs(want).max()), what

@@ -338,3 +338,35 @@ def test_prefill_ignores_what_lies_past_the_last_token(ctx, dtype, d, H, n, wind
     got = out.cpu().numpy()
     assert np.isfinite(got).all(), "rows past the last token reached the output"
     assert_within_tolerance(got, want, "rows past the end")
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_prefill_randomised_shapes(ctx, seed):
+    """Seeded random launch shapes: head counts, ragged sequence lists (some of one token, some crossing many query
+    tiles), windows from 0 to beyond the longest sequence, document starts, slopes, period hints that apply, do not apply
+    or are wrong, with and without the span summary; always against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    dtype = [capi.I8, capi.E4M3][seed % 2]
+    d = [64, 128][(seed // 2) % 2]
+    H = int(rng.choice([1, 2, 3, 5, 8, 12, 16]))
+    n_seq = int(rng.integers(1, 7))
+    seq_lens = [int(x) for x in rng.choice([1, 2, 63, 64, 65, 127, 128, 129, 200, 333, 512, 700], n_seq)]
+    if seed % 3 == 0:
+        seq_lens = [int(rng.choice([128, 256, 384]))] * n_seq      # equal lengths: the period hint can apply
+    n = sum(seq_lens)
+    window = int(rng.choice([0, 1, 2, 31, 64, 100, 256, 10 ** 6]))
+    slope = float(rng.choice([0.0, 0.0, 0.25, 0.5]))
+    flags = (rng.random(n) < 0.01).astype(np.uint8) if seed % 2 else None
+    q, qs, k, ks, v, vs = make_qkv(900 + seed, n, H, d, dtype)
+    st, fi = orc.make_spans(seq_lens, window, flags)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, slope)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    args = (dtype, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), slope)
+    tiles = ctx.build_span_tiles(t(st), t(fi))
+    period = int(rng.choice([0, seq_lens[0], 128, 2 * seq_lens[0], 96]))
+    outs = [ctx.compute_val_lookup(*args).cpu().numpy(),
+            ctx.compute_val_lookup(*args, span_tiles=tiles, causal_period=period).cpu().numpy()]
+    what = f"seed {seed}: dtype {dtype} d {d} H {H} seqs {seq_lens} window {window} slope {slope} period {period}"
+    assert np.array_equal(outs[0], outs[1]), what
+    assert_within_tolerance(outs[0], want, what)
+    assert not outs[0][fi < st].any(), what
