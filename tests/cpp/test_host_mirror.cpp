@@ -9,6 +9,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <memory>
 #include <vector>
 
 #include "../../oracle/tsattn_oracle.h"
@@ -288,9 +289,275 @@ static int RunLayerCase(int width, float slope, int headDim, bool oneProjectionM
     return fails;
 }
 
+// A layer's matrices on the host (what the oracle reads) and their device copies (what the layer reads).
+struct TLayerData {
+    std::vector<int8_t> QK, QV, K, V, Comb, Expand, Contract;
+    tso_layer_params L = {};
+    TAttentionMatrices Att;
+    int8_t *Proj = nullptr;
+
+    TLayerData(const TModelDims &dims, int width, float slope, unsigned &seed)
+    {
+        const int dim = dims.Dim, qsum = dims.GetQSum(), kvDim = qsum * 4, reluDim = qsum;
+        auto randMatrix = [&](size_t n) {
+            std::vector<int8_t> m(n);
+            for (auto &x : m) x = tso_float_to_i8(Gauss(seed) * 32.0f);
+            return m;
+        };
+        QK = randMatrix((size_t)qsum * dim); QV = randMatrix((size_t)qsum * dim); K = randMatrix((size_t)qsum * dim); V = randMatrix((size_t)qsum * dim);
+        Comb = randMatrix((size_t)dim * kvDim); Expand = randMatrix((size_t)reluDim * dim); Contract = randMatrix((size_t)dim * reluDim);
+        L.dim = dim; L.head_count = dims.HeadCount; L.head_dim = dims.QDim; L.relu_dim = reluDim;
+        L.qk = QK.data(); L.qv = QV.data(); L.k = K.data(); L.v = V.data(); L.combiner = Comb.data(); L.expand = Expand.data(); L.contract = Contract.data();
+        L.qv_scale = 0.031f; L.combiner_scale = 0.027f; L.contract_scale = 0.035f;
+        L.attention_width = width; L.alibi_slope = slope;
+        std::vector<int8_t> all;
+        for (const auto *m : {&QK, &QV, &K, &V}) all.insert(all.end(), m->begin(), m->end());
+        Proj = ToDevice(all);
+        Att.QK = Proj; Att.QV = Proj + QK.size(); Att.K = Proj + 2 * QK.size(); Att.V = Proj + 3 * QK.size();
+        Att.Combiner = ToDevice(Comb); Att.Expand = ToDevice(Expand); Att.Contract = ToDevice(Contract);
+        Att.QVScale = L.qv_scale; Att.CombinerScale = L.combiner_scale; Att.ContractScale = L.contract_scale;
+        Att.AttentionWidth = width; Att.AlibiSlope = slope;
+    }
+    ~TLayerData()
+    {
+        (void)hipFree(Proj);
+        for (const int8_t *p : {Att.Combiner, Att.Expand, Att.Contract}) (void)hipFree((void *)p);
+    }
+    TLayerData(const TLayerData &) = delete;
+};
+
+// The oracle's KV cache of one layer, in the planar layout of TAttentionVecHistory.
+struct TCpuCache {
+    int B, H, MaxLen, D;
+    std::vector<uint8_t> K, V;
+    std::vector<float> KScale;
+    std::vector<int32_t> Len;
+    TCpuCache(int b, int h, int maxLen, int d) : B(b), H(h), MaxLen(maxLen), D(d), K((size_t)b * h * maxLen * d), V(K.size()), KScale((size_t)b * h * maxLen), Len(b, 0) {}
+    void Step(const tso_layer_params &L, int nSeq, const int32_t *t, const float *rope, float *state, float *valLookup)
+    {
+        tso_add_lookup_product(&L, nSeq, t, rope, state, K.data(), V.data(), (int64_t)H * MaxLen * D, (int64_t)MaxLen * D, D, KScale.data(),
+                               (int64_t)H * MaxLen, MaxLen, Len.data(), MaxLen, valLookup, 4);
+    }
+};
+
+// The prompt form of the layer: all tokens of two fragments in one call against the oracle's token-by-token run of
+// the same layer.  Every token's projections depend on its own input state only, so the rows both sides append to the
+// cache must be identical bytes; attention output and new state within the attention tolerance.
+static int RunPromptLayerCase(int width, float slope, int headDim)
+{
+    const int B = 2, H = 4, d = headDim, dim = 512, maxLen = 256;
+    const int fragLen[B] = {150, 70};
+    const int len = fragLen[0] + fragLen[1], qsum = H * d;
+    TModelDims dims;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim;
+    unsigned seed = 4242u + width * 5 + headDim;
+    tsattn_config cfg = {};
+    cfg.device = 0; cfg.max_seqs = B; cfg.max_heads = H; cfg.max_head_dim = d;
+    tsattn_handle_t handle = nullptr;
+    if (tsattn_create(&cfg, &handle) != TSATTN_OK) { printf("tsattn_create: %s\n", tsattn_last_error()); return 1; }
+    int fails = 0;
+    {
+        TLayerData data(dims, width, slope, seed);
+        TAttentionVecHistory cache(handle, TSATTN_I8, B, H, maxLen, d);
+        TCpuCache cpu(B, H, maxLen, d);
+        TLayerComputer layer(handle, dims, len);
+        std::vector<float> rope((size_t)maxLen * d);
+        tsattn_fill_rope_table(d, maxLen, rope.data());
+        float *ropeDev = ToDevice(rope);
+        // spans, positions and fragment borders
+        TAttentionInfo attInfo;
+        attInfo.Init();
+        std::vector<int32_t> seqOffset = {0}, pos;
+        for (int b = 0; b < B; ++b) {
+            AddWindowSpans(seqOffset.back(), fragLen[b], width, nullptr, &attInfo);
+            for (int i = 0; i < fragLen[b]; ++i) pos.push_back(i);
+            seqOffset.push_back(seqOffset.back() + fragLen[b]);
+        }
+        std::vector<int32_t> spanStart(len), spanFinish(len);
+        for (int i = 0; i < len; ++i) {
+            const int n = attInfo.SpanPtr[i + 1] - attInfo.SpanPtr[i];
+            spanStart[i] = n ? attInfo.Spans[attInfo.SpanPtr[i]].Start : 0;
+            spanFinish[i] = n ? attInfo.Spans[attInfo.SpanPtr[i]].Finish : -1;
+        }
+        int32_t *spanStartDev = ToDevice(spanStart), *spanFinishDev = ToDevice(spanFinish), *seqOffsetDev = ToDevice(seqOffset), *posDev = ToDevice(pos);
+        std::vector<float> state((size_t)len * dim);
+        for (auto &x : state) x = Gauss(seed) * 3.0f;
+        float *stateDev = ToDevice(state);
+
+        // oracle: token by token, each fragment on its own cache rows
+        std::vector<float> want = state, wantVal((size_t)len * qsum);
+        for (int b = 0; b < B; ++b) {
+            for (int i = 0; i < fragLen[b]; ++i) {
+                // one sequence at a time: shift the cache views to sequence b
+                const int row = seqOffset[b] + i;
+                int32_t t = i;
+                const size_t off = (size_t)b * H * maxLen;
+                tso_add_lookup_product(&data.L, 1, &t, rope.data(), &want[(size_t)row * dim], cpu.K.data() + off * d, cpu.V.data() + off * d,
+                                       (int64_t)H * maxLen * d, (int64_t)maxLen * d, d, cpu.KScale.data() + off, (int64_t)H * maxLen, maxLen,
+                                       &cpu.Len[b], maxLen, &wantVal[(size_t)row * qsum], 4);
+            }
+        }
+        layer.AddLookupProductPrompt(len, seqOffsetDev, posDev, ropeDev, maxLen, data.Att, spanStartDev, spanFinishDev, nullptr, 0, &cache, stateDev,
+                                     nullptr);
+        HIP_OK(hipDeviceSynchronize());
+        std::vector<float> got(state.size()), gotVal(wantVal.size()), ksg(cpu.KScale.size());
+        std::vector<uint8_t> kg(cpu.K.size()), vg(cpu.V.size());
+        std::vector<int32_t> lenGpu(B);
+        HIP_OK(hipMemcpy(got.data(), stateDev, got.size() * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(gotVal.data(), layer.GetValLookup(), gotVal.size() * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(kg.data(), cache.QVState, kg.size(), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(vg.data(), cache.VState, vg.size(), hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(ksg.data(), cache.QVStateScale, ksg.size() * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(lenGpu.data(), cache.Length, B * 4, hipMemcpyDeviceToHost));
+        if (lenGpu != cpu.Len) { printf("  cache lengths differ\n"); ++fails; }
+        for (int b = 0; b < B; ++b) {
+            for (int h = 0; h < H; ++h) {
+                const size_t r0 = ((size_t)b * H + h) * maxLen;
+                if (memcmp(&kg[r0 * d], &cpu.K[r0 * d], (size_t)fragLen[b] * d) || memcmp(&vg[r0 * d], &cpu.V[r0 * d], (size_t)fragLen[b] * d)) {
+                    printf("  cache rows of fragment %d head %d differ\n", b, h); ++fails;
+                }
+                if (memcmp(&ksg[r0], &cpu.KScale[r0], (size_t)fragLen[b] * 4)) { printf("  key scales of fragment %d head %d differ\n", b, h); ++fails; }
+            }
+        }
+        // the prefill tolerance (probabilities go through fp16 there): attention output rescaled to unit variance within
+        // 2e-2 at most and 2e-3 on average; the state, which takes single int8 flips from it, within 5e-2 of its rms at
+        // most and 5e-3 in the root mean square
+        double rms = 0, maxState = 0, rmsState = 0, maxVal = 0, meanVal = 0, valMean = 0, valStd = 0;
+        for (float x : want) rms += (double)x * x;
+        rms = sqrt(rms / want.size());
+        for (size_t i = 0; i < want.size(); ++i) {
+            const double e = fabs((double)got[i] - want[i]) / rms;
+            maxState = fmax(maxState, e);
+            rmsState += e * e;
+        }
+        rmsState = sqrt(rmsState / want.size());
+        for (float x : wantVal) valMean += x;
+        valMean /= wantVal.size();
+        for (float x : wantVal) valStd += (x - valMean) * (x - valMean);
+        valStd = sqrt(valStd / wantVal.size());
+        for (size_t i = 0; i < wantVal.size(); ++i) {
+            const double e = fabs((double)gotVal[i] - wantVal[i]) / valStd;
+            maxVal = fmax(maxVal, e);
+            meanVal += e / wantVal.size();
+        }
+        if (maxVal > 2e-2 || meanVal > 2e-3 || maxState > 5e-2 || rmsState > 5e-3) ++fails;
+        printf("prompt layer width %4d slope %.2f d %3d: %d tokens in %d fragments, valLookup error / std max %.2e mean %.2e, state error / rms max %.2e "
+               "rms %.2e  %s\n", width, slope, d, len, B, maxVal, meanVal, maxState, rmsState, fails ? "FAIL" : "ok");
+        for (void *p : {(void *)ropeDev, (void *)spanStartDev, (void *)spanFinishDev, (void *)seqOffsetDev, (void *)posDev, (void *)stateDev}) HIP_OK(hipFree(p));
+    }
+    tsattn_destroy(handle);
+    return fails;
+}
+
+// ComputePrediction over three layers (narrow, ALiBi, wide) for a few tokens per sequence, each side on its own caches
+// and states.  The oracle's pass is its own parts in the reference's order: embedding, layers, NormalizeState, the final
+// product, SoftMax.  Small differences of the attention output flip single int8 roundings downstream, so the
+// distributions agree to a tolerance, and the greedy choice wherever the oracle's best label leads by a clear margin.
+static int RunPredictionCase()
+{
+    const int B = 3, H = 2, d = 128, dim = 256, maxLen = 16, vocab = 1024, steps = 5;
+    TModelDims dims;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim;
+    unsigned seed = 777u;
+    tsattn_config cfg = {};
+    cfg.device = 0; cfg.max_seqs = B; cfg.max_heads = H; cfg.max_head_dim = d;
+    tsattn_handle_t handle = nullptr;
+    if (tsattn_create(&cfg, &handle) != TSATTN_OK) { printf("tsattn_create: %s\n", tsattn_last_error()); return 1; }
+    int fails = 0;
+    {
+        const int widths[3] = {1, 4, 1000};
+        const float slopes[3] = {0.0f, 0.5f, 0.0f};
+        std::vector<std::unique_ptr<TLayerData>> layers;
+        std::vector<std::unique_ptr<TAttentionVecHistory>> caches;
+        std::vector<TCpuCache> cpuCaches;
+        TInferModel model;
+        std::vector<TAttentionVecHistory *> cachePtrs;
+        for (int l = 0; l < 3; ++l) {
+            layers.emplace_back(new TLayerData(dims, widths[l], slopes[l], seed));
+            caches.emplace_back(new TAttentionVecHistory(handle, TSATTN_I8, B, H, maxLen, d));
+            cpuCaches.emplace_back(B, H, maxLen, d);
+            model.LayerArr.push_back(layers.back()->Att);
+            cachePtrs.push_back(caches.back().get());
+        }
+        std::vector<int8_t> embed((size_t)vocab * dim), finalLayer((size_t)vocab * dim);
+        for (auto &x : embed) x = tso_float_to_i8(Gauss(seed) * 32.0f);
+        for (auto &x : finalLayer) x = tso_float_to_i8(Gauss(seed) * 32.0f);
+        std::vector<float> bias(vocab);
+        for (auto &x : bias) x = Gauss(seed) * 0.5f;
+        int8_t *embedDev = ToDevice(embed), *finalDev = ToDevice(finalLayer);
+        float *biasDev = ToDevice(bias);
+        model.LabelEmbed = embedDev; model.LabelEmbedScale = 0.04f; model.LabelCount = vocab;
+        model.FinalLayer = finalDev; model.FinalLayerScale = 0.08f; model.VocabSize = vocab; model.Bias = biasDev;
+        TLayerComputer layer(handle, dims, B, vocab);
+        std::vector<float> rope((size_t)maxLen * d);
+        tsattn_fill_rope_table(d, maxLen, rope.data());
+        float *ropeDev = ToDevice(rope);
+        float *stateDev = nullptr, *probDev = nullptr;
+        int32_t *labelDev = nullptr, *tDev = nullptr, *choiceDev = nullptr;
+        HIP_OK(hipMalloc((void **)&stateDev, (size_t)B * dim * 4));
+        HIP_OK(hipMalloc((void **)&probDev, (size_t)B * vocab * 4));
+        HIP_OK(hipMalloc((void **)&labelDev, B * 4));
+        HIP_OK(hipMalloc((void **)&tDev, B * 4));
+        HIP_OK(hipMalloc((void **)&choiceDev, B * 4));
+        std::vector<int32_t> labels = {5, 900, 333};
+        double maxProb = 0;
+        int choicesChecked = 0;
+        for (int step = 0; step < steps; ++step) {
+            std::vector<int32_t> t(B, step);
+            HIP_OK(hipMemcpy(labelDev, labels.data(), B * 4, hipMemcpyHostToDevice));
+            HIP_OK(hipMemcpy(tDev, t.data(), B * 4, hipMemcpyHostToDevice));
+            ComputePrediction(layer, model, cachePtrs, labelDev, tDev, ropeDev, maxLen, stateDev, probDev, choiceDev, nullptr);
+            HIP_OK(hipDeviceSynchronize());
+            // the oracle's pass
+            std::vector<float> state((size_t)B * dim), want((size_t)B * vocab);
+            tso_embed_rows(B, dim, labels.data(), 1, embed.data(), vocab, model.LabelEmbedScale, state.data());
+            for (int l = 0; l < 3; ++l) cpuCaches[l].Step(layers[l]->L, B, t.data(), rope.data(), state.data(), nullptr);
+            std::vector<uint8_t> norm((size_t)B * dim);
+            std::vector<float> tileScale(dim / STATE_NORM_TILE);
+            for (int b = 0; b < B; ++b) tso_normalize_heads(TSO_I8, &state[(size_t)b * dim], dim, dim / STATE_NORM_TILE, VEC_SCALE, &norm[(size_t)b * dim], tileScale.data());
+            std::vector<int32_t> logits((size_t)B * vocab), wantChoice(B);
+            tso_matmul_i8((const int8_t *)norm.data(), dim, finalLayer.data(), dim, B, vocab, dim, 0, 0.0f, logits.data(), vocab);
+            const float finalScale = sqrtf(1.0f / (float)dim) * (1.0f / 0.693147f) * model.FinalLayerScale * VEC_SCALE;
+            tso_softmax_rows(B, vocab, logits.data(), finalScale, bias.data(), 0, want.data(), wantChoice.data());
+            std::vector<float> got(want.size());
+            std::vector<int32_t> choice(B);
+            HIP_OK(hipMemcpy(got.data(), probDev, got.size() * 4, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(choice.data(), choiceDev, B * 4, hipMemcpyDeviceToHost));
+            for (int b = 0; b < B; ++b) {
+                const float *w = &want[(size_t)b * vocab], *g = &got[(size_t)b * vocab];
+                float best = 0, second = 0;
+                double sum = 0;
+                for (int k = 0; k < vocab; ++k) {
+                    if (w[k] > best) { second = best; best = w[k]; } else if (w[k] > second) second = w[k];
+                    maxProb = fmax(maxProb, fabs((double)g[k] - w[k]) / (w[k] + 1e-3));
+                    sum += g[k];
+                }
+                if (fabs(sum - 1) > 1e-4) { printf("  step %d: probabilities of sequence %d sum to %.6f\n", step, b, sum); ++fails; }
+                if (best > 1.3f * second) {
+                    ++choicesChecked;
+                    if (choice[b] != wantChoice[b]) { printf("  step %d: sequence %d chose %d, oracle %d\n", step, b, choice[b], wantChoice[b]); ++fails; }
+                }
+            }
+            labels = choice; // greedy generation: the GPU's choice is both sides' next label
+        }
+        if (maxProb > 0.1) ++fails;
+        printf("ComputePrediction: 3 layers, %d tokens x %d sequences, vocabulary %d: max |p - p_oracle| / (p_oracle + 1e-3) %.2e, %d greedy choices compared  %s\n",
+               steps, B, vocab, maxProb, choicesChecked, fails ? "FAIL" : "ok");
+        for (void *p : {(void *)embedDev, (void *)finalDev, (void *)biasDev, (void *)ropeDev, (void *)stateDev, (void *)probDev, (void *)labelDev, (void *)tDev, (void *)choiceDev})
+            HIP_OK(hipFree(p));
+    }
+    tsattn_destroy(handle);
+    return fails;
+}
+
 int main()
 {
     int fails = 0;
+    fails += RunPromptLayerCase(1000, 0.0f, 128);
+    fails += RunPromptLayerCase(64, 0.5f, 128);
+    fails += RunPromptLayerCase(1, 0.0f, 64);
+    fails += RunPromptLayerCase(0, 0.0f, 128);
+    fails += RunPredictionCase();
     fails += RunLayerCase(1000, 0.0f, 128, true);
     fails += RunLayerCase(1000, 0.0f, 128, false);
     fails += RunLayerCase(4, 0.5f, 128, true);

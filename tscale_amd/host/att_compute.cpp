@@ -214,13 +214,13 @@ void ComputeValLookup(int width, float alibiSlope, const TAttentionVecHistory &h
 
 // ---- one layer of the int8 inference path ----------------------------------------------------------------------
 
-TLayerComputer::TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, int seqCount)
-    : Handle(handle), Dims(dims), SeqCount(seqCount)
+TLayerComputer::TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, int maxRows, int64_t maxOutputs)
+    : Handle(handle), Dims(dims), MaxRows(maxRows)
 {
     TS_VERIFY(dims.QDim == dims.TTDim && (dims.QDim == 64 || dims.QDim == 128), "QDim %d TTDim %d: equal, 64 or 128", dims.QDim, dims.TTDim);
     TS_VERIFY(dims.Dim % STATE_NORM_TILE == 0, "Dim %d is not a multiple of %d", dims.Dim, STATE_NORM_TILE);
     ReluDim = dims.HeadCount * dims.QDim;
-    const size_t n = (size_t)seqCount, qsum = (size_t)dims.GetQSum();
+    const size_t n = (size_t)maxRows, qsum = (size_t)dims.GetQSum();
     auto alloc = [](void **p, size_t bytes) { CheckHip(hipMalloc(p, bytes), "hipMalloc(layer buffers)"); };
     alloc((void **)&NormState, n * dims.Dim);
     alloc((void **)&Q4, n * qsum * 4);
@@ -229,12 +229,15 @@ TLayerComputer::TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, i
     alloc((void **)&QvHeadScale, n * dims.HeadCount * 4);
     alloc((void **)&VHeadScale, n * dims.HeadCount * 4);
     alloc((void **)&ValLookup, n * qsum * 4);
-    // the int32 results of the matrix products: up to 16 planes (K split over workgroups) of the widest one
+    // the int32 results of the matrix products: 16 planes of the widest one with few rows (K split over workgroups), one
+    // plane otherwise
     size_t widest = 4 * qsum > (size_t)dims.Dim ? 4 * qsum : (size_t)dims.Dim;
     if ((size_t)ReluDim > widest) widest = ReluDim;
-    PlaneElems = (int64_t)(n * widest);
-    alloc((void **)&Planes, (size_t)PlaneElems * 16 * 4);
-    WorkspaceBytes = (int64_t)(16 * 4 * n * dims.Dim);
+    if ((size_t)maxOutputs > widest) widest = (size_t)maxOutputs;
+    const size_t fewRows = n < 128 ? n : 128;
+    const size_t planeElems = (16 * fewRows > n ? 16 * fewRows : n) * widest;
+    alloc((void **)&Planes, planeElems * 4);
+    WorkspaceBytes = (int64_t)(16 * 4 * fewRows * dims.Dim);
     alloc(&Workspace, (size_t)WorkspaceBytes);
     // values carry the constant VEC_SCALE (cpu_infer.cpp:454)
     std::vector<float> vs(n * dims.HeadCount, VEC_SCALE);
@@ -247,73 +250,114 @@ TLayerComputer::~TLayerComputer()
     for (void *p : all) (void)hipFree(p);
 }
 
-void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
-                                      TAttentionVecHistory *pKVCache, float *state, void *stream)
+// MulForward, result left as int32 planes in Planes (their sum is the product); returns the number of planes
+int TLayerComputer::MulForwardPlanes(int rows, const uint8_t *vec, int k, const int8_t *matr, int n, void *stream)
 {
-    TAttentionVecHistory &kvCache = *pKVCache;
+    tsattn_matmul_args a = {};
+    int planes = 0;
+    a.m = rows; a.n = n; a.k = k;
+    a.a = vec; a.a_pitch = k; a.w = matr; a.w_pitch = k;
+    a.mode = TSATTN_MM_I32_PLANES; a.out = Planes; a.out_pitch = n; a.planes_out = &planes;
+    Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
+    return planes;
+}
+
+// NormalizeState on int32 planes or on a float array: per group of groupDim values, to int8 (fields of `a` preset by the
+// caller select rotation, scale output, ReLU, the residual update)
+static void Normalize(tsattn_handle_t handle, tsattn_produce_args a, int rows, const void *src, bool srcI32, int planes, int groups,
+                      int groupDim, uint8_t *dst, void *stream)
+{
+    a.src_dtype = srcI32 ? TSATTN_SRC_I32 : TSATTN_SRC_F32;
+    a.dst_dtype = TSATTN_I8;
+    a.n_rows = rows; a.n_heads = groups; a.head_dim = groupDim;
+    a.src = src; a.src_pitch = (int64_t)groups * groupDim;
+    a.src_planes = planes; a.src_plane_stride = (int64_t)rows * groups * groupDim;
+    a.rotate_dir = 1; a.vec_scale = VEC_SCALE;
+    if (a.scale_mult == 0) a.scale_mult = 1;
+    a.dst = dst; a.dst_pitch = (int64_t)groups * groupDim;
+    Check(tsattn_rope_normalize_rows(handle, &a, stream), "tsattn_rope_normalize_rows");
+}
+
+// state -> NormalizeState -> the four projections -> ApplyRope on qk and qv, NormalizeState per head on all four: Q4 holds
+// rows of qk, qv, k, v heads; QvHeadScale the key scales as [row][head] (token form) or [head][row] planes (prompt form)
+void TLayerComputer::Projections(int rows, const int32_t *pos, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
+                                 bool scalePlanes, const float *state, void *stream)
+{
     const int dim = Dims.Dim, headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
-    TS_VERIFY(kvCache.SeqCount == SeqCount && kvCache.HeadCount == headCount && kvCache.HeadDim == headDim && kvCache.DType == TSATTN_I8,
-              "the KV cache does not match the layer (%d sequences, %d heads of %d, int8)", SeqCount, headCount, headDim);
-
-    // MulForward, result left as int32 planes in Planes (their sum is the product); returns the number of planes
-    auto mulForward = [&](const uint8_t *vec, int k, const int8_t *matr, int n) {
-        tsattn_matmul_args a = {};
-        int planes = 0;
-        a.m = SeqCount; a.n = n; a.k = k;
-        a.a = vec; a.a_pitch = k; a.w = matr; a.w_pitch = k;
-        a.mode = TSATTN_MM_I32_PLANES; a.out = Planes; a.out_pitch = n; a.planes_out = &planes;
-        Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
-        return planes;
-    };
-    // NormalizeState on Planes or on a float array: per group of groupDim values, to int8
-    auto normalize = [&](tsattn_produce_args a, const void *src, bool srcI32, int planes, int groups, int groupDim, uint8_t *dst) {
-        a.src_dtype = srcI32 ? TSATTN_SRC_I32 : TSATTN_SRC_F32;
-        a.dst_dtype = TSATTN_I8;
-        a.n_rows = SeqCount; a.n_heads = groups; a.head_dim = groupDim;
-        a.src = src; a.src_pitch = (int64_t)groups * groupDim;
-        a.src_planes = planes; a.src_plane_stride = (int64_t)SeqCount * groups * groupDim;
-        a.rotate_dir = 1; a.vec_scale = VEC_SCALE;
-        if (a.scale_mult == 0) a.scale_mult = 1;
-        a.dst = dst; a.dst_pitch = (int64_t)groups * groupDim;
-        Check(tsattn_rope_normalize_rows(Handle, &a, stream), "tsattn_rope_normalize_rows");
-    };
-
-    normalize({}, state, false, 1, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState);
-
-    // The four projections.  Matrices that lie one after the other in memory (QK, QV, K, V) are one product; the
-    // result rows hold the qk, qv, k and v heads in that order either way.
+    TS_VERIFY(rows <= MaxRows, "%d rows, buffers for %d", rows, MaxRows);
+    Normalize(Handle, {}, rows, state, false, 1, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
+    // Matrices that lie one after the other in memory (QK, QV, K, V) are one product; the result rows hold the qk, qv, k
+    // and v heads in that order either way.
     const size_t matBytes = (size_t)qsum * dim;
     int planes = 1;
     if ((const int8_t *)att.QV == att.QK + matBytes && att.K == att.QV + matBytes && att.V == att.K + matBytes) {
-        planes = mulForward(NormState, dim, att.QK, 4 * qsum);
+        planes = MulForwardPlanes(rows, NormState, dim, att.QK, 4 * qsum, stream);
     } else {
         const int8_t *mats[4] = {att.QK, att.QV, att.K, att.V};
         for (int i = 0; i < 4; ++i) {
             tsattn_matmul_args a = {};
-            a.m = SeqCount; a.n = qsum; a.k = dim;
+            a.m = rows; a.n = qsum; a.k = dim;
             a.a = NormState; a.a_pitch = dim; a.w = mats[i]; a.w_pitch = dim;
             a.mode = TSATTN_MM_I32; a.out = Planes + (size_t)i * qsum; a.out_pitch = 4 * qsum;
             a.workspace = Workspace; a.workspace_bytes = WorkspaceBytes;
             Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
         }
     }
-    // ApplyRope on qk and qv, NormalizeState per head on all four, in one call; the cached key scale takes the matrix
-    // scale: qvMult *= att.QVScale * VEC_SCALE * CalcDotScale(dim)
+    // the cached key scale takes the matrix scale: qvMult *= att.QVScale * VEC_SCALE * CalcDotScale(dim)
+    tsattn_produce_args a = {};
+    a.pos = pos; a.rope = ropeBuf; a.rope_len = ropeLen; a.rope_heads = 2 * headCount;
+    a.scale = QvHeadScale;
+    if (scalePlanes) { a.scale_pitch = rows; a.scale_row_stride = 1; }           // [head][row], what tsattn_prefill reads
+    else { a.scale_pitch = 1; a.scale_row_stride = headCount; }                   // [row][head], what the cache append reads
+    a.scale_head_begin = headCount; a.scale_head_count = headCount;
+    a.scale_mult = att.QVScale * VEC_SCALE * sqrtf(1.0f / (float)dim);
+    Normalize(Handle, a, rows, Planes, true, planes, 4 * headCount, headDim, Q4, stream);
+}
+
+// KVProduct, combiner (its AddScaled done by the normalisation that follows: state += delta * scale, then normalise),
+// expand, per-head normalisation + ReLU, contract + AddScaled
+void TLayerComputer::AfterAttention(int rows, const TAttentionMatrices &att, float *state, void *stream)
+{
+    const int dim = Dims.Dim, headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
+    const uint8_t *k = Q4 + 2 * (size_t)qsum;
+    Check(tsattn_kv_product(Handle, rows, headCount, headDim, COMBINER_REP, k, 4 * (int64_t)qsum, TSATTN_OUT_F32, ValLookup, qsum, 1.0f, Kv,
+                            (int64_t)qsum * COMBINER_REP, stream), "tsattn_kv_product");
+    const int kvDim = qsum * COMBINER_REP;
+    int planes = MulForwardPlanes(rows, Kv, kvDim, att.Combiner, dim, stream);
     {
         tsattn_produce_args a = {};
-        a.pos = t; a.rope = ropeBuf; a.rope_len = ropeLen; a.rope_heads = 2 * headCount;
-        a.scale = QvHeadScale; a.scale_pitch = 1; a.scale_row_stride = headCount; // [seq][head], what the cache append reads
-        a.scale_head_begin = headCount; a.scale_head_count = headCount;
-        a.scale_mult = att.QVScale * VEC_SCALE * sqrtf(1.0f / (float)dim);
-        normalize(a, Planes, true, planes, 4 * headCount, headDim, Q4);
+        a.resid = state; a.resid_pitch = dim; a.resid_scale = att.CombinerScale * VEC_SCALE * sqrtf(1.0f / (float)kvDim);
+        Normalize(Handle, a, rows, Planes, true, planes, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
     }
-    const uint8_t *qk = Q4, *qv = Q4 + qsum, *k = Q4 + 2 * (size_t)qsum, *v = Q4 + 3 * (size_t)qsum;
+    planes = MulForwardPlanes(rows, NormState, dim, att.Expand, ReluDim, stream);
+    {
+        tsattn_produce_args a = {};
+        a.relu = 1;
+        Normalize(Handle, a, rows, Planes, true, planes, headCount, ReluDim / headCount, Relu, stream);
+    }
+    tsattn_matmul_args ca = {};
+    ca.m = rows; ca.n = dim; ca.k = ReluDim;
+    ca.a = Relu; ca.a_pitch = ReluDim; ca.w = att.Contract; ca.w_pitch = ReluDim;
+    ca.mode = TSATTN_MM_ADD_SCALED; ca.scale = att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim);
+    ca.out = state; ca.out_pitch = dim; ca.workspace = Workspace; ca.workspace_bytes = WorkspaceBytes;
+    Check(tsattn_matmul_i8(Handle, &ca, stream), "tsattn_matmul_i8");
+}
+
+void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
+                                      TAttentionVecHistory *pKVCache, float *state, void *stream)
+{
+    TAttentionVecHistory &kvCache = *pKVCache;
+    const int headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum(), rows = kvCache.SeqCount;
+    TS_VERIFY(kvCache.HeadCount == headCount && kvCache.HeadDim == headDim && kvCache.DType == TSATTN_I8,
+              "the KV cache does not match the layer (%d heads of %d, int8)", headCount, headDim);
+    Projections(rows, t, ropeBuf, ropeLen, att, false, state, stream);
+    const uint8_t *qk = Q4, *qv = Q4 + qsum, *v = Q4 + 3 * (size_t)qsum;
     const int64_t pitch4 = 4 * (int64_t)qsum;
 
     // kvCache.AddVectors(qv, qvHeadScale, v) and ComputeValLookup(width, slope, dims, kvCache, qk, &valLookup)
     tsattn_decode_args da = {};
     da.dtype = TSATTN_I8; da.q_dtype = TSATTN_Q_8BIT;
-    da.n_seqs = SeqCount; da.n_heads = headCount; da.head_dim = headDim;
+    da.n_seqs = rows; da.n_heads = headCount; da.head_dim = headDim;
     da.q = qk; da.q_pitch = pitch4; da.q_scale = nullptr; da.q_scale_const = VEC_SCALE;
     da.k_cache = kvCache.QVState; da.v_cache = kvCache.VState;
     da.seq_stride = (int64_t)headCount * kvCache.MaxLen * headDim;
@@ -327,7 +371,7 @@ void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, in
     if (att.AttentionWidth == 0) {
         // the token attends to the row being written: append first, in its own call
         tsattn_append_args aa = {};
-        aa.n_seqs = SeqCount; aa.n_heads = headCount; aa.head_dim = headDim;
+        aa.n_seqs = rows; aa.n_heads = headCount; aa.head_dim = headDim;
         aa.k_new = qv; aa.v_new = v; aa.new_pitch = pitch4; aa.k_scale_new = QvHeadScale; aa.v_scale_new = VHeadScale;
         aa.k_cache = kvCache.QVState; aa.v_cache = kvCache.VState;
         aa.seq_stride = da.seq_stride; aa.head_stride = da.head_stride; aa.tok_stride = da.tok_stride;
@@ -339,30 +383,67 @@ void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, in
         da.k_new = qv; da.v_new = v; da.new_pitch = pitch4; da.k_scale_new = QvHeadScale; da.v_scale_new = VHeadScale;
     }
     Check(tsattn_decode(Handle, &da, stream), "tsattn_decode");
+    AfterAttention(rows, att, state, stream);
+}
 
-    Check(tsattn_kv_product(Handle, SeqCount, headCount, headDim, COMBINER_REP, k, pitch4, TSATTN_OUT_F32, ValLookup, qsum, 1.0f, Kv,
-                            (int64_t)qsum * COMBINER_REP, stream), "tsattn_kv_product");
-    // combiner; its AddScaled is done by the normalisation that follows (state += delta * scale, then normalise)
-    const int kvDim = qsum * COMBINER_REP;
-    planes = mulForward(Kv, kvDim, att.Combiner, dim);
-    {
-        tsattn_produce_args a = {};
-        a.resid = state; a.resid_pitch = dim; a.resid_scale = att.CombinerScale * VEC_SCALE * sqrtf(1.0f / (float)kvDim);
-        normalize(a, Planes, true, planes, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState);
+void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
+                                            const TAttentionMatrices &att, const int32_t *spanStart, const int32_t *spanFinish,
+                                            const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
+                                            void *stream)
+{
+    TAttentionVecHistory &kvCache = *pKVCache;
+    const int headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
+    TS_VERIFY(kvCache.HeadCount == headCount && kvCache.HeadDim == headDim && kvCache.DType == TSATTN_I8,
+              "the KV cache does not match the layer (%d heads of %d, int8)", headCount, headDim);
+    Projections(len, pos, ropeBuf, ropeLen, att, true, state, stream);
+    const uint8_t *qk = Q4, *qv = Q4 + qsum, *v = Q4 + 3 * (size_t)qsum;
+    const int64_t pitch4 = 4 * (int64_t)qsum;
+    // every token's attention over the earlier tokens of its fragment: the prefill form of ComputeValLookup
+    tsattn_prefill_args pa = {};
+    pa.dtype = TSATTN_I8; pa.out_dtype = TSATTN_OUT_F32;
+    pa.n_tokens = len; pa.n_heads = headCount; pa.head_dim = headDim;
+    pa.q = qk; pa.k = qv; pa.v = v; pa.q_pitch = pa.k_pitch = pa.v_pitch = pitch4;
+    pa.q_scale = nullptr; pa.q_scale_const = VEC_SCALE; pa.k_scale = QvHeadScale; pa.v_scale = nullptr; pa.v_scale_const = VEC_SCALE;
+    pa.scale_pitch = len;
+    pa.span_start = spanStart; pa.span_finish = spanFinish; pa.span_tiles = spanTiles; pa.causal_period = causalPeriod;
+    pa.alibi_slope = att.AlibiSlope;
+    pa.out = ValLookup; pa.out_pitch = (int64_t)qsum * 4;
+    Check(tsattn_prefill(Handle, &pa, stream), "tsattn_prefill");
+    // kvCache.AddVectors for every token at once
+    tsattn_fill_args fa = {};
+    fa.n_seqs = kvCache.SeqCount; fa.n_heads = headCount; fa.head_dim = headDim; fa.n_tokens = len;
+    fa.seq_offset = seqOffset; fa.k = qv; fa.v = v; fa.pitch = pitch4;
+    fa.k_scale = QvHeadScale; fa.v_scale = VHeadScale; fa.scale_pitch = len; // VHeadScale: the constant in every slot
+    fa.k_cache = kvCache.QVState; fa.v_cache = kvCache.VState;
+    fa.seq_stride = (int64_t)headCount * kvCache.MaxLen * headDim;
+    fa.head_stride = (int64_t)kvCache.MaxLen * headDim;
+    fa.tok_stride = headDim;
+    fa.k_scale_cache = kvCache.QVStateScale; fa.v_scale_cache = kvCache.VStateScale;
+    fa.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; fa.s_head_stride = kvCache.MaxLen;
+    fa.cache_len = kvCache.Length; fa.max_len = kvCache.MaxLen;
+    Check(tsattn_cache_fill(Handle, &fa, stream), "tsattn_cache_fill");
+    AfterAttention(len, att, state, stream);
+}
+
+void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const std::vector<TAttentionVecHistory *> &kvCaches,
+                       const int32_t *labels, const int32_t *t, const float *ropeBuf, int64_t ropeLen, float *state,
+                       float *prediction, int32_t *choice, void *stream)
+{
+    TS_VERIFY(kvCaches.size() == model.LayerArr.size() && !kvCaches.empty(), "%d caches for %d layers", (int)kvCaches.size(), (int)model.LayerArr.size());
+    const int dim = layer.Dims.Dim, rows = kvCaches[0]->SeqCount;
+    // embedding
+    Check(tsattn_embed_rows(layer.Handle, rows, dim, labels, 1, model.LabelEmbed, dim, model.LabelCount, model.LabelEmbedScale, state, dim, stream),
+          "tsattn_embed_rows");
+    // apply layers
+    for (size_t d = 0; d < model.LayerArr.size(); ++d) layer.AddLookupProduct(t, ropeBuf, ropeLen, model.LayerArr[d], kvCaches[d], state, stream);
+    if (prediction || choice) {
+        Normalize(layer.Handle, {}, rows, state, false, 1, dim / STATE_NORM_TILE, STATE_NORM_TILE, layer.NormState, stream);
+        const int planes = layer.MulForwardPlanes(rows, layer.NormState, dim, model.FinalLayer, (int)model.VocabSize, stream);
+        // finalScale = CalcDotScale(dim) * CalcFinalLayerMult() * params.FinalLayerScale * VEC_SCALE
+        const float finalScale = sqrtf(1.0f / (float)dim) * (1.0f / 0.693147f) * model.FinalLayerScale * VEC_SCALE;
+        Check(tsattn_softmax_rows(layer.Handle, rows, model.VocabSize, layer.Planes, planes, (int64_t)rows * model.VocabSize, model.VocabSize, finalScale,
+                                  model.Bias, prediction, model.VocabSize, choice, stream), "tsattn_softmax_rows");
     }
-    // relu
-    planes = mulForward(NormState, dim, att.Expand, ReluDim);
-    {
-        tsattn_produce_args a = {};
-        a.relu = 1;
-        normalize(a, Planes, true, planes, headCount, ReluDim / headCount, Relu);
-    }
-    tsattn_matmul_args ca = {};
-    ca.m = SeqCount; ca.n = dim; ca.k = ReluDim;
-    ca.a = Relu; ca.a_pitch = ReluDim; ca.w = att.Contract; ca.w_pitch = ReluDim;
-    ca.mode = TSATTN_MM_ADD_SCALED; ca.scale = att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim);
-    ca.out = state; ca.out_pitch = dim; ca.workspace = Workspace; ca.workspace_bytes = WorkspaceBytes;
-    Check(tsattn_matmul_i8(Handle, &ca, stream), "tsattn_matmul_i8");
 }
 
 } // namespace NTsAttn

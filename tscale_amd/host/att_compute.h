@@ -9,7 +9,8 @@
 //   TAttentionVecHistory::AddVectors       gpt/train/cpu_infer.cpp:397-410            TAttentionVecHistory::AddVectors
 //   ComputeValLookup (KV cache)            gpt/train/cpu_infer.cpp:413-460 (call :509) NTsAttn::ComputeValLookup
 //   TCPUModelParams::TAttentionMatrices    gpt/train/cpu_infer.cpp:60-77              NTsAttn::TAttentionMatrices
-//   AddLookupProduct                       gpt/train/cpu_infer.cpp:465-527            TLayerComputer::AddLookupProduct
+//   AddLookupProduct                       gpt/train/cpu_infer.cpp:465-527            TLayerComputer::AddLookupProduct(Prompt)
+//   ComputePrediction                      gpt/train/cpu_infer.cpp:552-582            NTsAttn::ComputePrediction
 //
 // All arithmetic runs in libtsattn.so through the C ABI of include/tsattn.h; this layer owns the
 // per-context device buffers (allocated once, like TAttentionComputeCtx::AllocateCuda,
@@ -145,26 +146,37 @@ constexpr float VEC_SCALE = 1.0f / 24; // gpt/train/cpu_infer.cpp:16
 constexpr int STATE_NORM_TILE = 128;   // gpt/model_params/model_dim.h:22
 constexpr int COMBINER_REP = 4;        // gpt/model_params/model_dim.h:12
 
-// AddLookupProduct for a batch: one new token per sequence, every sequence with its own state row and KV cache.
-// Owns the intermediate vectors (allocated once for seqCount sequences).  11 or 12 launches per call: the four
-// projections are one product when QK, QV, K and V lie one after the other in memory, the normalisations that follow
-// them are one call, K-split products leave their parts for the consumer to add up, and the combiner's AddScaled is
-// done by the normalisation after it.  QDim == TTDim == 64 or 128; the feed-forward
-// width is reluDim = HeadCount * QDim (ReluMult 1 at QDim 128).
+// AddLookupProduct for a batch of rows.  Token form: one new token per sequence, every sequence with its own state row
+// and KV cache (append + attention over the cache).  Prompt form: all tokens of a batch of fragments at once (one
+// prefill launch, one cache fill).  Owns the intermediate vectors (allocated once for maxRows rows).  11 or 12 launches
+// per call: the four projections are one product when QK, QV, K and V lie one after the other in memory, the
+// normalisations that follow them are one call, K-split products leave their parts for the consumer to add up, and the
+// combiner's AddScaled is done by the normalisation after it.  QDim == TTDim == 64 or 128; the feed-forward width is
+// reluDim = HeadCount * QDim (ReluMult 1 at QDim 128).
+struct TInferModel; // below
+
 class TLayerComputer
 {
     tsattn_handle_t Handle = nullptr;
     TModelDims Dims;
-    int SeqCount = 0, ReluDim = 0;
+    int MaxRows = 0, ReluDim = 0;
     uint8_t *NormState = nullptr, *Q4 = nullptr, *Kv = nullptr, *Relu = nullptr; // Q4: rows of qk, qv, k, v heads
     float *QvHeadScale = nullptr, *VHeadScale = nullptr, *ValLookup = nullptr;
-    int32_t *Planes = nullptr; // int32 results of the matrix products, up to 16 planes
-    int64_t PlaneElems = 0;
+    int32_t *Planes = nullptr; // int32 results of the matrix products: up to 16 planes with few rows, one otherwise
     void *Workspace = nullptr;
     int64_t WorkspaceBytes = 0;
 
+    int MulForwardPlanes(int rows, const uint8_t *vec, int k, const int8_t *matr, int n, void *stream);
+    void Projections(int rows, const int32_t *pos, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att, bool scalePlanes,
+                     const float *state, void *stream);
+    void AfterAttention(int rows, const TAttentionMatrices &att, float *state, void *stream);
+    friend void ComputePrediction(TLayerComputer &, const TInferModel &, const std::vector<TAttentionVecHistory *> &, const int32_t *,
+                                  const int32_t *, const float *, int64_t, float *, float *, int32_t *, void *);
+
   public:
-    TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, int seqCount);
+    // maxOutputs: the widest matrix product a caller will run through this object's buffers (the vocabulary size for
+    // ComputePrediction; 0 = the layer's own products only)
+    TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, int maxRows, int64_t maxOutputs = 0);
     ~TLayerComputer();
     TLayerComputer(const TLayerComputer &) = delete;
     TLayerComputer &operator=(const TLayerComputer &) = delete;
@@ -173,7 +185,34 @@ class TLayerComputer
     // state: device [seqCount][Dim] fp32, updated in place; the cache gets the new rows and its lengths grow by one.
     void AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
                           TAttentionVecHistory *pKVCache, float *state, void *stream);
-    const float *GetValLookup() const { return ValLookup; } // [seqCount][HeadCount*TTDim] of the last call
+    // len tokens of the cache's sequences, concatenated (seqOffset: device int32 [seqCount + 1]); pos: device int32 [len],
+    // each token's position in its sequence; spans (and optionally their summary and the launch-order hint) of
+    // att.AttentionWidth as for tsattn_prefill; state: device [len][Dim]; the tokens' rows are appended to the cache.
+    void AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
+                                const TAttentionMatrices &att, const int32_t *spanStart, const int32_t *spanFinish,
+                                const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
+                                void *stream);
+    const float *GetValLookup() const { return ValLookup; } // [rows][HeadCount*TTDim] of the last call
 };
+
+// The model around the layers: TCPUModelParams of the reference (gpt/train/cpu_infer.cpp:58-86), device copies.
+struct TInferModel {
+    const int8_t *LabelEmbed = nullptr; // [LabelCount][Dim]
+    float LabelEmbedScale = 0;
+    int64_t LabelCount = 0;
+    std::vector<TAttentionMatrices> LayerArr;
+    const int8_t *FinalLayer = nullptr; // [VocabSize][Dim]
+    float FinalLayerScale = 0;
+    int64_t VocabSize = 0;
+    const float *Bias = nullptr;        // [VocabSize]
+};
+
+// ComputePrediction (gpt/train/cpu_infer.cpp:552-582) for one new token per sequence: embedding of `labels` (device
+// int32 [seqCount], one label per token) -> every layer's AddLookupProduct on its own cache -> NormalizeState,
+// MulForward(FinalLayer), SoftMax.  state: device scratch [seqCount][Dim].  prediction (device [seqCount][VocabSize],
+// nullable) receives the distribution, choice (device int32 [seqCount], nullable) the most likely label.
+void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const std::vector<TAttentionVecHistory *> &kvCaches,
+                       const int32_t *labels, const int32_t *t, const float *ropeBuf, int64_t ropeLen, float *state,
+                       float *prediction, int32_t *choice, void *stream);
 
 } // namespace NTsAttn
