@@ -29,7 +29,7 @@ dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
 @pytest.mark.parametrize("m,n,k", [
     (1, 32, 64), (32, 2048, 2048), (31, 100, 192), (33, 33, 64), (64, 40, 1024), (128, 96, 320),     # few rows
     (129, 128, 64), (300, 257, 192), (1000, 130, 2048), (256, 256, 4096), (131, 1, 128),             # many rows
-    (8192, 4096, 128), (8000, 4100, 64),                                                             # many rows, tall output tiles
+    (8192, 4096, 128), (8000, 4100, 64), (8000, 4100, 384), (4096, 8192, 1024),                      # the largest output tiles
 ])
 def test_matmul_int32_bit_exact(ctx, m, n, k):
     rng = np.random.default_rng(m + 7 * n + k)
@@ -50,7 +50,7 @@ def test_matmul_extremes(ctx, m):
     assert got[0, 0] == 127 * 127 * k and got[1, 0] == -127 * 127 * k and got[0, 3] == -127 * 127 * k
 
 
-@pytest.mark.parametrize("m,n,k", [(32, 256, 512), (160, 192, 256)])
+@pytest.mark.parametrize("m,n,k", [(32, 256, 512), (160, 192, 256), (4100, 8190, 128)])
 def test_matmul_scaled_forms_and_pitches(ctx, m, n, k):
     """f32 output, AddScaled into a state with a padded pitch, operands with padded pitches; nothing outside the
     [m, n] block is written."""

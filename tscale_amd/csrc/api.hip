@@ -70,6 +70,8 @@ int tsattn_create(const tsattn_config *cfg, tsattn_handle_t *out)
     if (cfg->device < 0 || cfg->device >= n_dev) return fail(TSATTN_ERR_BAD_ARG, "tsattn_create: device %d of %d", cfg->device, n_dev);
     e = hipSetDevice(cfg->device);
     if (e != hipSuccess) return hip_fail(e, "hipSetDevice");
+    e = tsattn::prepare_matmul_i8();
+    if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
     tsattn_ctx *c = new tsattn_ctx();
     c->device = cfg->device;
     c->max_seqs = cfg->max_seqs;

@@ -7,6 +7,7 @@
 // 64 x 64 each, v_mfma_i32_32x32x32_i8; bound by the matrix cores.  Few rows (one token per sequence): the
 // weights are read once from HBM, 32 weight rows per workgroup with K split over its four waves; bound by HBM.
 // Integer sums are exact, so every decomposition gives the same bits.
+#include <type_traits>
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -274,6 +275,137 @@ __global__ __launch_bounds__(GT_THREADS, 2) void gemm_tall_kernel(GemmParams p)
         }
 }
 
+// Wide tiles for the largest products: 256 x 256 outputs by eight waves of 128 x 64, K in steps of 64 bytes, one
+// workgroup per compute unit; per MFMA cycle this moves a third less through LDS and the caches than 256 x 128 tiles.
+// Each SIMD holds two of the waves, one from each half of the workgroup, and the halves run half a step apart: while
+// one half issues the 16 MFMAs of its step, the other does its memory work (requests its share of the tile three
+// steps on, which memory writes straight into LDS, and reads its operands of the next step from LDS), then they swap
+// at a barrier.  The MFMA pipe always has a wave feeding it and no wave waits for memory while it feeds.  Four LDS
+// buffers of 32 KiB: one being read, three tiles on their way (a request has two whole steps to land).
+// LDS rows are 64 bytes without padding; the 16-byte chunks of a row are permuted by (row / 4) % 4, which keeps the
+// row-per-lane operand reads free of bank conflicts; a memory-to-LDS request writes the 64 lanes' 16 bytes one after
+// the other, so the permutation is applied to the addresses the lanes request.  K must be a multiple of 64.
+constexpr int GW_THREADS = 512, GW_BM = 256, GW_BN = 256, GW_BK = 64, GW_NBUF = 4;
+constexpr int GW_BUF = (GW_BM + GW_BN) * GW_BK;
+constexpr int GW_LDS_BYTES = GW_NBUF * GW_BUF;
+
+template <int MODE>
+__global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t gw_lds[];
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int half = wave >> 2; // waves 0-3 and 4-7 land on SIMDs 0-3 each
+    const int wm = wave >> 2, wn = wave & 3;
+    const int li = lane & 31, g = lane >> 5;
+
+    // 8 x 8 blocks of tiles per XCD where the shape allows (see gemm_tiled_kernel)
+    const int64_t tiles_n = (p.n + GW_BN - 1) / GW_BN, tiles_m = (p.m + GW_BM - 1) / GW_BM;
+    int64_t tile_m, tile_n;
+    if (tiles_n % 8 == 0 && tiles_m % 8 == 0 && ((tiles_n >> 3) * (tiles_m >> 3)) % 8 == 0) {
+        const int64_t x = blockIdx.x & 7, l = blockIdx.x >> 3;
+        const int64_t sb = (l >> 6) * 8 + x, within = l & 63;
+        const int64_t sb_per_row = tiles_n >> 3;
+        tile_m = (sb / sb_per_row) * 8 + (within >> 3);
+        tile_n = (sb % sb_per_row) * 8 + (within & 7);
+    } else {
+        tile_m = blockIdx.x / tiles_n;
+        tile_n = blockIdx.x % tiles_n;
+    }
+    const int64_t m0 = tile_m * GW_BM, n0 = tile_n * GW_BN;
+    const __amdgpu_buffer_rsrc_t ar = rows_rsrc(p.a + m0 * p.a_pitch, p.m - m0 < GW_BM ? p.m - m0 : GW_BM, p.a_pitch, p.k);
+    const __amdgpu_buffer_rsrc_t wr = rows_rsrc(p.w + n0 * p.w_pitch, p.n - n0 < GW_BN ? p.n - n0 : GW_BN, p.w_pitch, p.k);
+    // A buffer holds 256 rows of A, then 256 rows of W.  A wave's request fills 16 rows (1 KiB): lane L writes the
+    // chunk at position L % 4 of row L / 4, which is chunk (L % 4) ^ perm(row) of the matrix row.  Rows
+    // wave * 16 + 128 i: perm depends on the lane only.
+    const int sr = wave * 16 + (lane >> 2), sc = (lane & 3) ^ ((lane >> 4) & 3);
+    const int a_off0 = sr * (int)p.a_pitch + sc * 16, a_off1 = a_off0 + 128 * (int)p.a_pitch;
+    const int w_off0 = sr * (int)p.w_pitch + sc * 16, w_off1 = w_off0 + 128 * (int)p.w_pitch;
+    auto request = [&](int kb, uint8_t *buf) __attribute__((always_inline)) { // tile at K offset kb -> buf
+        uint8_t *const d = buf + wave * 16 * GW_BK;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr)(d), 16, a_off0, kb, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr)(d + 128 * GW_BK), 16, a_off1, kb, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (lds_ptr)(d + 256 * GW_BK), 16, w_off0, kb, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (lds_ptr)(d + 384 * GW_BK), 16, w_off1, kb, 0, 0);
+    };
+    // operands: row li of each 32-row block, chunk 2 * h + g of its 64 bytes (h: which 32 bytes of the step)
+    const int f_perm = (li >> 2) & 3;
+    const int f_a = (wm * 128 + li) * GW_BK + ((g ^ f_perm) << 4);
+    const int f_w = (GW_BM + wn * 64 + li) * GW_BK + ((g ^ f_perm) << 4);
+    v4i fa[2][4], fw[2][2];
+    v16i acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = v16i{0};
+
+    // A barrier that waits for this wave's LDS reads only: __syncthreads() would also wait for every tile still on its
+    // way into LDS, which is exactly what must stay in flight.  What has to have landed is waited for by count.
+#define GW_BARRIER                                              \
+    do {                                                        \
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      \
+        __builtin_amdgcn_s_barrier();                           \
+        asm volatile("" ::: "memory");                          \
+    } while (0)
+    const int n_steps = (int)(p.k / GW_BK);
+    // requests past K fetch bytes that are never computed with (or zeros past the rows' end)
+    request(0, gw_lds);
+    request(GW_BK, gw_lds + GW_BUF);
+    request(2 * GW_BK, gw_lds + 2 * GW_BUF);
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); // this wave's share of the first tile has landed
+    GW_BARRIER;
+    if (half == 1) GW_BARRIER; // the second half of the workgroup runs half a step behind the first
+#define GW_FENCE __builtin_amdgcn_sched_barrier(0)
+    for (int s = 0; s < n_steps; ++s) {
+        uint8_t *const cur = gw_lds + (s & 3) * GW_BUF;
+        // memory half: request the tile of step s + 3 into the buffer step s - 1 was read from, read this step's
+        // operands, make sure this wave's share of the tile of step s + 1 has landed before the barrier
+        GW_FENCE;
+        request((s + 3) * GW_BK, gw_lds + ((s + 3) & 3) * GW_BUF);
+        GW_FENCE;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fa[h][i] = *(const v4i *)(cur + ((f_a + i * 32 * GW_BK) ^ (h * 32)));
+#pragma unroll
+            for (int j = 0; j < 2; ++j) fw[h][j] = *(const v4i *)(cur + ((f_w + j * 32 * GW_BK) ^ (h * 32)));
+        }
+        GW_FENCE;
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        GW_BARRIER;
+        // MFMA half
+        GW_FENCE;
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[h][i], fw[h][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_s_setprio(0);
+        GW_FENCE;
+        GW_BARRIER;
+    }
+#undef GW_FENCE
+    if (half == 0) GW_BARRIER;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // nothing may still be on its way into LDS when the workgroup ends
+#undef GW_BARRIER
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int64_t n = n0 + wn * 64 + j * 32 + li;
+            if (n >= p.n) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                if (m < p.m) store_out<MODE>(p, m, n, acc[i][j][r]);
+            }
+        }
+}
+
 // ---- few rows ---------------------------------------------------------------------------------------------------
 // One workgroup per 32 weight rows and part of K.  K is walked in slabs of 1024 bytes: every wave instruction asks
 // for 1 KiB of consecutive memory of one row (the weights are read once, so what matters is that HBM sees long
@@ -395,6 +527,14 @@ void launch_mode(const GemmParams &p, hipStream_t st)
     if (p.m > 32 * GS_MB) {
         // tall output tiles when there are enough rows to fill the chip with them
         const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN;
+        // wide tiles when there are two rounds of them for every compute unit
+        const int64_t wide = ((p.m + GW_BM - 1) / GW_BM) * ((p.n + GW_BN - 1) / GW_BN);
+        // (not for the read-modify-write output: with one workgroup per compute unit nothing runs under a tile's
+        // epilogue, and that one moves eight bytes per output)
+        if (wide >= 512 && p.k % GW_BK == 0 && MODE != TSATTN_MM_ADD_SCALED) {
+            hipLaunchKernelGGL((gemm_wide_kernel<MODE>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, p);
+            return;
+        }
         if (((p.m + 255) / 256) * tiles_n >= 1024) {
             if (p.k % GL_BK == 0) hipLaunchKernelGGL((gemm_tall_kernel<MODE>), dim3((unsigned)(((p.m + 255) / 256) * tiles_n)), dim3(GT_THREADS), 0, st, p);
             else hipLaunchKernelGGL((gemm_tiled_kernel<MODE, 4>), dim3((unsigned)(((p.m + 255) / 256) * tiles_n)), dim3(GT_THREADS), 0, st, p);
@@ -418,6 +558,15 @@ int split_for(const GemmParams &p, int64_t room_bytes)
 }
 
 } // namespace
+
+// Once per device, before the first product: the wide-tile kernels use more LDS than a launch may ask for by default.
+hipError_t prepare_matmul_i8()
+{
+    hipError_t e = hipFuncSetAttribute((const void *)gemm_wide_kernel<TSATTN_MM_I32>, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)gemm_wide_kernel<TSATTN_MM_F32>, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
+    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)gemm_wide_kernel<TSATTN_MM_ADD_SCALED>, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
+    return e;
+}
 
 hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out)
 {

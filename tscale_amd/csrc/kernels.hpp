@@ -147,6 +147,7 @@ struct GemmParams {
 };
 
 hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out);
+hipError_t prepare_matmul_i8(); // once per device, before the first product
 
 struct HeadParams {
     int64_t n_rows;
