@@ -321,6 +321,18 @@ int tsattn_softmax_rows(tsattn_handle_t h, int64_t n_rows, int64_t n, const int3
                         int64_t src_pitch, float scale, const float *bias, float *prob, int64_t prob_pitch, int32_t *argmax,
                         void *stream);
 
+/* SampleFromDistr (gpt/train/cpu_infer.cpp:585-599), the Gumbel-max choice from a distribution:
+ * choice[row] = the first k of the largest score[k] = (float)(logf(prob[k]) / temperature - log(-log(u[k]))), with
+ * u[k] = (r[k] + 0.5) / 2^32 in double, which is GenRandReal3 of the reference's 32-bit generator
+ * (lib/random/mersenne.h:233-235, TXRng = TMersenne<ui32>, gpt/rng/xrng.h:4).  rnd: device uint32 [n_rows][rnd_pitch],
+ * the words r supplied by the caller (for instance that generator's stream), or NULL: the word of (row, k) is then
+ * the upper half of splitmix64's output function applied to seed + (offset + row * n + k + 1) * 0x9E3779B97F4A7C15 --
+ * a counter-based generator: same seed and offset, same choices; advance offset by n_rows * n per call.  This is not
+ * the reference's MT19937 stream; the distribution of the choices is the same.  temperature > 0.
+ * prob f32 [n_rows][prob_pitch] (tsattn_softmax_rows' output); choice int32 [n_rows]. */
+int tsattn_sample_rows(tsattn_handle_t h, int64_t n_rows, int64_t n, const float *prob, int64_t prob_pitch, float temperature,
+                       const uint32_t *rnd, int64_t rnd_pitch, uint64_t seed, uint64_t offset, int32_t *choice, void *stream);
+
 /* The table ApplyRope reads: FillRopeBuf, gpt/att/rope.cpp:4-24.  Host function, host memory:
  * table[t * head_dim + x], t < max_len; copy it to the device once. */
 void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table);

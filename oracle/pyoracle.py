@@ -270,6 +270,25 @@ def softmax_rows(vec, scale, bias=None, exp2_mode=0):
     return prob, arg
 
 
+def mix32(seed, index):
+    L = lib()
+    L.tso_mix32.restype = ctypes.c_uint32
+    return int(L.tso_mix32(ctypes.c_uint64(seed), ctypes.c_uint64(index)))
+
+
+def sample_rows(prob, temperature, rnd=None, seed=0, offset=0):
+    """prob float32 [n_rows, n] -> the Gumbel-max choice per row, int32 [n_rows]; rnd: uint32 words [n_rows, n] or None
+    (the counter generator on seed and offset)."""
+    L = lib()
+    prob = _c_arr(prob, np.float32)
+    n_rows, n = prob.shape
+    r = None if rnd is None else _c_arr(rnd, np.uint32)
+    choice = np.empty(n_rows, dtype=np.int32)
+    L.tso_sample_rows(ctypes.c_int64(n_rows), ctypes.c_int64(n), _p(prob), ctypes.c_int64(n), ctypes.c_float(temperature), _p(r),
+                      ctypes.c_int64(n), ctypes.c_uint64(seed), ctypes.c_uint64(offset), _p(choice))
+    return choice
+
+
 def make_spans(seq_lens, window, doc_start_flag=None):
     L = lib()
     off = np.zeros(len(seq_lens) + 1, dtype=np.int64)

@@ -56,6 +56,10 @@
  *   tso_softmax_rows       train/cpu_infer.cpp:340-355   pinned: scipy's softmax on ln 2 * w (a library routine), rows
  *                                                         sum to 1, adding a constant to the bias changes nothing
  *                                                         while the largest w stays above 0
+ *   tso_sample_rows        train/cpu_infer.cpp:585-599   pinned: frequencies of the choices follow prob^(1/T) normalised
+ *                                                         (the Gumbel-max identity; temperatures 1 and 2), a tiny
+ *                                                         temperature gives the largest probability, words handed in
+ *                                                         and words from the counter generator agree
  *
  * The reference holds no golden vectors or known-answer tests for this path, and the two files
  * that contain it (gpt_cpu.cpp, cpu_infer.cpp) cannot be compiled without the CUDA SDK, so the
@@ -990,4 +994,35 @@ void tso_softmax_rows(int64_t n_rows, int64_t n, const int32_t *vec, float scale
         }
     }
     free(buf);
+}
+
+/* ------------------------------------------------------------------------------------------ */
+/* SampleFromDistr: train/cpu_infer.cpp:585-599                                               */
+
+uint32_t tso_mix32(uint64_t seed, uint64_t index)
+{
+    uint64_t z = seed + (index + 1) * 0x9E3779B97F4A7C15ull; /* splitmix64's output function on a counter */
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (uint32_t)(z >> 32);
+}
+
+void tso_sample_rows(int64_t n_rows, int64_t n, const float *prob, int64_t prob_pitch, float temperature, const uint32_t *rnd,
+                     int64_t rnd_pitch, uint64_t seed, uint64_t offset, int32_t *choice)
+{
+    for (int64_t row = 0; row < n_rows; ++row) {
+        float best = -1e38f;
+        int64_t res = 0;
+        for (int64_t k = 0; k < n; ++k) {
+            const uint32_t r = rnd ? rnd[row * rnd_pitch + k] : tso_mix32(seed, offset + (uint64_t)(row * n + k));
+            const double u = ((double)r + 0.5) * (1.0 / 4294967296.0);
+            const float score = (float)((double)(logf(prob[row * prob_pitch + k]) / temperature) - log(-log(u)));
+            if (score > best) {
+                best = score;
+                res = k;
+            }
+        }
+        choice[row] = (int32_t)res;
+    }
 }

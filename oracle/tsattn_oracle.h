@@ -149,6 +149,15 @@ void tso_embed_rows(int64_t n_rows, int dim, const int32_t *labels, int labels_p
 void tso_softmax_rows(int64_t n_rows, int64_t n, const int32_t *vec, float scale, const float *bias, int exp2_mode, float *prob,
                       int32_t *argmax);
 
+/* ---- SampleFromDistr (train/cpu_infer.cpp:585-599): the Gumbel-max choice ----
+ * score[k] = (float)(logf(prob[k]) / temperature - log(-log(u[k]))), u[k] = (r[k] + 0.5) / 2^32 in double (GenRandReal3 of the
+ * reference's 32-bit generator, lib/random/mersenne.h:233-235); choice = the first k of the largest score above -1e38, else 0.
+ * rnd: the words r, [n_rows][rnd_pitch], or NULL: r[k] of row `row` = tso_mix32(seed, offset + row * n + k) (a counter-based
+ * generator, not the reference's MT19937 stream). */
+uint32_t tso_mix32(uint64_t seed, uint64_t index);
+void tso_sample_rows(int64_t n_rows, int64_t n, const float *prob, int64_t prob_pitch, float temperature, const uint32_t *rnd,
+                     int64_t rnd_pitch, uint64_t seed, uint64_t offset, int32_t *choice);
+
 /* softmax buffer of cpu_infer.cpp:220-281 on its own (for bounding the polynomial):
  * in: n logits (the caller includes the leading 0 if wanted); out: n weights already multiplied by
  * Scale.  Returns Scale. */

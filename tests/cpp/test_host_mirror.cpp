@@ -538,6 +538,13 @@ static int RunPredictionCase()
                     if (choice[b] != wantChoice[b]) { printf("  step %d: sequence %d chose %d, oracle %d\n", step, b, choice[b], wantChoice[b]); ++fails; }
                 }
             }
+            // a sampled choice from the same distribution: the oracle on the probabilities the device produced
+            SampleFromDistr(handle, B, vocab, probDev, 0.9f, 1313, (uint64_t)step * B * vocab, choiceDev, nullptr);
+            HIP_OK(hipDeviceSynchronize());
+            std::vector<int32_t> sampled(B), wantSampled(B);
+            HIP_OK(hipMemcpy(sampled.data(), choiceDev, B * 4, hipMemcpyDeviceToHost));
+            tso_sample_rows(B, vocab, got.data(), vocab, 0.9f, nullptr, 0, 1313, (uint64_t)step * B * vocab, wantSampled.data());
+            if (sampled != wantSampled) { printf("  step %d: sampled choices differ from the oracle's\n", step); ++fails; }
             labels = choice; // greedy generation: the GPU's choice is both sides' next label
         }
         if (maxProb > 0.1) ++fails;

@@ -1,5 +1,5 @@
-"""GPU: the embedding sum and the final softmax with the greedy choice (ComputePrediction, gpt/train/cpu_infer.cpp:552-582)
-through the C ABI against the oracle."""
+"""GPU: the embedding sum, the final softmax with the greedy choice (ComputePrediction, gpt/train/cpu_infer.cpp:552-582) and
+the sampled choice (SampleFromDistr, :585-599) through the C ABI against the oracle."""
 import numpy as np
 import pytest
 import torch
@@ -63,3 +63,39 @@ def test_softmax_rows_ties_and_negative_rows(ctx):
     assert arg.cpu().numpy().tolist() == [77, 0]
     want, _ = orc.softmax_rows(tie, 1e-3)
     assert np.abs(prob.cpu().numpy() - want).max() < 1e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_rows,n,temperature", [(8, 50257, 1.0), (32, 1000, 0.7), (3, 77, 2.5)])
+def test_sample_rows_matches_the_oracle(ctx, n_rows, n, temperature):
+    """SampleFromDistr on the device against the oracle, with the caller's random words and with the counter-based
+    generator.  Scores are compared through the choice: a different index is accepted only where the oracle's own
+    scores of the two indices are within rounding of each other (logf and log differ in the last bit between libm
+    and the device)."""
+    rng = np.random.default_rng(n)
+    w = (rng.standard_normal((n_rows, n)) * 3).astype(np.float32)
+    prob = np.exp(w - w.max(axis=1, keepdims=True)); prob = (prob / prob.sum(axis=1, keepdims=True)).astype(np.float32)
+    prob[0, 5] = 0.0                                                     # never chosen
+    words = rng.integers(0, 2**32, (n_rows, n), dtype=np.uint64).astype(np.uint32)
+    dprob = torch.from_numpy(prob).cuda()
+    for rnd, seed, offset in ((words, 0, 0), (None, 1313, 12345)):
+        want = orc.sample_rows(prob, temperature, rnd=rnd, seed=seed, offset=offset)
+        drnd = None if rnd is None else torch.from_numpy(rnd.view(np.int32)).cuda()
+        got = ctx.sample_rows(dprob, temperature, rnd=drnd, seed=seed, offset=offset).cpu().numpy()
+        for i in np.nonzero(got != want)[0]:
+            r = rnd[i] if rnd is not None else np.array([orc.mix32(seed, offset + i * n + k) for k in range(n)], dtype=np.uint32)
+            u = (r.astype(np.float64) + 0.5) / 2.0**32
+            with np.errstate(divide="ignore"):
+                score = np.log(prob[i].astype(np.float64)) / temperature - np.log(-np.log(u))
+            assert abs(score[got[i]] - score[want[i]]) < 1e-5 * max(1.0, abs(score[want[i]])), (i, got[i], want[i])
+        assert got[0] != 5
+
+
+@pytest.mark.gpu
+def test_sample_rows_argument_checks(ctx):
+    from tscale_amd import capi
+    prob = torch.full((2, 10), 0.1, dtype=torch.float32, device="cuda")
+    with pytest.raises(capi.TsattnError):
+        ctx.sample_rows(prob, 0.0)
+    with pytest.raises(capi.TsattnError):
+        ctx.sample_rows(prob, -1.0)

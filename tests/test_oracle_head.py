@@ -43,3 +43,30 @@ def test_softmax_rows_is_a_base_2_softmax_with_a_floor_on_the_maximum():
     # ties: the first index wins
     tie = np.zeros((1, 16), dtype=np.int32); tie[0, [5, 9]] = 7
     assert orc.softmax_rows(tie, 1.0)[1].tolist() == [5]
+
+
+def test_sample_rows_draws_from_the_tempered_distribution():
+    """SampleFromDistr (cpu_infer.cpp:585-599) is the Gumbel-max trick: argmax of log p / T + Gumbel noise is a draw
+    from p^(1/T) normalised.  A wrong sign, a missing logarithm or a dropped temperature changes the frequencies."""
+    p = np.array([0.4, 0.25, 0.15, 0.1, 0.07, 0.03], dtype=np.float32)
+    draws = 200000
+    prob = np.tile(p, (draws, 1))
+    for temperature in (1.0, 2.0):
+        choice = orc.sample_rows(prob, temperature, seed=17, offset=int(temperature * 1000))
+        want = p.astype(np.float64) ** (1.0 / temperature)
+        want /= want.sum()
+        freq = np.bincount(choice, minlength=6) / draws
+        sigma = np.sqrt(want * (1 - want) / draws)
+        assert (np.abs(freq - want) < 4.5 * sigma).all(), (temperature, freq, want)
+    # a tiny temperature: the noise no longer matters, the largest probability wins; ties go to the first index
+    rng = np.random.default_rng(5)
+    q = rng.random((64, 300)).astype(np.float32)
+    q[np.arange(64), rng.integers(0, 300, 64)] = 3.0           # a clear winner per row
+    q /= q.sum(axis=1, keepdims=True)
+    assert np.array_equal(orc.sample_rows(q, 1e-3, seed=3), q.argmax(axis=1))
+    # words handed in by the caller and the counter generator's own words are the same thing
+    words = np.array([[orc.mix32(99, 7 + r * 300 + k) for k in range(300)] for r in range(4)], dtype=np.uint32)
+    assert np.array_equal(orc.sample_rows(q[:4], 0.8, rnd=words), orc.sample_rows(q[:4], 0.8, seed=99, offset=7))
+    # probability zero is never chosen
+    z = np.zeros((3, 50), dtype=np.float32); z[:, 31] = 1.0
+    assert (orc.sample_rows(z, 1.0, seed=1) == 31).all()

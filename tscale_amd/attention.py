@@ -206,6 +206,20 @@ class AttentionContext:
                                                 _ptr(prob), n, _ptr(argmax), _stream_ptr()))
         return prob, argmax
 
+    def sample_rows(self, prob, temperature, rnd=None, seed=0, offset=0, choice=None):
+        """SampleFromDistr (cpu_infer.cpp:585-599), the Gumbel-max choice: prob f32 [n_rows, n] -> int32 [n_rows].  rnd: the
+        caller's uint32 words [n_rows, n], or None = the counter-based generator on (seed, offset)."""
+        n_rows, n = prob.shape
+        assert prob.dtype == torch.float32 and prob.stride(1) == 1
+        if rnd is not None:
+            assert rnd.shape == prob.shape and rnd.element_size() == 4 and rnd.stride(1) == 1
+        if choice is None:
+            choice = torch.empty(n_rows, dtype=torch.int32, device=prob.device)
+        capi.check(self.lib.tsattn_sample_rows(self.handle, n_rows, n, _ptr(prob), prob.stride(0), float(temperature), _ptr(rnd),
+                                               rnd.stride(0) if rnd is not None else 0, int(seed), int(offset), _ptr(choice),
+                                               _stream_ptr()))
+        return choice
+
     def build_spans(self, seq_offset, n_tokens, window, doc_start_flag=None):
         """seq_offset: int32 [n_seqs+1] on the device.  Returns (span_start, span_finish) int32 [n_tokens]."""
         st = torch.empty(n_tokens, dtype=torch.int32, device=self.device)

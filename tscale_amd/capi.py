@@ -104,7 +104,7 @@ class FillArgs(_c.Structure):
 
 
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_embed_rows", "tsattn_softmax_rows", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
+           "tsattn_decode", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_embed_rows", "tsattn_softmax_rows", "tsattn_sample_rows", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
 
 _lib = None
 
@@ -153,6 +153,9 @@ def load():
         L.tsattn_softmax_rows.restype = _c.c_int
         L.tsattn_softmax_rows.argtypes = [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_float,
                                           _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p]
+        L.tsattn_sample_rows.restype = _c.c_int
+        L.tsattn_sample_rows.argtypes = [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_float, _c.c_void_p, _c.c_int64,
+                                         _c.c_uint64, _c.c_uint64, _c.c_void_p, _c.c_void_p]
         L.tsattn_quantize_rows.restype = _c.c_int
         L.tsattn_quantize_rows.argtypes = [_c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64,
                                            _c.c_int, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64,

@@ -414,6 +414,23 @@ int tsattn_softmax_rows(tsattn_handle_t h, int64_t n_rows, int64_t n, const int3
     return TSATTN_OK;
 }
 
+int tsattn_sample_rows(tsattn_handle_t h, int64_t n_rows, int64_t n, const float *prob, int64_t prob_pitch, float temperature,
+                       const uint32_t *rnd, int64_t rnd_pitch, uint64_t seed, uint64_t offset, int32_t *choice, void *stream)
+{
+    if (!h) return fail(TSATTN_ERR_BAD_ARG, "tsattn_sample_rows: null handle");
+    if (n_rows < 0 || n <= 0 || n > 0x7fffffff) return fail(TSATTN_ERR_BAD_ARG, "tsattn_sample_rows: sizes");
+    if (n_rows == 0) return TSATTN_OK;
+    if (!prob || !choice) return fail(TSATTN_ERR_BAD_ARG, "tsattn_sample_rows: null data pointer");
+    if (prob_pitch < n || (rnd && rnd_pitch < n)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_sample_rows: pitches must cover a row");
+    if (!(temperature > 0.0f)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_sample_rows: temperature %g must be positive", (double)temperature);
+    tsattn::HeadParams p = {};
+    p.n_rows = n_rows; p.n = n; p.prob = const_cast<float *>(prob); p.prob_pitch = prob_pitch; p.temperature = temperature;
+    p.rnd = rnd; p.rnd_pitch = rnd_pitch; p.seed = seed; p.offset = offset; p.argmax = choice;
+    hipError_t e = tsattn::launch_sample_rows(p, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "sampling launch");
+    return TSATTN_OK;
+}
+
 void tsattn_fill_rope_table(int head_dim, int64_t max_len, float *table)
 {
     if (!table || head_dim <= 0 || head_dim % 64 || max_len <= 0) return;

@@ -1,6 +1,6 @@
 // The two ends of the int8 inference path around the layers (ComputePrediction, gpt/train/cpu_infer.cpp:552-582):
 // the embedding sum that makes the first state, and the softmax over the final layer's products with the greedy
-// choice of the next token.
+// choice of the next token; and the sampled choice (SampleFromDistr, :585-599).
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -90,6 +90,49 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
     for (int64_t k = tid; k < p.n; k += SM_THREADS) p.prob[row * p.prob_pitch + k] = fast_exp2(fmaxf(softmax_logit(p, row, k) - M, -127.0f)) * inv;
 }
 
+
+// SampleFromDistr (cpu_infer.cpp:585-599), the Gumbel-max choice, one workgroup per row:
+// score[k] = (float)(logf(prob[k]) / temperature - log(-log(u))), u = (r + 0.5) / 2^32 in double (GenRandReal3 of the
+// reference's 32-bit generator); the first k of the largest score above -1e38, else 0.  r: the caller's words, or a
+// 64-bit mix of (seed, offset + row * n + k), the output function of splitmix64 on a counter.
+__device__ inline uint32_t mix32(uint64_t seed, uint64_t index)
+{
+    uint64_t z = seed + (index + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (uint32_t)(z >> 32);
+}
+
+__global__ __launch_bounds__(SM_THREADS) void sample_rows_kernel(HeadParams p)
+{
+    __shared__ float s_max[SM_THREADS / WAVE];
+    __shared__ int s_arg[SM_THREADS / WAVE];
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    float best = -1e38f;
+    int arg = 0x7fffffff;
+    for (int64_t k = tid; k < p.n; k += SM_THREADS) {
+        const uint32_t r = p.rnd ? p.rnd[row * p.rnd_pitch + k] : mix32(p.seed, p.offset + (uint64_t)(row * p.n + k));
+        const double u = ((double)r + 0.5) * (1.0 / 4294967296.0);
+        const float score = (float)((double)(logf(p.prob[row * p.prob_pitch + k]) / p.temperature) - log(-log(u)));
+        if (score > best) { best = score; arg = (int)k; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, WAVE);
+        const int oa = __shfl_xor(arg, o, WAVE);
+        if (ob > best || (ob == best && oa < arg)) { best = ob; arg = oa; }
+    }
+    if (lane == 0) { s_max[wave] = best; s_arg[wave] = arg; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < SM_THREADS / WAVE; ++w) {
+            if (s_max[w] > best || (s_max[w] == best && s_arg[w] < arg)) { best = s_max[w]; arg = s_arg[w]; }
+        }
+        p.argmax[row] = arg == 0x7fffffff ? 0 : arg;
+    }
+}
+
 hipError_t launch_embed_rows(const HeadParams &p, hipStream_t st)
 {
     const int64_t n = p.n_rows * (p.dim / 16);
@@ -102,6 +145,13 @@ hipError_t launch_softmax_rows(const HeadParams &p, hipStream_t st)
 {
     if (p.n_rows == 0 || p.n == 0) return hipSuccess;
     hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)p.n_rows), dim3(SM_THREADS), 0, st, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_sample_rows(const HeadParams &p, hipStream_t st)
+{
+    if (p.n_rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(sample_rows_kernel, dim3((unsigned)p.n_rows), dim3(SM_THREADS), 0, st, p);
     return hipGetLastError();
 }
 

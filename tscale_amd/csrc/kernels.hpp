@@ -170,10 +170,16 @@ struct HeadParams {
     float *prob;
     int64_t prob_pitch;
     int32_t *argmax;
+    // sampling
+    float temperature;
+    const uint32_t *rnd;
+    int64_t rnd_pitch;
+    uint64_t seed, offset;
 };
 
 hipError_t launch_embed_rows(const HeadParams &p, hipStream_t st);
 hipError_t launch_softmax_rows(const HeadParams &p, hipStream_t st);
+hipError_t launch_sample_rows(const HeadParams &p, hipStream_t st);
 
 struct FillParams {
     const int32_t *seq_offset;

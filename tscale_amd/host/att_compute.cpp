@@ -446,4 +446,11 @@ void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const st
     }
 }
 
+void SampleFromDistr(tsattn_handle_t handle, int rows, int64_t vocabSize, const float *prediction, float temperature, uint64_t seed,
+                     uint64_t offset, int32_t *choice, void *stream)
+{
+    Check(tsattn_sample_rows(handle, rows, vocabSize, prediction, vocabSize, temperature, nullptr, 0, seed, offset, choice, stream),
+          "tsattn_sample_rows");
+}
+
 } // namespace NTsAttn

@@ -11,6 +11,7 @@
 //   TCPUModelParams::TAttentionMatrices    gpt/train/cpu_infer.cpp:60-77              NTsAttn::TAttentionMatrices
 //   AddLookupProduct                       gpt/train/cpu_infer.cpp:465-527            TLayerComputer::AddLookupProduct(Prompt)
 //   ComputePrediction                      gpt/train/cpu_infer.cpp:552-582            NTsAttn::ComputePrediction
+//   SampleFromDistr                        gpt/train/cpu_infer.cpp:585-599            NTsAttn::SampleFromDistr
 //
 // All arithmetic runs in libtsattn.so through the C ABI of include/tsattn.h; this layer owns the
 // per-context device buffers (allocated once, like TAttentionComputeCtx::AllocateCuda,
@@ -214,5 +215,11 @@ struct TInferModel {
 void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const std::vector<TAttentionVecHistory *> &kvCaches,
                        const int32_t *labels, const int32_t *t, const float *ropeBuf, int64_t ropeLen, float *state,
                        float *prediction, int32_t *choice, void *stream);
+
+// SampleFromDistr (gpt/train/cpu_infer.cpp:585-599) for every row of a batch of distributions: the Gumbel-max choice at
+// the given temperature.  The random words come from the library's counter-based generator (same seed and offset:
+// same choices; advance offset by rows * vocabSize per call), not from the reference's MT19937 stream.
+void SampleFromDistr(tsattn_handle_t handle, int rows, int64_t vocabSize, const float *prediction, float temperature, uint64_t seed,
+                     uint64_t offset, int32_t *choice, void *stream);
 
 } // namespace NTsAttn
