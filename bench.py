@@ -380,10 +380,10 @@ class Int8Layers:
 
 def bench_token_step(ctx, steps):
     """One generated token per sequence through all 24 layers (per layer: state normalisation, four projections,
-    RoPE + per-head normalisation, cache append + attention over the cache, KVProduct, combiner, feed-forward; 11-12
+    RoPE + per-head normalisation, cache append + attention over the cache with KVProduct, combiner, feed-forward; 9-10
     library calls), B32 at cache length 2048+."""
     import torch
-    from tscale_amd.attention import add_lookup_product
+    from tscale_amd.attention import add_lookup_product, flush_state
     m = Int8Layers(ctx, cache_len=2048, seed=1313 + 9)
     B, H, d, dim, qsum = m.B, m.H, m.d, m.dim, m.H * m.d
     state = torch.randn((B, dim), device="cuda", generator=m.g)
@@ -391,8 +391,10 @@ def bench_token_step(ctx, steps):
     room = torch.empty(16 * 4 * B * max(dim, qsum), dtype=torch.uint8, device="cuda")
     keep = {}
     def step():
+        pending = None
         for layer, c in zip(m.layers, m.caches):
-            add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep)
+            _, pending = add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep, pending=pending, defer=True)
+        flush_state(ctx, pending, state)
         t.add_(1)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -410,7 +412,7 @@ def bench_token_step(ctx, steps):
     n = m.prompt + 1 + reps // 2
     cache_bytes = sum(B * H * min(n - 1, w) * (2 * d + 8) for w, _ in m.sched)
     return {"config": "24 layers, B32, cache length ~2048+, model width 2048, 16 heads x 128, int8 weights and KV cache; "
-                      "11-12 library calls per layer in one HIP graph per token",
+                      "9-10 library calls per layer in one HIP graph per token",
             "ms_per_token_step": round(ms, 4), "tokens_per_s": round(B / ms * 1e3, 1),
             "weight_bytes": m.weight_bytes, "cache_bytes_per_step": cache_bytes,
             "GB/s": round((m.weight_bytes + cache_bytes) / ms / 1e6, 1),
@@ -424,7 +426,7 @@ def bench_generate_model(ctx, steps):
     import numpy as np
     import torch
     from tscale_amd import capi
-    from tscale_amd.attention import add_lookup_product, VEC_SCALE, STATE_NORM_TILE
+    from tscale_amd.attention import add_lookup_product, flush_state, VEC_SCALE
     m = Int8Layers(ctx, cache_len=2048, seed=1313 + 11)
     B, H, d, dim, qsum = m.B, m.H, m.d, m.dim, m.H * m.d
     vocab = 50257
@@ -442,9 +444,10 @@ def bench_generate_model(ctx, steps):
     keep = {}
     def step():
         ctx.embed_rows(labels, embed, 0.03, out=state)
+        pending = None
         for layer, c in zip(m.layers, m.caches):
-            add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep)
-        norm, _ = ctx.rope_normalize_rows(state, dim // STATE_NORM_TILE, capi.I8)
+            _, pending = add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep, pending=pending, defer=True)
+        norm = flush_state(ctx, pending, state)
         logits = ctx.matmul_i8(norm, final, mode=capi.MM_I32_PLANES, out=planes)
         ctx.softmax_rows(logits, final_scale, bias, want_prob=False, argmax=labels)
         t.add_(1)

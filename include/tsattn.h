@@ -149,6 +149,15 @@ typedef struct tsattn_decode_args {
     const void *k_new, *v_new; /* [n_seqs][n_heads*head_dim] 8-bit */
     int64_t new_pitch;         /* bytes per sequence, multiple of 16 */
     const float *k_scale_new, *v_scale_new; /* [n_seqs][n_heads]; NULL = leave the scale planes untouched */
+    /* Optional fused consumer (kv_out == NULL = off): KVProduct of the result with the token's K vector, as
+     * tsattn_kv_product(k = kv_k, value = out, mult = kv_mult) would make it from `out` afterwards (cpu_infer.cpp:511,
+     * :320-337); `out` is written as well. */
+    const void *kv_k;          /* int8 [n_seqs][n_heads*head_dim], row pitch kv_k_pitch bytes, 4-byte aligned */
+    int64_t kv_k_pitch;
+    void *kv_out;              /* int8 [n_seqs][n_heads*kv_rep*head_dim], row pitch kv_out_pitch bytes */
+    int64_t kv_out_pitch;
+    int kv_rep;                /* 1..4 */
+    float kv_mult;
 } tsattn_decode_args;
 
 int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream);

@@ -187,3 +187,30 @@ def test_decode_randomised_shapes(ctx, seed):
         assert cache.cache_len.cpu().numpy().tolist() == new_lens, what
         assert np.array_equal(cache.k.cpu().numpy(), k) and np.array_equal(cache.k_scale.cpu().numpy(), ks), what
     assert np.abs(out - want).max() < 1e-4 * max(1.0, np.abs(want).max()), what
+
+
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("window,splits", [(10 ** 6, 1), (10 ** 6, 4), (64, 0), (0, 1), (1, 2)])
+def test_decode_fused_kv_product_equals_the_separate_call(ctx, d, window, splits):
+    """KVProduct written by the decode launches (one split: by the attention kernel; several: by the merge) is what
+    tsattn_kv_product makes from the stored output, byte for byte, and what the oracle makes from it; sequences
+    without keys give zeros."""
+    B, H, L, rep = 5, 4, 300, 4
+    lens = [300, 1, 17, 0, 129]
+    rng = np.random.default_rng(d + window % 1000 + splits)
+    k, v, ks, vs = make_cache(900 + d, capi.I8, B, H, L, d, lens)
+    q, qs = orc.quantize_rows(capi.I8, rng.standard_normal((B, H * d)).astype(np.float32), H)
+    cache = gpu_cache(ctx, capi.I8, k, v, ks, vs, lens)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    kvec = rng.integers(-127, 128, (B, H * d + 16)).astype(np.int8)          # the token's K vector, padded pitch
+    dk = dev(kvec.view(np.uint8))[:, :H * d]
+    kv = torch.full((B, H * rep * d + 32), 99, dtype=torch.uint8, device="cuda")
+    mult = 0.75
+    out = ctx.compute_val_lookup_decode(cache, dev(q), dev(np.ascontiguousarray(qs.T)), window, 0.25, n_splits=splits,
+                                        kv_product=(dk, kv[:, :H * rep * d], rep, mult))
+    torch.cuda.synchronize()
+    want = ctx.kv_product(dk, out, H, rep, mult=mult).cpu().numpy()
+    assert np.array_equal(kv[:, :H * rep * d].cpu().numpy(), want)
+    assert (kv[:, H * rep * d:] == 99).all()
+    assert np.array_equal(want.view(np.int8), orc.kv_product(kvec[:, :H * d], out.cpu().numpy(), H, rep, mult))
+    assert not want[3].any()                                                   # the empty sequence

@@ -8,7 +8,7 @@ import torch
 
 from oracle import pyoracle as orc
 from tscale_amd import KVCache, capi
-from tscale_amd.attention import VEC_SCALE, add_lookup_product
+from tscale_amd.attention import VEC_SCALE, add_lookup_product, flush_state
 
 pytestmark = pytest.mark.gpu
 
@@ -121,3 +121,44 @@ def test_prompt_layer_equals_the_oracle_token_by_token(ctx, width, slope):
     rms = np.sqrt((want.astype(np.float64) ** 2).mean())
     assert np.abs(got - want).max() / rms < 5e-2
     assert np.sqrt(((got - want).astype(np.float64) ** 2).mean()) / rms < 5e-3
+
+
+def test_deferred_state_updates_give_the_same_bits(ctx):
+    """Three layers, three tokens: each layer's last state update left to the next layer's first normalisation (and to
+    flush_state after the last) gives the same states, cache rows and attention outputs as updating at once."""
+    B, H, d, dim, max_len = 4, 2, 128, 256, 8
+    qsum = H * d
+    rng = np.random.default_rng(77)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    mat = lambda n, k: dev(np.clip(np.rint(rng.standard_normal((n, k)) * 32), -127, 127).astype(np.int8).view(np.uint8))
+    layers = [{"proj": mat(4 * qsum, dim), "combiner": mat(dim, qsum * 4), "expand": mat(qsum, dim), "contract": mat(dim, qsum),
+               "qv_scale": 0.031, "combiner_scale": 0.027, "contract_scale": 0.035, "width": w, "slope": s}
+              for w, s in ((1, 0.0), (0, 0.0), (1000, 0.5))]
+    rope = dev(orc.fill_rope(d, 64))
+    start = rng.standard_normal((B, dim)).astype(np.float32) * 2
+    results = []
+    for defer in (False, True):
+        caches = [KVCache(ctx, capi.I8, B, H, max_len, d) for _ in layers]
+        for c in caches:
+            c.k.zero_(); c.v.zero_(); c.k_scale.zero_(); c.v_scale.fill_(VEC_SCALE); c.cache_len.zero_()
+        state = dev(start)
+        keep, vals = {}, []
+        for step in range(3):
+            t = torch.full((B,), step, dtype=torch.int32, device="cuda")
+            pending = None
+            for layer, c in zip(layers, caches):
+                if defer:
+                    val, pending = add_lookup_product(ctx, layer, c, t, rope, state, scratch=keep, pending=pending, defer=True)
+                else:
+                    val = add_lookup_product(ctx, layer, c, t, rope, state, scratch=keep)
+                vals.append(val.cpu().numpy().copy())
+            if defer:
+                norm = flush_state(ctx, pending, state)
+                want_norm, _ = ctx.rope_normalize_rows(state, dim // 128, capi.I8)
+                assert torch.equal(norm, want_norm)
+        torch.cuda.synchronize()
+        results.append((state.cpu().numpy(), [c.k.cpu().numpy() for c in caches], [c.k_scale.cpu().numpy() for c in caches], vals))
+    a, b = results
+    assert np.array_equal(a[0], b[0])
+    for x, y in zip(a[1] + a[2] + a[3], b[1] + b[2] + b[3]):
+        assert np.array_equal(x, y)

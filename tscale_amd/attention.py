@@ -273,9 +273,11 @@ class AttentionContext:
 
     # ---- decode ---------------------------------------------------------------------------------
     def compute_val_lookup_decode(self, cache, q, q_scale, window, alibi_slope, out=None, n_splits=0,
-                                  debug_qk_acc=None, max_len=None, append=None):
+                                  debug_qk_acc=None, max_len=None, append=None, kv_product=None):
         """q: uint8 [B, H*d] with q_scale f32 [B, H] (or a number), or bfloat16 [B, H*d] (quantised in the kernel).
-        append = (k_new, k_scale_new, v_new, v_scale_new): KVCache.add_vectors fused into the same launches."""
+        append = (k_new, k_scale_new, v_new, v_scale_new): KVCache.add_vectors fused into the same launches.
+        kv_product = (k, kv_out, rep, mult): KVProduct of the result with the token's K vector, written by the same
+        launches (k uint8 [B, H*d], kv_out uint8 [B, H*rep*d])."""
         B, H, d = cache.n_seqs, cache.n_heads, cache.head_dim
         if out is None:
             out = torch.empty((B, H * d), dtype=torch.float32, device=q.device)
@@ -303,6 +305,10 @@ class AttentionContext:
             k_new, ks_new, v_new, vs_new = append
             a.k_new, a.v_new, a.new_pitch = _ptr(k_new), _ptr(v_new), k_new.stride(0)
             a.k_scale_new, a.v_scale_new = _ptr(ks_new), _ptr(vs_new)
+        if kv_product is not None:
+            kk, kv_out, rep, mult = kv_product
+            a.kv_k, a.kv_k_pitch, a.kv_out, a.kv_out_pitch = _ptr(kk), kk.stride(0), _ptr(kv_out), kv_out.stride(0)
+            a.kv_rep, a.kv_mult = int(rep), float(mult)
         capi.check(self.lib.tsattn_decode(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
 
@@ -312,14 +318,17 @@ STATE_NORM_TILE = 128     # gpt/model_params/model_dim.h:22
 COMBINER_REP = 4          # gpt/model_params/model_dim.h:12
 
 
-def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None, scratch=None):
+def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None, scratch=None, pending=None, defer=False):
     """One layer of the int8 inference path for one new token per sequence: AddLookupProduct,
-    gpt/train/cpu_infer.cpp:465-527, as a chain of 11-12 library calls (the C++ form is NTsAttn::TLayerComputer).
+    gpt/train/cpu_infer.cpp:465-527, as a chain of 10-11 library calls (the C++ form is NTsAttn::TLayerComputer).
     layer: dict with uint8 (int8 bytes) matrices proj [4*H*d, dim] (the QK, QV, K and V matrices one after the other),
     combiner [dim, 4*H*d], expand [H*d, dim], contract [dim, H*d], floats qv_scale, combiner_scale, contract_scale, and
     width, slope.  cache: KVCache whose value scales are VEC_SCALE; t: int32 [B] positions; rope: table of
     fill_rope_table; state: f32 [B, dim], updated in place.  scratch: dict for buffers kept between calls.
-    Returns the attention output [B, H*d]."""
+    Returns the attention output [B, H*d].
+    defer=True leaves the layer's last state update (contract's AddScaled) undone and returns (attention output,
+    pending): the next layer's first normalisation does it when given `pending` (one launch less per layer), and
+    flush_state does it after the last layer."""
     B, dim = state.shape
     H, d = cache.n_heads, cache.head_dim
     qsum = H * d
@@ -330,19 +339,27 @@ def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None, scratc
         sc["planes"] = torch.empty((16, B, max(4 * qsum, dim)), dtype=torch.int32, device=state.device)
         sc["v_scale"] = torch.full((B, H), VEC_SCALE, dtype=torch.float32, device=state.device)
     planes_buf, v_scale = sc["planes"], sc["v_scale"]
-    norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
+    if pending is not None:   # the previous layer's contract product, still in parts: state += sum * scale, then normalise
+        norm, _ = ctx.rope_normalize_rows(pending[0], groups, capi.I8, resid=state, resid_scale=pending[1])
+    else:
+        norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
     # the four projections as one product; RoPE on the qk and qv heads, per-head normalisation of all four in one call
     proj = ctx.matmul_i8(norm, layer["proj"], mode=capi.MM_I32_PLANES, out=planes_buf)
     key_mult = float(f32(layer["qv_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(dim))))
     q4, qv_scale = ctx.rope_normalize_rows(proj, 4 * H, capi.I8, pos=t, rope=rope, scale_mult=key_mult, row_major_scale=True,
                                            rope_heads=2 * H, scale_heads=(H, H))
     qk, qv, k, v = q4[:, :qsum], q4[:, qsum:2 * qsum], q4[:, 2 * qsum:3 * qsum], q4[:, 3 * qsum:]
+    if "kv" not in sc:
+        sc["kv"] = torch.empty((B, qsum * COMBINER_REP), dtype=torch.uint8, device=state.device)
+        sc["val"] = torch.empty((B, qsum), dtype=torch.float32, device=state.device)
+    kv, val = sc["kv"], sc["val"]
+    fused_kv = (k, kv, COMBINER_REP, 1.0)   # KVProduct written by the attention launches themselves
     if layer["width"] == 0:   # the token attends to the row being written: append first
         cache.add_vectors(qv, qv_scale, v, v_scale)
-        val = ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, 0, layer["slope"])
+        ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, 0, layer["slope"], out=val, kv_product=fused_kv)
     else:
-        val = ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, layer["width"], layer["slope"], append=(qv, qv_scale, v, v_scale))
-    kv = ctx.kv_product(k, val, H, COMBINER_REP)
+        ctx.compute_val_lookup_decode(cache, qk, VEC_SCALE, layer["width"], layer["slope"], out=val, append=(qv, qv_scale, v, v_scale),
+                                      kv_product=fused_kv)
     # combiner; its AddScaled is done by the normalisation that follows
     delta = ctx.matmul_i8(kv, layer["combiner"], mode=capi.MM_I32_PLANES, out=planes_buf)
     norm, _ = ctx.rope_normalize_rows(delta, groups, capi.I8, resid=state,
@@ -350,9 +367,19 @@ def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None, scratc
     relu_src = ctx.matmul_i8(norm, layer["expand"], mode=capi.MM_I32_PLANES, out=planes_buf)
     relu, _ = ctx.rope_normalize_rows(relu_src, H, capi.I8, relu=True)
     relu_dim = relu_src.shape[-1]
-    ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state, workspace=workspace,
-                  scale=float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim)))))
+    contract_scale = float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim))))
+    if defer:
+        parts = ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_I32_PLANES, out=planes_buf)
+        return val, (parts, contract_scale)
+    ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state, workspace=workspace, scale=contract_scale)
     return val
+
+
+def flush_state(ctx, pending, state):
+    """The state update a deferred add_lookup_product left undone; returns NormalizeState of the updated state (what
+    ComputePrediction multiplies with the final layer)."""
+    norm, _ = ctx.rope_normalize_rows(pending[0], state.shape[1] // STATE_NORM_TILE, capi.I8, resid=state, resid_scale=pending[1])
+    return norm
 
 
 def add_lookup_product_prompt(ctx, layer, cache, seq_offset, pos, rope, state, span_start, span_finish, span_tiles=None,

@@ -57,6 +57,8 @@ class DecodeArgs(_c.Structure):
         ("alibi_slope", _c.c_float), ("out", _c.c_void_p), ("n_splits", _c.c_int),
         ("debug_qk_acc", _c.c_void_p), ("debug_pitch", _c.c_int64), ("k_new", _c.c_void_p), ("v_new", _c.c_void_p),
         ("new_pitch", _c.c_int64), ("k_scale_new", _c.c_void_p), ("v_scale_new", _c.c_void_p),
+        ("kv_k", _c.c_void_p), ("kv_k_pitch", _c.c_int64), ("kv_out", _c.c_void_p), ("kv_out_pitch", _c.c_int64),
+        ("kv_rep", _c.c_int), ("kv_mult", _c.c_float),
     ]
 
 

@@ -189,7 +189,7 @@ int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
         if (want > h->max_splits) want = h->max_splits;
         splits = (int)want;
     }
-    tsattn::DecodeParams p;
+    tsattn::DecodeParams p = {};
     p.q = (const uint8_t *)a->q; p.q_pitch = a->q_pitch; p.q_scale = a->q_scale; p.q_scale_const = a->q_scale_const;
     p.k = (const uint8_t *)a->k_cache; p.v = (const uint8_t *)a->v_cache;
     p.seq_stride = a->seq_stride; p.head_stride = a->head_stride; p.tok_stride = a->tok_stride;
@@ -204,6 +204,16 @@ int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
     p.ks_new = a->k_scale_new; p.vs_new = a->v_scale_new;
     p.cache_len_rw = const_cast<int32_t *>(a->cache_len); p.max_len = a->max_len;
     p.seq_done = h->seq_done;
+    if (a->kv_out) {
+        if (!a->kv_k) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: the fused KVProduct needs kv_k");
+        if (a->dtype != TSATTN_I8) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: the fused KVProduct is defined for int8 keys");
+        if (a->kv_rep < 1 || a->kv_rep > 4) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: kv_rep %d (1..4)", a->kv_rep);
+        if (((uintptr_t)a->kv_k & 3) || a->kv_k_pitch % 4 || a->kv_k_pitch < (int64_t)a->n_heads * a->head_dim ||
+            a->kv_out_pitch < (int64_t)a->n_heads * a->head_dim * a->kv_rep)
+            return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: kv_k must be 4-byte aligned and the kv pitches must cover a row");
+        p.kv_k = (const uint8_t *)a->kv_k; p.kv_k_pitch = a->kv_k_pitch; p.kv_out = (uint8_t *)a->kv_out; p.kv_out_pitch = a->kv_out_pitch;
+        p.kv_rep = a->kv_rep; p.kv_mult = a->kv_mult;
+    }
     if (a->k_new || a->v_new) {
         if (!a->k_new || !a->v_new) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: fused append needs both k_new and v_new");
         if (a->window == 0) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: fused append is not available with window 0; call tsattn_cache_append first");

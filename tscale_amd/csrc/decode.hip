@@ -121,6 +121,21 @@ __device__ inline void accumulate_values(float w, v4i vv, float *acc)
     }
 }
 
+// KVProduct of a finished output element (gpt/train/cpu_infer.cpp:320-337): kv[head][blk][x] = int8((k[head][x ^ blk] *
+// value) * mult) for blk < rep; x ^ blk stays inside x's aligned group of four key bytes.  The same arithmetic as
+// kv_product_kernel on the stored output.
+template <int D>
+__device__ inline void kv_product_store(const uint8_t *kv_k, int64_t kv_k_pitch, uint8_t *kv_out, int64_t kv_out_pitch, int rep, float mult,
+                                        int64_t seq, int head, int x, float value)
+{
+    const uint32_t kw = *(const uint32_t *)(kv_k + seq * kv_k_pitch + (int64_t)head * D + (x & ~3));
+    for (int blk = 0; blk < rep; ++blk) {
+        const float key = (float)(int8_t)((kw >> (8 * ((x ^ blk) & 3))) & 0xff);
+        const float y = (key * value) * mult;
+        kv_out[seq * kv_out_pitch + ((int64_t)head * rep + blk) * D + x] = (uint8_t)float_to_i8(y);
+    }
+}
+
 template <int DTYPE, int D, bool QBF16, bool DUMP>
 __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams p)
 {
@@ -193,7 +208,10 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
     const int64_t part = ((int64_t)seq * p.n_heads + head) * p.n_splits + split;
     if (s0 >= s1) { // nothing to do: neutral partial (max 0, sum 0, zeros)
         if (direct) {
-            if (tid < D) p.out[((int64_t)seq * p.n_heads + head) * D + tid] = 0.0f;
+            if (tid < D) {
+                p.out[((int64_t)seq * p.n_heads + head) * D + tid] = 0.0f;
+                if (p.kv_out) kv_product_store<D>(p.kv_k, p.kv_k_pitch, p.kv_out, p.kv_out_pitch, p.kv_rep, p.kv_mult, seq, head, tid, 0.0f);
+            }
             if (count_row) {
                 __syncthreads(); // every thread has read the old length
                 report_done();
@@ -329,7 +347,9 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
         }
         if (direct) {
             // the only split: add the zero vector's weight 2^-M (M >= 0 by construction) and normalise here
-            p.out[((int64_t)seq * p.n_heads + head) * D + tid] = o / (L + fast_exp2(-M));
+            const float res = o / (L + fast_exp2(-M));
+            p.out[((int64_t)seq * p.n_heads + head) * D + tid] = res;
+            if (p.kv_out) kv_product_store<D>(p.kv_k, p.kv_k_pitch, p.kv_out, p.kv_out_pitch, p.kv_rep, p.kv_mult, seq, head, tid, res);
         } else {
             p.part_acc[part * D + tid] = o;
             if (tid == 0) { p.part_ml[part * 2] = M; p.part_ml[part * 2 + 1] = L; }
@@ -341,7 +361,8 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeParams 
 // out = sum_s acc_s 2^(m_s - M) / (2^-M + sum_s l_s 2^(m_s - M)),  M = max(0, max_s m_s)
 template <int D>
 __global__ __launch_bounds__(D) void decode_merge_kernel(const float *part_acc, const float *part_ml, int n_splits, float *out,
-                                                         int32_t *bump_len, int n_heads, int max_len)
+                                                         int32_t *bump_len, int n_heads, int max_len, const uint8_t *kv_k,
+                                                         int64_t kv_k_pitch, uint8_t *kv_out, int64_t kv_out_pitch, int kv_rep, float kv_mult)
 {
     const int64_t sh = blockIdx.x; // seq * n_heads + head
     const int x = threadIdx.x;
@@ -360,7 +381,9 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(const float *part_acc, 
         L += part_ml[(sh * n_splits + s) * 2 + 1] * f;
         o += part_acc[(sh * n_splits + s) * D + x] * f;
     }
-    out[sh * D + x] = o / L;
+    const float res = o / L;
+    out[sh * D + x] = res;
+    if (kv_out) kv_product_store<D>(kv_k, kv_k_pitch, kv_out, kv_out_pitch, kv_rep, kv_mult, sh / n_heads, (int)(sh % n_heads), x, res);
 }
 
 template <int DTYPE, int D>
@@ -389,8 +412,8 @@ hipError_t launch_decode(const DecodeParams &p, int dtype, int head_dim, bool qb
     if (p.n_splits == 1) return hipSuccess; // the split kernel wrote the output (and counted a fused append's row) itself
     dim3 mgrid((unsigned)(n_seqs * p.n_heads));
     int32_t *bump = p.k_new ? p.cache_len_rw : nullptr;
-    if (head_dim == 128) hipLaunchKernelGGL((decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p.part_acc, p.part_ml, p.n_splits, out, bump, p.n_heads, p.max_len);
-    else hipLaunchKernelGGL((decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p.part_acc, p.part_ml, p.n_splits, out, bump, p.n_heads, p.max_len);
+    if (head_dim == 128) hipLaunchKernelGGL((decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p.part_acc, p.part_ml, p.n_splits, out, bump, p.n_heads, p.max_len, p.kv_k, p.kv_k_pitch, p.kv_out, p.kv_out_pitch, p.kv_rep, p.kv_mult);
+    else hipLaunchKernelGGL((decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p.part_acc, p.part_ml, p.n_splits, out, bump, p.n_heads, p.max_len, p.kv_k, p.kv_k_pitch, p.kv_out, p.kv_out_pitch, p.kv_rep, p.kv_mult);
     return hipGetLastError();
 }
 

@@ -36,6 +36,13 @@ struct DecodeParams {
     int32_t *cache_len_rw;
     int max_len;
     int32_t *seq_done; // [n_seqs] arrival counters of the single-split fused append, zero between launches
+    // fused KVProduct of the output (kv_out null = off)
+    const uint8_t *kv_k;
+    int64_t kv_k_pitch;
+    uint8_t *kv_out;
+    int64_t kv_out_pitch;
+    int kv_rep;
+    float kv_mult;
 };
 
 hipError_t launch_decode(const DecodeParams &p, int dtype, int head_dim, bool qbf16, int n_seqs, float *out, hipStream_t st);

@@ -278,14 +278,36 @@ static void Normalize(tsattn_handle_t handle, tsattn_produce_args a, int rows, c
     Check(tsattn_rope_normalize_rows(handle, &a, stream), "tsattn_rope_normalize_rows");
 }
 
+// NormalizeState(state) into NormState; a state update left pending by the previous call (the contract product's parts
+// in Planes) is done first, by the same launch
+void TLayerComputer::NormalizeState(int rows, float *state, void *stream)
+{
+    const int dim = Dims.Dim;
+    if (PendingPlanes > 0) {
+        TS_VERIFY(rows == PendingRows, "a state update of %d rows is pending, this call has %d", PendingRows, rows);
+        tsattn_produce_args a = {};
+        a.resid = state; a.resid_pitch = dim; a.resid_scale = PendingScale;
+        Normalize(Handle, a, rows, Planes, true, PendingPlanes, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
+        PendingPlanes = 0;
+    } else {
+        Normalize(Handle, {}, rows, state, false, 1, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
+    }
+}
+
+const uint8_t *TLayerComputer::FlushState(int rows, float *state, void *stream)
+{
+    NormalizeState(rows, state, stream);
+    return NormState;
+}
+
 // state -> NormalizeState -> the four projections -> ApplyRope on qk and qv, NormalizeState per head on all four: Q4 holds
 // rows of qk, qv, k, v heads; QvHeadScale the key scales as [row][head] (token form) or [head][row] planes (prompt form)
 void TLayerComputer::Projections(int rows, const int32_t *pos, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
-                                 bool scalePlanes, const float *state, void *stream)
+                                 bool scalePlanes, float *state, void *stream)
 {
     const int dim = Dims.Dim, headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
     TS_VERIFY(rows <= MaxRows, "%d rows, buffers for %d", rows, MaxRows);
-    Normalize(Handle, {}, rows, state, false, 1, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
+    NormalizeState(rows, state, stream);
     // Matrices that lie one after the other in memory (QK, QV, K, V) are one product; the result rows hold the qk, qv, k
     // and v heads in that order either way.
     const size_t matBytes = (size_t)qsum * dim;
@@ -314,14 +336,17 @@ void TLayerComputer::Projections(int rows, const int32_t *pos, const float *rope
     Normalize(Handle, a, rows, Planes, true, planes, 4 * headCount, headDim, Q4, stream);
 }
 
-// KVProduct, combiner (its AddScaled done by the normalisation that follows: state += delta * scale, then normalise),
+// KVProduct (unless the attention call made it), combiner (its AddScaled done by the normalisation that follows:
+// state += delta * scale, then normalise),
 // expand, per-head normalisation + ReLU, contract + AddScaled
-void TLayerComputer::AfterAttention(int rows, const TAttentionMatrices &att, float *state, void *stream)
+void TLayerComputer::AfterAttention(int rows, const TAttentionMatrices &att, bool kvDone, bool deferStateUpdate, float *state, void *stream)
 {
     const int dim = Dims.Dim, headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
     const uint8_t *k = Q4 + 2 * (size_t)qsum;
-    Check(tsattn_kv_product(Handle, rows, headCount, headDim, COMBINER_REP, k, 4 * (int64_t)qsum, TSATTN_OUT_F32, ValLookup, qsum, 1.0f, Kv,
-                            (int64_t)qsum * COMBINER_REP, stream), "tsattn_kv_product");
+    if (!kvDone) {
+        Check(tsattn_kv_product(Handle, rows, headCount, headDim, COMBINER_REP, k, 4 * (int64_t)qsum, TSATTN_OUT_F32, ValLookup, qsum, 1.0f, Kv,
+                                (int64_t)qsum * COMBINER_REP, stream), "tsattn_kv_product");
+    }
     const int kvDim = qsum * COMBINER_REP;
     int planes = MulForwardPlanes(rows, Kv, kvDim, att.Combiner, dim, stream);
     {
@@ -335,16 +360,23 @@ void TLayerComputer::AfterAttention(int rows, const TAttentionMatrices &att, flo
         a.relu = 1;
         Normalize(Handle, a, rows, Planes, true, planes, headCount, ReluDim / headCount, Relu, stream);
     }
+    const float contractScale = att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim);
+    if (deferStateUpdate) {
+        PendingPlanes = MulForwardPlanes(rows, Relu, ReluDim, att.Contract, dim, stream);
+        PendingScale = contractScale;
+        PendingRows = rows;
+        return;
+    }
     tsattn_matmul_args ca = {};
     ca.m = rows; ca.n = dim; ca.k = ReluDim;
     ca.a = Relu; ca.a_pitch = ReluDim; ca.w = att.Contract; ca.w_pitch = ReluDim;
-    ca.mode = TSATTN_MM_ADD_SCALED; ca.scale = att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim);
+    ca.mode = TSATTN_MM_ADD_SCALED; ca.scale = contractScale;
     ca.out = state; ca.out_pitch = dim; ca.workspace = Workspace; ca.workspace_bytes = WorkspaceBytes;
     Check(tsattn_matmul_i8(Handle, &ca, stream), "tsattn_matmul_i8");
 }
 
 void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
-                                      TAttentionVecHistory *pKVCache, float *state, void *stream)
+                                      TAttentionVecHistory *pKVCache, float *state, void *stream, bool deferStateUpdate)
 {
     TAttentionVecHistory &kvCache = *pKVCache;
     const int headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum(), rows = kvCache.SeqCount;
@@ -368,6 +400,9 @@ void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, in
     da.cache_len = kvCache.Length; da.max_len = kvCache.MaxLen;
     da.window = att.AttentionWidth; da.alibi_slope = att.AlibiSlope;
     da.out = ValLookup;
+    // KVProduct(k, valLookup) is written by the attention launches themselves
+    da.kv_k = Q4 + 2 * (size_t)qsum; da.kv_k_pitch = pitch4; da.kv_out = Kv; da.kv_out_pitch = (int64_t)qsum * COMBINER_REP;
+    da.kv_rep = COMBINER_REP; da.kv_mult = 1.0f;
     if (att.AttentionWidth == 0) {
         // the token attends to the row being written: append first, in its own call
         tsattn_append_args aa = {};
@@ -383,7 +418,7 @@ void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, in
         da.k_new = qv; da.v_new = v; da.new_pitch = pitch4; da.k_scale_new = QvHeadScale; da.v_scale_new = VHeadScale;
     }
     Check(tsattn_decode(Handle, &da, stream), "tsattn_decode");
-    AfterAttention(rows, att, state, stream);
+    AfterAttention(rows, att, true, deferStateUpdate, state, stream);
 }
 
 void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
@@ -422,7 +457,7 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
     fa.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; fa.s_head_stride = kvCache.MaxLen;
     fa.cache_len = kvCache.Length; fa.max_len = kvCache.MaxLen;
     Check(tsattn_cache_fill(Handle, &fa, stream), "tsattn_cache_fill");
-    AfterAttention(len, att, state, stream);
+    AfterAttention(len, att, false, false, state, stream);
 }
 
 void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const std::vector<TAttentionVecHistory *> &kvCaches,
@@ -435,9 +470,10 @@ void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const st
     Check(tsattn_embed_rows(layer.Handle, rows, dim, labels, 1, model.LabelEmbed, dim, model.LabelCount, model.LabelEmbedScale, state, dim, stream),
           "tsattn_embed_rows");
     // apply layers
-    for (size_t d = 0; d < model.LayerArr.size(); ++d) layer.AddLookupProduct(t, ropeBuf, ropeLen, model.LayerArr[d], kvCaches[d], state, stream);
+    // every layer leaves its last state update to the next one's first normalisation, the last layer to FlushState
+    for (size_t d = 0; d < model.LayerArr.size(); ++d) layer.AddLookupProduct(t, ropeBuf, ropeLen, model.LayerArr[d], kvCaches[d], state, stream, true);
+    layer.FlushState(rows, state, stream); // NormalizeState of the final state
     if (prediction || choice) {
-        Normalize(layer.Handle, {}, rows, state, false, 1, dim / STATE_NORM_TILE, STATE_NORM_TILE, layer.NormState, stream);
         const int planes = layer.MulForwardPlanes(rows, layer.NormState, dim, model.FinalLayer, (int)model.VocabSize, stream);
         // finalScale = CalcDotScale(dim) * CalcFinalLayerMult() * params.FinalLayerScale * VEC_SCALE
         const float finalScale = sqrtf(1.0f / (float)dim) * (1.0f / 0.693147f) * model.FinalLayerScale * VEC_SCALE;

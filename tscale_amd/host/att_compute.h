@@ -149,8 +149,8 @@ constexpr int COMBINER_REP = 4;        // gpt/model_params/model_dim.h:12
 
 // AddLookupProduct for a batch of rows.  Token form: one new token per sequence, every sequence with its own state row
 // and KV cache (append + attention over the cache).  Prompt form: all tokens of a batch of fragments at once (one
-// prefill launch, one cache fill).  Owns the intermediate vectors (allocated once for maxRows rows).  11 or 12 launches
-// per call: the four projections are one product when QK, QV, K and V lie one after the other in memory, the
+// prefill launch, one cache fill).  Owns the intermediate vectors (allocated once for maxRows rows).  10 or 11 launches
+// per token call: the four projections are one product when QK, QV, K and V lie one after the other in memory, the
 // normalisations that follow them are one call, K-split products leave their parts for the consumer to add up, and the
 // combiner's AddScaled is done by the normalisation after it.  QDim == TTDim == 64 or 128; the feed-forward width is
 // reluDim = HeadCount * QDim (ReluMult 1 at QDim 128).
@@ -166,11 +166,14 @@ class TLayerComputer
     int32_t *Planes = nullptr; // int32 results of the matrix products: up to 16 planes with few rows, one otherwise
     void *Workspace = nullptr;
     int64_t WorkspaceBytes = 0;
+    int PendingPlanes = 0, PendingRows = 0; // a deferred state update: the contract product's parts in Planes
+    float PendingScale = 0;
 
     int MulForwardPlanes(int rows, const uint8_t *vec, int k, const int8_t *matr, int n, void *stream);
     void Projections(int rows, const int32_t *pos, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att, bool scalePlanes,
-                     const float *state, void *stream);
-    void AfterAttention(int rows, const TAttentionMatrices &att, float *state, void *stream);
+                     float *state, void *stream);
+    void AfterAttention(int rows, const TAttentionMatrices &att, bool kvDone, bool deferStateUpdate, float *state, void *stream);
+    void NormalizeState(int rows, float *state, void *stream);
     friend void ComputePrediction(TLayerComputer &, const TInferModel &, const std::vector<TAttentionVecHistory *> &, const int32_t *,
                                   const int32_t *, const float *, int64_t, float *, float *, int32_t *, void *);
 
@@ -184,8 +187,13 @@ class TLayerComputer
 
     // t: device int32 [seqCount], the new tokens' positions; ropeBuf: device table of FillRopeBuf with ropeLen rows;
     // state: device [seqCount][Dim] fp32, updated in place; the cache gets the new rows and its lengths grow by one.
+    // deferStateUpdate: leave the layer's last state update (contract's AddScaled) to the first normalisation of the next
+    // call on the same state rows, or to FlushState -- one launch less per layer; until then `state` lacks that update.
     void AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
-                          TAttentionVecHistory *pKVCache, float *state, void *stream);
+                          TAttentionVecHistory *pKVCache, float *state, void *stream, bool deferStateUpdate = false);
+    // Does a pending state update and returns NormalizeState(state) (device, int8 [rows][Dim]), which is what
+    // ComputePrediction multiplies with the final layer.
+    const uint8_t *FlushState(int rows, float *state, void *stream);
     // len tokens of the cache's sequences, concatenated (seqOffset: device int32 [seqCount + 1]); pos: device int32 [len],
     // each token's position in its sequence; spans (and optionally their summary and the launch-order hint) of
     // att.AttentionWidth as for tsattn_prefill; state: device [len][Dim]; the tokens' rows are appended to the cache.
