@@ -4,7 +4,7 @@
 // operation: the same float products, the sum of squares taken in index order, no fused multiply-adds, so the
 // bytes and scales are identical to a CPU evaluation in that order.
 //
-// A workgroup takes 32 consecutive (row, head) pairs.  The rotated values go to LDS (row pitch d+1 floats, so
+// A workgroup takes 32 (8 in a small launch) consecutive (row, head) pairs.  The rotated values go to LDS (row pitch d+1 floats, so
 // that 32 lanes walking 32 different pairs in step hit 32 different banks); then lane j of the first wave sums
 // pair j's squares one after the other, which keeps the summation order while 32 sums advance together; then
 // all threads convert and write the bytes out, sixteen per thread, consecutively.
@@ -15,23 +15,24 @@
 
 namespace tsattn {
 
-constexpr int PR_PAIRS = 32;
+constexpr int PR_PAIRS = 32;       // (row, head) pairs per workgroup
+constexpr int PR_PAIRS_FEW = 8;    // ... of a small launch: more workgroups, each with less to wait for
 
 // every float operation below is meant as written: no fused multiply-adds
 #pragma clang fp contract(off)
 
-template <int D, int DST, bool SRC_I32>
+template <int D, int DST, bool SRC_I32, int PAIRS>
 __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
 {
     constexpr int PITCH = D + 1;
-    __shared__ float vals[PR_PAIRS * PITCH];
-    __shared__ float mults[PR_PAIRS];
-    __shared__ int64_t s_row[PR_PAIRS];
-    __shared__ int s_head[PR_PAIRS], s_pos[PR_PAIRS];
+    __shared__ float vals[PAIRS * PITCH];
+    __shared__ float mults[PAIRS];
+    __shared__ int64_t s_row[PAIRS];
+    __shared__ int s_head[PAIRS], s_pos[PAIRS];
     const int tid = threadIdx.x;
-    const int64_t pair0 = (int64_t)blockIdx.x * PR_PAIRS;
+    const int64_t pair0 = (int64_t)blockIdx.x * PAIRS;
     const int64_t n_pairs = p.n_rows * p.n_heads;
-    const int n_here = (int)(n_pairs - pair0 < PR_PAIRS ? n_pairs - pair0 : PR_PAIRS);
+    const int n_here = (int)(n_pairs - pair0 < PAIRS ? n_pairs - pair0 : PAIRS);
 
     if (tid < n_here) {
         const int64_t pair = pair0 + tid;
@@ -46,7 +47,7 @@ __global__ __launch_bounds__(256) void rope_normalize_kernel(ProduceParams p)
     // ---- load + rotate: four (k, k+32) couples per thread and step, 16-byte loads; all loads of a thread are
     //      issued before the first is used ------------------------------------------------------------------
     constexpr int PER_PAIR = D / 8;
-    constexpr int STEPS = PR_PAIRS * PER_PAIR / 256;
+    constexpr int STEPS = (PAIRS * PER_PAIR + 255) / 256;
     v4f v0[STEPS], v1[STEPS], cs[STEPS], sn[STEPS];
 #pragma unroll
     for (int st = 0; st < STEPS; ++st) {
@@ -172,8 +173,16 @@ hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head
 {
     const int64_t n_pairs = p.n_rows * p.n_heads;
     if (n_pairs == 0) return hipSuccess;
-    dim3 grid((unsigned)((n_pairs + PR_PAIRS - 1) / PR_PAIRS)), block(256);
-#define TSATTN_PR(D_, DST_, I32_) hipLaunchKernelGGL((rope_normalize_kernel<D_, DST_, I32_>), grid, block, 0, st, p)
+    // a small launch (one token per sequence) is a chain of waits -- positions, rows, the ordered sums -- that more,
+    // smaller workgroups get through sooner; a large one is bound by memory and takes 32 pairs per workgroup
+    const bool few = n_pairs <= 4096;
+    const int per_wg = few ? PR_PAIRS_FEW : PR_PAIRS;
+    dim3 grid((unsigned)((n_pairs + per_wg - 1) / per_wg)), block(256);
+#define TSATTN_PR(D_, DST_, I32_)                                                                                   \
+    do {                                                                                                            \
+        if (few) hipLaunchKernelGGL((rope_normalize_kernel<D_, DST_, I32_, PR_PAIRS_FEW>), grid, block, 0, st, p);  \
+        else hipLaunchKernelGGL((rope_normalize_kernel<D_, DST_, I32_, PR_PAIRS>), grid, block, 0, st, p);          \
+    } while (0)
     if (head_dim == 128 && dst_dtype == TSATTN_I8 && !src_i32) TSATTN_PR(128, TSATTN_I8, false);
     else if (head_dim == 128 && dst_dtype == TSATTN_I8 && src_i32) TSATTN_PR(128, TSATTN_I8, true);
     else if (head_dim == 128 && dst_dtype == TSATTN_E4M3 && !src_i32) TSATTN_PR(128, TSATTN_E4M3, false);
