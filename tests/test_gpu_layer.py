@@ -162,3 +162,52 @@ def test_deferred_state_updates_give_the_same_bits(ctx):
     assert np.array_equal(a[0], b[0])
     for x, y in zip(a[1] + a[2] + a[3], b[1] + b[2] + b[3]):
         assert np.array_equal(x, y)
+
+
+@pytest.mark.parametrize("width,slope", [(64, 0.5), (10 ** 6, 0.0)])
+def test_prompt_form_equals_token_form_at_model_width(ctx, width, slope):
+    """At the 1.5B-style width (2048, 16 heads of 128): 32 sequences of 128 tokens through the prompt form of the layer
+    (products of 4096 rows: the large-tile kernels, the producer's 32-pair launches, one prefill launch, one cache
+    fill) and the same tokens one position at a time through the token form (few-row products, fused append +
+    attention + KVProduct): the same cache bytes and key scales, attention outputs within the prefill tolerance,
+    states equal up to flips of int8 roundings -- the comparison NCPUInfer::Check makes (cpu_infer.cpp:658-683)."""
+    from tests.common import assert_within_tolerance
+    from tscale_amd import AttentionContext
+    from tscale_amd.attention import add_lookup_product_prompt
+    H, d, dim, B, S = 16, 128, 2048, 32, 128
+    qsum, n = H * d, B * S
+    big = AttentionContext(0, max_seqs=B, max_heads=H, max_head_dim=d)
+    try:
+        g = torch.Generator(device="cuda"); g.manual_seed(width % 1000)
+        mat = lambda r, k: (torch.randn((r, k), device="cuda", generator=g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
+        layer = {"proj": mat(4 * qsum, dim), "combiner": mat(dim, qsum * 4), "expand": mat(qsum, dim), "contract": mat(dim, qsum),
+                 "qv_scale": 0.031, "combiner_scale": 0.027, "contract_scale": 0.035, "width": width, "slope": slope}
+        rope = torch.from_numpy(orc.fill_rope(d, S)).cuda()
+        state0 = torch.randn((n, dim), device="cuda", generator=g) * 2          # token (b, p) at row b * S + p
+        # prompt form
+        c1 = KVCache(big, capi.I8, B, H, S, d); c1.v_scale.fill_(VEC_SCALE)
+        seq_offset = torch.arange(0, n + 1, S, dtype=torch.int32, device="cuda")
+        pos = torch.arange(S, dtype=torch.int32, device="cuda").repeat(B)
+        st, fi = big.build_spans(seq_offset, n, min(width, S))
+        s1 = state0.clone()
+        v1 = add_lookup_product_prompt(big, layer, c1, seq_offset, pos, rope, s1, st, fi)
+        # token form: position p of every sequence at step p
+        c2 = KVCache(big, capi.I8, B, H, S, d); c2.v_scale.fill_(VEC_SCALE)
+        s2 = state0.view(B, S, dim).transpose(0, 1).contiguous()                  # [S, B, dim]
+        v2 = torch.empty((S, B, qsum), dtype=torch.float32, device="cuda")
+        keep = {}
+        for p_ in range(S):
+            t = torch.full((B,), p_, dtype=torch.int32, device="cuda")
+            v2[p_] = add_lookup_product(big, layer, c2, t, rope, s2[p_], scratch=keep)
+        torch.cuda.synchronize()
+        assert torch.equal(c1.cache_len, c2.cache_len) and int(c1.cache_len[0]) == S
+        assert torch.equal(c1.k, c2.k) and torch.equal(c1.v, c2.v) and torch.equal(c1.k_scale, c2.k_scale)
+        a_val = v1.view(B, S, qsum).transpose(0, 1).cpu().numpy().reshape(n, qsum)
+        assert_within_tolerance(a_val, v2.cpu().numpy().reshape(n, qsum), "attention output, prompt form against token form")
+        got = s1.view(B, S, dim).transpose(0, 1).cpu().numpy().astype(np.float64)
+        want = s2.cpu().numpy().astype(np.float64)
+        rms = np.sqrt((want ** 2).mean())
+        assert np.abs(got - want).max() / rms < 5e-2
+        assert np.sqrt(((got - want) ** 2).mean()) / rms < 5e-3
+    finally:
+        big.close()
