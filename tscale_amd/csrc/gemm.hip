@@ -42,10 +42,9 @@ __device__ inline void store_out(const GemmParams &p, int64_t m, int64_t n, int 
 }
 
 // ---- many rows --------------------------------------------------------------------------------------------------
-// Output tiles of GT_BM x 128, K in steps of 64 bytes through LDS (two buffers), four waves as 2 x 2, each wave
-// (GT_BM / 2) x 64 = MT x 2 MFMA tiles.  What limits an int8 product here is LDS bandwidth: one 32x32x32 MFMA takes 32
-// cycles and two KiB of operands, so operands have to be used several times from registers: MT = 4 reads 6 KiB per 8
-// MFMAs.
+// Products too small for the wide tiles below: output tiles of 64 MT x 128 (MT = 2 in use), K in steps of 64 bytes
+// through LDS (two buffers), four waves as 2 x 2, each wave 32 MT x 64 = MT x 2 MFMA tiles.  One 32x32x32 MFMA takes 32
+// cycles and two KiB of operands, so operands have to be used several times from registers.
 template <int MODE, int MT>
 __global__ __launch_bounds__(GT_THREADS, 2) void gemm_tiled_kernel(GemmParams p)
 {
@@ -173,108 +172,6 @@ __global__ __launch_bounds__(GT_THREADS, 2) void gemm_tiled_kernel(GemmParams p)
         }
 }
 
-// Tall tiles for large products: 256 x 128 outputs, K in steps of 128 bytes (a row's whole cache line per request),
-// one LDS buffer and one step of requests held in registers while the previous step is computed from LDS; waves of
-// 128 x 64.  K must be a multiple of 128.
-constexpr int GL_BK = 128, GL_PITCH = GL_BK + 16, GL_BM = 256;
-
-template <int MODE>
-__global__ __launch_bounds__(GT_THREADS, 2) void gemm_tall_kernel(GemmParams p)
-{
-    constexpr int MT = 4;
-    constexpr int A_CH = GL_BM * GL_BK / 16 / GT_THREADS, W_CH = GT_BN * GL_BK / 16 / GT_THREADS; // 8 and 4
-    __shared__ __attribute__((aligned(16))) uint8_t a_lds[GL_BM * GL_PITCH];
-    __shared__ __attribute__((aligned(16))) uint8_t w_lds[GT_BN * GL_PITCH];
-    const int tid = threadIdx.x;
-    const int lane = tid & (WAVE - 1);
-    const int wave = tid / WAVE;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int li = lane & 31, g = lane >> 5;
-
-    // 8 x 8 blocks of tiles per XCD where the shape allows (see gemm_tiled_kernel)
-    const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN, tiles_m = (p.m + GL_BM - 1) / GL_BM;
-    int64_t tile_m, tile_n;
-    if (tiles_n % 8 == 0 && tiles_m % 8 == 0 && ((tiles_n >> 3) * (tiles_m >> 3)) % 8 == 0) {
-        const int64_t x = blockIdx.x & 7, l = blockIdx.x >> 3;
-        const int64_t sb = (l >> 6) * 8 + x, within = l & 63;
-        const int64_t sb_per_row = tiles_n >> 3;
-        tile_m = (sb / sb_per_row) * 8 + (within >> 3);
-        tile_n = (sb % sb_per_row) * 8 + (within & 7);
-    } else {
-        tile_m = blockIdx.x / tiles_n;
-        tile_n = blockIdx.x % tiles_n;
-    }
-    const int64_t m0 = tile_m * GL_BM, n0 = tile_n * GT_BN;
-    const __amdgpu_buffer_rsrc_t ar = rows_rsrc(p.a + m0 * p.a_pitch, p.m - m0 < GL_BM ? p.m - m0 : GL_BM, p.a_pitch, p.k);
-    const __amdgpu_buffer_rsrc_t wr = rows_rsrc(p.w + n0 * p.w_pitch, p.n - n0 < GT_BN ? p.n - n0 : GT_BN, p.w_pitch, p.k);
-    int a_off[A_CH], w_off[W_CH], a_dst[A_CH], w_dst[W_CH];
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) {
-        const int ch = tid + i * GT_THREADS, r = ch >> 3, c = ch & 7; // eight lanes per row: its whole 128 bytes
-        a_off[i] = r * (int)p.a_pitch + c * 16;
-        a_dst[i] = r * GL_PITCH + c * 16;
-    }
-#pragma unroll
-    for (int i = 0; i < W_CH; ++i) {
-        const int ch = tid + i * GT_THREADS, r = ch >> 3, c = ch & 7;
-        w_off[i] = r * (int)p.w_pitch + c * 16;
-        w_dst[i] = r * GL_PITCH + c * 16;
-    }
-    v4i ra[A_CH], rw[W_CH];
-    auto load = [&](int kb) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < A_CH; ++i) ra[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, a_off[i], kb, 0));
-#pragma unroll
-        for (int i = 0; i < W_CH; ++i) rw[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, w_off[i], kb, 0));
-    };
-    auto stage = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < A_CH; ++i) *(v4i *)(a_lds + a_dst[i]) = ra[i];
-#pragma unroll
-        for (int i = 0; i < W_CH; ++i) *(v4i *)(w_lds + w_dst[i]) = rw[i];
-    };
-    v16i acc[MT][2];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = v16i{0};
-
-    const int n_steps = (int)(p.k / GL_BK);
-    const uint8_t *ab = a_lds + (wm * 128 + li) * GL_PITCH + 16 * g;
-    const uint8_t *wb = w_lds + (wn * 64 + li) * GL_PITCH + 16 * g;
-    load(0);
-    for (int s = 0; s < n_steps; ++s) {
-        stage();
-        load((s + 1) * GL_BK); // past K: zeros or other bytes of the tile, never computed with
-        __syncthreads();
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            v4i a[MT], w[2];
-#pragma unroll
-            for (int j = 0; j < 2; ++j) w[j] = *(const v4i *)(wb + j * 32 * GL_PITCH + 32 * ks);
-#pragma unroll
-            for (int i = 0; i < MT; ++i) a[i] = *(const v4i *)(ab + i * 32 * GL_PITCH + 32 * ks);
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], w[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads(); // everybody has read the step before it is overwritten
-    }
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t n = n0 + wn * 64 + j * 32 + li;
-            if (n >= p.n) continue;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
-                if (m < p.m) store_out<MODE>(p, m, n, acc[i][j][r]);
-            }
-        }
-}
-
 // Wide tiles for the largest products: 256 x 256 outputs by eight waves of 128 x 64, K in steps of 64 bytes, one
 // workgroup per compute unit; per MFMA cycle this moves a third less through LDS and the caches than 256 x 128 tiles.
 // Each SIMD holds two of the waves, one from each half of the workgroup, and the halves run half a step apart: while
@@ -392,18 +289,47 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
     if (half == 0) GW_BARRIER;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // nothing may still be on its way into LDS when the workgroup ends
 #undef GW_BARRIER
+    if constexpr (MODE == TSATTN_MM_ADD_SCALED) {
+        // state += sum * scale: the 32 old values of a block of rows are requested together, then updated and stored
+        // (element by element every store would have to be waited for before the next load, which it might overlap;
+        // with one workgroup per compute unit nothing else runs under those waits)
+#pragma clang fp contract(off)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i) {
+            float old[2][16];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t n = n0 + wn * 64 + j * 32 + li;
-            if (n >= p.n) continue;
+            for (int j = 0; j < 2; ++j) {
+                const int64_t n = n0 + wn * 64 + j * 32 + li;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
-                if (m < p.m) store_out<MODE>(p, m, n, acc[i][j][r]);
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                    old[j][r] = (n < p.n && m < p.m) ? ((const float *)p.out)[m * p.out_pitch + n] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int64_t n = n0 + wn * 64 + j * 32 + li;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                    if (n < p.n && m < p.m) ((float *)p.out)[m * p.out_pitch + n] = old[j][r] + (float)acc[i][j][r] * p.scale;
+                }
             }
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int64_t n = n0 + wn * 64 + j * 32 + li;
+                if (n >= p.n) continue;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                    if (m < p.m) store_out<MODE>(p, m, n, acc[i][j][r]);
+                }
+            }
+    }
 }
 
 // ---- few rows ---------------------------------------------------------------------------------------------------
@@ -525,22 +451,11 @@ template <int MODE>
 void launch_mode(const GemmParams &p, hipStream_t st)
 {
     if (p.m > 32 * GS_MB) {
-        // tall output tiles when there are enough rows to fill the chip with them
+        // wide tiles when there are two rounds of them for every compute unit, 128 x 128 tiles otherwise
         const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN;
-        // wide tiles when there are two rounds of them for every compute unit
         const int64_t wide = ((p.m + GW_BM - 1) / GW_BM) * ((p.n + GW_BN - 1) / GW_BN);
-        // (not for the read-modify-write output: with one workgroup per compute unit nothing runs under a tile's
-        // epilogue, and that one moves eight bytes per output)
-        if (wide >= 512 && p.k % GW_BK == 0 && MODE != TSATTN_MM_ADD_SCALED) {
-            hipLaunchKernelGGL((gemm_wide_kernel<MODE>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, p);
-            return;
-        }
-        if (((p.m + 255) / 256) * tiles_n >= 1024) {
-            if (p.k % GL_BK == 0) hipLaunchKernelGGL((gemm_tall_kernel<MODE>), dim3((unsigned)(((p.m + 255) / 256) * tiles_n)), dim3(GT_THREADS), 0, st, p);
-            else hipLaunchKernelGGL((gemm_tiled_kernel<MODE, 4>), dim3((unsigned)(((p.m + 255) / 256) * tiles_n)), dim3(GT_THREADS), 0, st, p);
-        } else {
-            hipLaunchKernelGGL((gemm_tiled_kernel<MODE, 2>), dim3((unsigned)(((p.m + 127) / 128) * tiles_n)), dim3(GT_THREADS), 0, st, p);
-        }
+        if (wide >= 512) hipLaunchKernelGGL((gemm_wide_kernel<MODE>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, p);
+        else hipLaunchKernelGGL((gemm_tiled_kernel<MODE, 2>), dim3((unsigned)(((p.m + 127) / 128) * tiles_n)), dim3(GT_THREADS), 0, st, p);
         return;
     }
     hipLaunchKernelGGL((gemm_skinny_kernel<MODE>), dim3((unsigned)((p.n + GS_BN - 1) / GS_BN), 1), dim3(GS_THREADS), 0, st, p);
