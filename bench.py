@@ -31,7 +31,7 @@ PEAK_HBM_GBPS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, scaled
 # by what the same counters read for a copy kernel of known size).  None until measured; the numbers
 # and commands are in profiles/.
-MEASURED_TRAFFIC = {"prefill_c2": 71.4e6, "decode_c3": 1113.2e6}  # bytes per launch (profiles/*.md)
+MEASURED_TRAFFIC = {"prefill_c2": 71.4e6, "decode_c3": 1108.0e6}  # bytes per launch (profiles/*.md)
 
 
 def pairs(S, W):

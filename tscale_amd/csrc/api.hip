@@ -178,9 +178,11 @@ int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
     int splits = a->n_splits;
     if (splits < 0 || splits > h->max_splits) return fail(TSATTN_ERR_SCRATCH, "tsattn_decode: n_splits %d exceeds the handle's %d", splits, h->max_splits);
     if (splits == 0) {
-        // enough workgroups to fill 256 CUs several times over, but at least 512 cache rows per split
+        // One workgroup streams its rows fast enough that one or two per compute unit reach the memory's rate, and every
+        // split beyond that only adds to the merge: about 384 workgroups in all (measured best at 4096 rows: 1 split from
+        // 256 (sequence, head) pairs up, 4 at 128, 8 at 32 and below), and at least 512 cache rows per split
         const int64_t pairs = (int64_t)a->n_seqs * a->n_heads;
-        int64_t want = (4096 + pairs - 1) / pairs;
+        int64_t want = 384 / pairs;
         int64_t rows = a->max_len;   // rows one query can see
         if (a->window < rows) rows = a->window > 0 ? a->window : 1;
         int64_t by_len = (rows + 511) / 512;
