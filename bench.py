@@ -474,7 +474,8 @@ def bench_generate_model(ctx, steps):
 
 def bench_prompt_pass(ctx, steps):
     """The prompt of the same configuration through the same 24 layers in batch form (add_lookup_product_prompt):
-    32 x 2048 tokens, per layer one prefill attention launch, one cache fill, seven matrix products in four calls."""
+    32 x 2048 tokens, per layer one prefill attention launch, one cache fill, seven matrix products in four calls, each
+    with the normalisation that follows it as its epilogue."""
     import torch
     from tscale_amd.attention import add_lookup_product_prompt
     m = Int8Layers(ctx, cache_len=0, seed=1313 + 10)
@@ -488,11 +489,12 @@ def bench_prompt_pass(ctx, steps):
     state = torch.empty_like(state0)
     def run():
         state.copy_(state0)
+        norm = None
         for layer, c in zip(m.layers, m.caches):
             c.cache_len.zero_()
             w = layer["width"]
-            add_lookup_product_prompt(ctx, layer, c, off, pos, m.rope, state, *spans[w], span_tiles=tiles[w],
-                                      causal_period=m.prompt if w >= m.prompt else 0)
+            _, norm = add_lookup_product_prompt(ctx, layer, c, off, pos, m.rope, state, *spans[w], span_tiles=tiles[w],
+                                                causal_period=m.prompt if w >= m.prompt else 0, norm=norm, want_norm=True)
     ms = gpu_time_ms(run, 2, 1)
     assert bool(torch.isfinite(state).all()) and int(m.caches[0].cache_len[0]) == m.prompt
     att_flops = sum(prefill_flops(B, m.prompt, H, d, w) for w, _ in m.sched)

@@ -310,6 +310,15 @@ typedef struct tsattn_matmul_args {
     void *workspace;
     int64_t workspace_bytes;
     int *planes_out;           /* TSATTN_MM_I32_PLANES: host int that receives the number of planes */
+    const struct tsattn_produce_args *epilogue; /* optional, TSATTN_MM_I32_PLANES only (host pointer, read during the call):
+                                  tsattn_rope_normalize_rows applied to the product, as that call would be afterwards with
+                                  src = out (its src, src_dtype, src_pitch, src_planes, src_plane_stride, n_rows and n_heads
+                                  are taken from the product: n_heads = n / head_dim, which must divide n).  This is the
+                                  reference's projection with its normalising epilogue (TStoreRowTileNormalizeRope,
+                                  gpt/compute/gpt_rope.cuh:4-66, lib/cuda/cuda_matmul.cuh:146-204).  Large products with an
+                                  int8 result do it in the product's own kernel and never write the int32 sums; otherwise
+                                  the library makes the two launches.  Either way `out` is scratch: what it holds after the
+                                  call is unspecified. */
 } tsattn_matmul_args;
 
 int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *stream);

@@ -397,9 +397,21 @@ static int RunPromptLayerCase(int width, float slope, int headDim)
                                        &cpu.Len[b], maxLen, &wantVal[(size_t)row * qsum], 4);
             }
         }
+        // (with the state update "deferred": for this many rows the last product does it and normalises the new state)
         layer.AddLookupProductPrompt(len, seqOffsetDev, posDev, ropeDev, maxLen, data.Att, spanStartDev, spanFinishDev, nullptr, 0, &cache, stateDev,
-                                     nullptr);
+                                     nullptr, true);
+        const uint8_t *normDev = layer.FlushState(len, stateDev, nullptr);
         HIP_OK(hipDeviceSynchronize());
+        {
+            std::vector<uint8_t> normGpu((size_t)len * dim), normWant(dim);
+            std::vector<float> stateGpu((size_t)len * dim), tileScale(dim / STATE_NORM_TILE);
+            HIP_OK(hipMemcpy(normGpu.data(), normDev, normGpu.size(), hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(stateGpu.data(), stateDev, stateGpu.size() * 4, hipMemcpyDeviceToHost));
+            for (int r = 0; r < len; ++r) {
+                tso_normalize_heads(TSO_I8, &stateGpu[(size_t)r * dim], dim, dim / STATE_NORM_TILE, VEC_SCALE, normWant.data(), tileScale.data());
+                if (memcmp(normWant.data(), &normGpu[(size_t)r * dim], dim)) { printf("  NormalizeState of row %d differs\n", r); ++fails; break; }
+            }
+        }
         std::vector<float> got(state.size()), gotVal(wantVal.size()), ksg(cpu.KScale.size());
         std::vector<uint8_t> kg(cpu.K.size()), vg(cpu.V.size());
         std::vector<int32_t> lenGpu(B);

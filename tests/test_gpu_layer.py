@@ -211,3 +211,44 @@ def test_prompt_form_equals_token_form_at_model_width(ctx, width, slope):
         assert np.sqrt(((got - want) ** 2).mean()) / rms < 5e-3
     finally:
         big.close()
+
+
+def test_chained_prompt_layers_give_the_same_bits(ctx):
+    """Two layers over a prompt of 4096 tokens (products large enough to normalise their own tiles): handing the second
+    layer the normalised state the first layer's last product made gives the same bits as normalising afresh."""
+    from tscale_amd import AttentionContext
+    from tscale_amd.attention import add_lookup_product_prompt
+    H, d, dim, B, S = 4, 128, 1024, 8, 512
+    qsum, n = H * d, B * S
+    big = AttentionContext(0, max_seqs=B, max_heads=H, max_head_dim=d)
+    try:
+        g = torch.Generator(device="cuda"); g.manual_seed(5)
+        mat = lambda r, k: (torch.randn((r, k), device="cuda", generator=g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
+        layers = [{"proj": mat(4 * qsum, dim), "combiner": mat(dim, qsum * 4), "expand": mat(qsum, dim), "contract": mat(dim, qsum),
+                   "qv_scale": 0.031, "combiner_scale": 0.027, "contract_scale": 0.035, "width": w, "slope": sl} for w, sl in ((64, 0.5), (10 ** 6, 0.0))]
+        rope = torch.from_numpy(orc.fill_rope(d, S)).cuda()
+        state0 = torch.randn((n, dim), device="cuda", generator=g) * 2
+        seq_offset = torch.arange(0, n + 1, S, dtype=torch.int32, device="cuda")
+        pos = torch.arange(S, dtype=torch.int32, device="cuda").repeat(B)
+        results = []
+        for chained in (False, True):
+            state = state0.clone()
+            caches = [KVCache(big, capi.I8, B, H, S, d) for _ in layers]
+            norm = None
+            for layer, c in zip(layers, caches):
+                c.v_scale.fill_(VEC_SCALE)
+                st, fi = big.build_spans(seq_offset, n, min(layer["width"], S))
+                if chained:
+                    _, norm = add_lookup_product_prompt(big, layer, c, seq_offset, pos, rope, state, st, fi, norm=norm, want_norm=True)
+                else:
+                    add_lookup_product_prompt(big, layer, c, seq_offset, pos, rope, state, st, fi)
+            torch.cuda.synchronize()
+            if chained:
+                want_norm, _ = big.rope_normalize_rows(state, dim // 128, capi.I8)
+                assert torch.equal(norm, want_norm)
+            results.append((state, [c.k for c in caches], [c.k_scale for c in caches]))
+        assert torch.equal(results[0][0], results[1][0])
+        for x, y in zip(results[0][1] + results[0][2], results[1][1] + results[1][2]):
+            assert torch.equal(x, y)
+    finally:
+        big.close()

@@ -107,3 +107,37 @@ def test_matmul_planes_sum_to_the_product(ctx, m, n, k):
     if (m, n, k) == (32, 2048, 8192):
         assert planes.shape[0] > 1, "this shape is meant to split K"
     assert np.array_equal(planes.sum(dim=0, dtype=torch.int32).cpu().numpy(), orc.matmul_i8(a, w))
+
+
+@pytest.mark.parametrize("m,n,k,d,variant", [
+    (4096, 8192, 256, 128, "rope"), (8192, 4096, 128, 128, "resid"), (4100, 8192, 192, 64, "rope"), (16384, 2048, 64, 128, "relu"),
+    (8000, 4224, 128, 64, "resid"),                                       # the product's kernel normalises its own tiles
+    (300, 512, 256, 128, "rope"), (32, 2048, 1024, 128, "resid"), (5, 256, 128, 64, "relu"),   # two launches
+])
+def test_matmul_with_the_producer_as_its_epilogue(ctx, m, n, k, d, variant):
+    """tsattn_matmul_i8 with an epilogue is the product followed by tsattn_rope_normalize_rows on it: the same bytes, the
+    same scales, the same updated residual, whichever way the library does it."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    H = n // d
+    a, w = dev(rand_i8(rng, (m, k)).view(np.uint8)), dev(rand_i8(rng, (n, k)).view(np.uint8))
+    kw = {}
+    if variant == "rope":
+        rope = dev(orc.fill_rope(d, 64))
+        pos = dev(rng.integers(-1, 70, m).astype(np.int32))              # out-of-table positions are clamped
+        kw = dict(pos=pos, rope=rope, scale_mult=0.37, rope_heads=max(1, H // 2), scale_heads=(H // 4, max(1, H // 4)))
+    elif variant == "relu":
+        kw = dict(relu=True, row_major_scale=True)
+    resid0 = rng.standard_normal((m, n)).astype(np.float32)
+    if variant == "resid":
+        r1, r2 = dev(resid0), dev(resid0)
+        kw = dict(resid=r1, resid_scale=0.011)
+    got_q, got_s = ctx.matmul_normalize(a, w, H, capi.I8, **kw)
+    sums = ctx.matmul_i8(a, w, mode=capi.MM_I32_PLANES)
+    if variant == "resid":
+        kw = dict(resid=r2, resid_scale=0.011)
+    want_q, want_s = ctx.rope_normalize_rows(sums, H, capi.I8, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(got_q, want_q)
+    assert torch.equal(got_s, want_s)
+    if variant == "resid":
+        assert torch.equal(r1, r2)

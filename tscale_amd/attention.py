@@ -91,6 +91,30 @@ class AttentionContext:
         self.lib.tsattn_fill_rope_table(head_dim, max_len, ctypes.c_void_p(host.data_ptr()))
         return host.to(self.device)
 
+    def _produce_args(self, n_rows, hd, device, n_heads, dtype, pos, rope, rotate_dir, vec_scale, scale_mult, row_major_scale, relu,
+                      rope_heads, scale_heads, resid, resid_scale):
+        """The producer's arguments (without its source) and its two results."""
+        q = torch.empty((n_rows, hd), dtype=torch.uint8, device=device)
+        n_scale = n_heads if scale_heads is None else scale_heads[1]
+        scale = torch.empty((n_rows, n_scale) if row_major_scale else (n_scale, n_rows), dtype=torch.float32, device=device)
+        a = capi.ProduceArgs()
+        a.dst_dtype = dtype
+        a.n_rows, a.n_heads, a.head_dim = n_rows, n_heads, hd // n_heads
+        a.pos, a.rope = _ptr(pos), _ptr(rope)
+        a.rope_len = 0 if rope is None else rope.shape[0]
+        a.rope_heads = int(rope_heads)
+        a.rotate_dir, a.vec_scale, a.scale_mult = float(rotate_dir), float(vec_scale), float(scale_mult)
+        a.dst, a.dst_pitch = _ptr(q), hd
+        a.scale, a.scale_pitch = _ptr(scale), (1 if row_major_scale else n_rows)
+        a.scale_row_stride = n_scale if row_major_scale else 1
+        if scale_heads is not None:
+            a.scale_head_begin, a.scale_head_count = int(scale_heads[0]), int(scale_heads[1])
+        a.relu = int(bool(relu))
+        if resid is not None:
+            assert resid.dtype == torch.float32 and resid.shape == (n_rows, hd) and resid.stride(1) == 1
+            a.resid, a.resid_pitch, a.resid_scale = _ptr(resid), resid.stride(0), float(resid_scale)
+        return a, q, scale
+
     def rope_normalize_rows(self, x, n_heads, dtype, pos=None, rope=None, rotate_dir=1.0, vec_scale=1.0 / 24,
                             scale_mult=1.0, row_major_scale=False, relu=False, rope_heads=0, scale_heads=None,
                             resid=None, resid_scale=1.0):
@@ -106,29 +130,42 @@ class AttentionContext:
             assert x.dtype == torch.int32
             planes = x.shape[0]
         n_rows, hd = x.shape[-2:]
-        q = torch.empty((n_rows, hd), dtype=torch.uint8, device=x.device)
-        n_scale = n_heads if scale_heads is None else scale_heads[1]
-        scale = torch.empty((n_rows, n_scale) if row_major_scale else (n_scale, n_rows), dtype=torch.float32, device=x.device)
-        a = capi.ProduceArgs()
+        a, q, scale = self._produce_args(n_rows, hd, x.device, n_heads, dtype, pos, rope, rotate_dir, vec_scale, scale_mult, row_major_scale,
+                                         relu, rope_heads, scale_heads, resid, resid_scale)
         a.src_dtype = capi.SRC_F32 if x.dtype == torch.float32 else capi.SRC_I32
-        a.dst_dtype = dtype
-        a.n_rows, a.n_heads, a.head_dim = n_rows, n_heads, hd // n_heads
         a.src, a.src_pitch = _ptr(x), hd
         a.src_planes, a.src_plane_stride = planes, n_rows * hd
-        a.pos, a.rope = _ptr(pos), _ptr(rope)
-        a.rope_len = 0 if rope is None else rope.shape[0]
-        a.rope_heads = int(rope_heads)
-        a.rotate_dir, a.vec_scale, a.scale_mult = float(rotate_dir), float(vec_scale), float(scale_mult)
-        a.dst, a.dst_pitch = _ptr(q), hd
-        a.scale, a.scale_pitch = _ptr(scale), (1 if row_major_scale else n_rows)
-        a.scale_row_stride = n_scale if row_major_scale else 1
-        if scale_heads is not None:
-            a.scale_head_begin, a.scale_head_count = int(scale_heads[0]), int(scale_heads[1])
-        a.relu = int(bool(relu))
-        if resid is not None:
-            assert resid.dtype == torch.float32 and resid.shape == (n_rows, hd) and resid.stride(1) == 1
-            a.resid, a.resid_pitch, a.resid_scale = _ptr(resid), resid.stride(0), float(resid_scale)
         capi.check(self.lib.tsattn_rope_normalize_rows(self.handle, ctypes.byref(a), _stream_ptr()))
+        return q, scale
+
+    def matmul_normalize(self, a, w, n_heads, dtype, scratch=None, **producer):
+        """MulForward followed by rope_normalize_rows on its int32 result, as one library call: the projection with its
+        normalising epilogue.  Large products with an int8 result never write the int32 sums (the product's kernel
+        normalises its own tiles).  a uint8 [m, k], w uint8 [n, k]; scratch: int32 room for 16 * m * n sums (m <= 128) or
+        m * n, made here if not given; producer: rope_normalize_rows' keyword arguments.  Returns (uint8 [m, n], scale)
+        like rope_normalize_rows."""
+        m, k = a.shape
+        n = w.shape[0]
+        assert w.shape[1] == k and a.stride(1) == 1 and w.stride(1) == 1
+        room = (16 if m <= 128 else 1) * m * n
+        if scratch is None:
+            scratch = torch.empty(room, dtype=torch.int32, device=a.device)
+        assert scratch.is_contiguous() and scratch.dtype == torch.int32 and scratch.numel() >= room
+        kw = dict(pos=None, rope=None, rotate_dir=1.0, vec_scale=1.0 / 24, scale_mult=1.0, row_major_scale=False, relu=False, rope_heads=0,
+                  scale_heads=None, resid=None, resid_scale=1.0)
+        kw.update(producer)
+        ep, q, scale = self._produce_args(m, n, a.device, n_heads, dtype, kw["pos"], kw["rope"], kw["rotate_dir"], kw["vec_scale"], kw["scale_mult"],
+                                          kw["row_major_scale"], kw["relu"], kw["rope_heads"], kw["scale_heads"], kw["resid"], kw["resid_scale"])
+        args = capi.MatmulArgs()
+        args.m, args.n, args.k = m, n, k
+        args.a, args.a_pitch = _ptr(a), a.stride(0)
+        args.w, args.w_pitch = _ptr(w), w.stride(0)
+        args.mode, args.scale = capi.MM_I32_PLANES, 1.0
+        args.out, args.out_pitch = _ptr(scratch), n
+        planes = ctypes.c_int(0)
+        args.planes_out = ctypes.pointer(planes)
+        args.epilogue = ctypes.cast(ctypes.pointer(ep), ctypes.c_void_p)
+        capi.check(self.lib.tsattn_matmul_i8(self.handle, ctypes.byref(args), _stream_ptr()))
         return q, scale
 
     def kv_product(self, k, value, n_heads, rep=4, mult=1.0):
@@ -383,39 +420,44 @@ def flush_state(ctx, pending, state):
 
 
 def add_lookup_product_prompt(ctx, layer, cache, seq_offset, pos, rope, state, span_start, span_finish, span_tiles=None,
-                              causal_period=0):
+                              causal_period=0, norm=None, want_norm=False):
     """The same layer for a whole batch of prompt tokens at once (sequences concatenated, seq_offset int32 [B+1], pos
     int32 [n_tokens] = each token's position in its sequence): every token's attention over the earlier tokens of its
     sequence is one tsattn_prefill launch, and the tokens' key and value rows go into the cache in one
     tsattn_cache_fill.  Token by token through add_lookup_product gives the same cache and the same states (a token's
     layer input does not depend on other tokens' outputs of the same layer).  state: f32 [n_tokens, dim], updated in
-    place; the spans are those of the layer's width (build_spans).  Returns the attention output."""
+    place; the spans are those of the layer's width (build_spans).  Returns the attention output.
+    norm: NormalizeState(state) where the caller has it (the previous layer's second result); want_norm=True returns
+    (attention output, NormalizeState(new state)), which the layer's last product then makes as its epilogue."""
     n, dim = state.shape
     H, d = cache.n_heads, cache.head_dim
     qsum = H * d
     groups = dim // STATE_NORM_TILE
     f32 = np.float32
-    norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
-    proj = ctx.matmul_i8(norm, layer["proj"], mode=capi.MM_I32_PLANES)
+    if norm is None:
+        norm, _ = ctx.rope_normalize_rows(state, groups, capi.I8)
+    # every product with its normalisation as epilogue (large products never write their int32 sums); one scratch
+    # buffer for whichever falls back to two launches
     key_mult = float(f32(layer["qv_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(dim))))
-    q4, qv_scale = ctx.rope_normalize_rows(proj, 4 * H, capi.I8, pos=pos, rope=rope, scale_mult=key_mult,
-                                           rope_heads=2 * H, scale_heads=(H, H))      # scales as [head][token] planes
-    del proj
+    room = torch.empty((16 if n <= 128 else 1) * n * max(4 * qsum, dim), dtype=torch.int32, device=state.device)
+    q4, qv_scale = ctx.matmul_normalize(norm, layer["proj"], 4 * H, capi.I8, room, pos=pos, rope=rope, scale_mult=key_mult,
+                                        rope_heads=2 * H, scale_heads=(H, H))      # scales as [head][token] planes
     qk, qv, k, v = q4[:, :qsum], q4[:, qsum:2 * qsum], q4[:, 2 * qsum:3 * qsum], q4[:, 3 * qsum:]
     val = ctx.compute_val_lookup(capi.I8, H, qk, qv, v, VEC_SCALE, qv_scale, VEC_SCALE, span_start, span_finish, layer["slope"],
                                  span_tiles=span_tiles, causal_period=causal_period)
     cache.fill_from_prefill(seq_offset, qv, qv_scale, v)       # value scales: the cache's constant VEC_SCALE
     kv = ctx.kv_product(k, val, H, COMBINER_REP)
-    delta = ctx.matmul_i8(kv, layer["combiner"], mode=capi.MM_I32_PLANES)
-    norm, _ = ctx.rope_normalize_rows(delta, groups, capi.I8, resid=state,
-                                      resid_scale=float(f32(layer["combiner_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(qsum * COMBINER_REP)))))
-    del delta, kv
-    relu_src = ctx.matmul_i8(norm, layer["expand"], mode=capi.MM_I32_PLANES)
-    relu, _ = ctx.rope_normalize_rows(relu_src, H, capi.I8, relu=True)
-    relu_dim = relu_src.shape[-1]
-    del relu_src
-    ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state,
-                  scale=float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim)))))
+    norm, _ = ctx.matmul_normalize(kv, layer["combiner"], groups, capi.I8, room, resid=state,
+                                   resid_scale=float(f32(layer["combiner_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(qsum * COMBINER_REP)))))
+    del kv
+    relu, _ = ctx.matmul_normalize(norm, layer["expand"], H, capi.I8, room, relu=True)
+    relu_dim = relu.shape[-1]
+    contract_scale = float(f32(layer["contract_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(relu_dim))))
+    if want_norm:   # state += product * scale, and the updated state normalised for whoever comes next
+        norm_next, _ = ctx.matmul_normalize(relu, layer["contract"], groups, capi.I8, room, resid=state, resid_scale=contract_scale)
+        return val, norm_next
+    del room
+    ctx.matmul_i8(relu, layer["contract"], mode=capi.MM_ADD_SCALED, out=state, scale=contract_scale)
     return val
 
 

@@ -90,6 +90,7 @@ class MatmulArgs(_c.Structure):
         ("m", _c.c_int64), ("n", _c.c_int64), ("k", _c.c_int64), ("a", _c.c_void_p), ("a_pitch", _c.c_int64),
         ("w", _c.c_void_p), ("w_pitch", _c.c_int64), ("mode", _c.c_int), ("scale", _c.c_float), ("out", _c.c_void_p),
         ("out_pitch", _c.c_int64), ("workspace", _c.c_void_p), ("workspace_bytes", _c.c_int64), ("planes_out", _c.POINTER(_c.c_int)),
+        ("epilogue", _c.c_void_p),
     ]
 
 

@@ -298,35 +298,37 @@ int tsattn_cache_fill(tsattn_handle_t h, const tsattn_fill_args *a, void *stream
     return TSATTN_OK;
 }
 
-int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, void *stream)
+// Checks a producer call's arguments and translates them; `who` names the entry point in messages.  Returns TSATTN_OK
+// with *empty set when there are no rows.
+static int fill_produce(const tsattn_produce_args *a, const char *who, tsattn::ProduceParams *out, bool *empty)
 {
-    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: null argument");
+    *empty = false;
     if (!dtype_ok(a->dst_dtype) || (a->src_dtype != TSATTN_SRC_F32 && a->src_dtype != TSATTN_SRC_I32))
-        return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_rope_normalize_rows: dtypes %d -> %d", a->src_dtype, a->dst_dtype);
-    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_rope_normalize_rows: head_dim %d (64 or 128 supported)", a->head_dim);
-    if (a->n_rows < 0 || a->n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: negative size");
-    if (a->n_rows == 0) return TSATTN_OK;
-    if (!a->src || !a->dst) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: null data pointer");
-    if (a->pos && (!a->rope || a->rope_len <= 0)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: positions given without a rope table");
+        return fail(TSATTN_ERR_UNSUPPORTED, "%s: dtypes %d -> %d", who, a->src_dtype, a->dst_dtype);
+    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "%s: head_dim %d (64 or 128 supported)", who, a->head_dim);
+    if (a->n_rows < 0 || a->n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "%s: negative size", who);
+    if (a->n_rows == 0) { *empty = true; return TSATTN_OK; }
+    if (!a->src || !a->dst) return fail(TSATTN_ERR_BAD_ARG, "%s: null data pointer", who);
+    if (a->pos && (!a->rope || a->rope_len <= 0)) return fail(TSATTN_ERR_BAD_ARG, "%s: positions given without a rope table", who);
     const int64_t row = (int64_t)a->n_heads * a->head_dim;
     if (a->src_pitch < row || a->dst_pitch < row || a->dst_pitch % 16 || a->src_pitch % 4 || !aligned16(a->dst) || !aligned16(a->src) ||
         (a->rope && !aligned16(a->rope)))
-        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: pitches must cover a row; src, dst and rope 16-byte aligned, pitches multiples of 16 bytes");
+        return fail(TSATTN_ERR_BAD_ARG, "%s: pitches must cover a row; src, dst and rope 16-byte aligned, pitches multiples of 16 bytes", who);
     const int64_t row_stride = a->scale_row_stride ? a->scale_row_stride : 1;
     if (a->scale_head_count < 0 || a->scale_head_begin < 0 || a->scale_head_begin + a->scale_head_count > a->n_heads)
-        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale head range outside the heads");
+        return fail(TSATTN_ERR_BAD_ARG, "%s: scale head range outside the heads", who);
     const int scale_heads = a->scale_head_count > 0 ? a->scale_head_count : a->n_heads;
     if (a->scale && (row_stride < 0 || a->scale_pitch <= 0 ||
                      !((row_stride == 1 && a->scale_pitch >= a->n_rows) || (a->scale_pitch == 1 && row_stride >= scale_heads))))
-        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: scale layout must be [heads][scale_pitch >= n_rows] or [n_rows][scale_row_stride >= heads]");
+        return fail(TSATTN_ERR_BAD_ARG, "%s: scale layout must be [heads][scale_pitch >= n_rows] or [n_rows][scale_row_stride >= heads]", who);
     if (a->src_planes < 0 || a->src_planes > 16 || (a->src_planes > 1 && (a->src_dtype != TSATTN_SRC_I32 || a->src_plane_stride < a->n_rows * a->src_pitch ||
                                                                            a->src_plane_stride % 4)))
-        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: up to 16 int32 source planes, at least n_rows * src_pitch elements apart, 16-byte aligned");
-    if (a->rope_heads < 0 || a->rope_heads > a->n_heads) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: rope_heads outside the heads");
+        return fail(TSATTN_ERR_BAD_ARG, "%s: up to 16 int32 source planes, at least n_rows * src_pitch elements apart, 16-byte aligned", who);
+    if (a->rope_heads < 0 || a->rope_heads > a->n_heads) return fail(TSATTN_ERR_BAD_ARG, "%s: rope_heads outside the heads", who);
     if (a->resid && (a->resid_pitch < row || a->resid_pitch % 4 || !aligned16(a->resid)))
-        return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: resid must be 16-byte aligned with a pitch that covers a row");
-    if (a->relu && a->dst_dtype != TSATTN_I8) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_rope_normalize_rows: relu with an int8 result only");
-    tsattn::ProduceParams p;
+        return fail(TSATTN_ERR_BAD_ARG, "%s: resid must be 16-byte aligned with a pitch that covers a row", who);
+    if (a->relu && a->dst_dtype != TSATTN_I8) return fail(TSATTN_ERR_UNSUPPORTED, "%s: relu with an int8 result only", who);
+    tsattn::ProduceParams &p = *out;
     p.src = a->src; p.src_pitch = a->src_pitch; p.n_rows = a->n_rows; p.n_heads = a->n_heads;
     p.pos = a->pos; p.rope = a->rope; p.rope_len = a->rope_len;
     p.rotate_dir = a->rotate_dir; p.vec_scale = a->vec_scale; p.scale_mult = a->scale_mult;
@@ -336,6 +338,16 @@ int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, 
     p.rope_heads = a->rope_heads > 0 ? a->rope_heads : a->n_heads;
     p.scale_head_begin = a->scale_head_count > 0 ? a->scale_head_begin : 0; p.scale_head_count = scale_heads;
     p.resid = a->resid; p.resid_pitch = a->resid_pitch; p.resid_scale = a->resid_scale;
+    return TSATTN_OK;
+}
+
+int tsattn_rope_normalize_rows(tsattn_handle_t h, const tsattn_produce_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_rope_normalize_rows: null argument");
+    tsattn::ProduceParams p;
+    bool empty;
+    const int rc = fill_produce(a, "tsattn_rope_normalize_rows", &p, &empty);
+    if (rc != TSATTN_OK || empty) return rc;
     hipError_t e = tsattn::launch_rope_normalize(p, a->dst_dtype, a->head_dim, a->src_dtype == TSATTN_SRC_I32, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "rope normalize launch");
     return TSATTN_OK;
@@ -380,7 +392,19 @@ int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *strea
         !aligned16(a->w) || (uintptr_t)a->out % 4)
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: pitches must cover a row; a, w and their pitches multiples of 16 bytes");
     if (a->a_pitch > (1 << 24) || a->w_pitch > (1 << 24)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: row pitch above 16 MiB");
-    tsattn::GemmParams p;
+    tsattn::GemmParams p = {};
+    if (a->epilogue) {
+        // the producer on the int32 result: its source is the product
+        if (a->mode != TSATTN_MM_I32_PLANES) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: an epilogue goes with the planes mode");
+        tsattn_produce_args e = *a->epilogue;
+        if (!head_dim_ok(e.head_dim) || a->n % e.head_dim) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: n %lld is not a whole number of the epilogue's heads", (long long)a->n);
+        e.src_dtype = TSATTN_SRC_I32; e.src = a->out; e.src_pitch = a->n; e.n_rows = a->m; e.n_heads = (int)(a->n / e.head_dim);
+        e.src_planes = 1; e.src_plane_stride = 0;
+        bool empty;
+        const int rc = fill_produce(&e, "tsattn_matmul_i8 (epilogue)", &p.ep, &empty);
+        if (rc != TSATTN_OK) return rc;
+        p.ep_head_dim = e.head_dim; p.ep_dst_dtype = e.dst_dtype;
+    }
     p.a = (const uint8_t *)a->a; p.w = (const uint8_t *)a->w; p.a_pitch = a->a_pitch; p.w_pitch = a->w_pitch;
     p.m = a->m; p.n = a->n; p.k = a->k; p.mode = a->mode; p.scale = a->scale; p.out = a->out; p.out_pitch = a->out_pitch;
     const bool ws_ok = a->workspace && a->workspace_bytes > 0 && aligned16(a->workspace);

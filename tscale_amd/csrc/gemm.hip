@@ -186,7 +186,7 @@ constexpr int GW_THREADS = 512, GW_BM = 256, GW_BN = 256, GW_BK = 64, GW_NBUF = 
 constexpr int GW_BUF = (GW_BM + GW_BN) * GW_BK;
 constexpr int GW_LDS_BYTES = GW_NBUF * GW_BUF;
 
-template <int MODE>
+template <int MODE, int EP_D>
 __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t gw_lds[];
@@ -289,7 +289,144 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
     if (half == 0) GW_BARRIER;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // nothing may still be on its way into LDS when the workgroup ends
 #undef GW_BARRIER
-    if constexpr (MODE == TSATTN_MM_ADD_SCALED) {
+    if constexpr (EP_D != 0) {
+        // The producer as the product's epilogue (the reference's projection kernels end the same way,
+        // TStoreRowTileNormalizeRope, gpt/compute/gpt_rope.cuh:4-66): the int32 sums never go to memory.  The tile's
+        // 256 columns are whole heads of EP_D; 64 of its rows at a time (block i of both row halves) go through LDS as
+        // floats -- after the residual update and the rotation, which are lane-local: a wave's 64 columns are one
+        // rotation block, x in acc[.][0] and x + 32 in acc[.][1] -- so that one thread per (row, head) can add up the
+        // squares in index order, as the producer kernel and the CPU path do.  Every float operation as written there.
+#pragma clang fp contract(off)
+        constexpr int HEADS_T = GW_BN / EP_D;  // heads per tile
+        constexpr int PAIRS = 64 * HEADS_T;    // (row, head) pairs per block of rows
+        constexpr int PITCH = EP_D + 4;        // rows 16 bytes aligned, 16 lanes' 16-byte reads on 64 different banks
+        static_assert((PAIRS * PITCH + PAIRS) * 4 <= GW_LDS_BYTES && PAIRS <= GW_THREADS, "the epilogue's LDS and threads");
+        float *const vals = (float *)gw_lds;
+        float *const mults = vals + PAIRS * PITCH;
+        const ProduceParams &e = p.ep;
+        const int head_t = (wn * 64) / EP_D, xbase = (wn * 64) % EP_D;
+        const int head = (int)(n0 / EP_D) + head_t;
+        const bool head_ok = head < e.n_heads;
+        const bool turn = head < e.rope_heads;
+        __syncthreads(); // every wave is done with the operand buffers
+        // Everything a block of rows needs from memory is requested before any of it is used or stored (row by row, each
+        // row's stores would have to be waited for before the next row's loads, which they might overlap), and the next
+        // block's requests go out before this block's sums and conversion, which they pass under.
+        float cs[16], sn[16], u0[16], u1[16];
+        auto request = [&](int i) __attribute__((always_inline)) {
+            if (e.pos) {
+                int t[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                    t[r] = m < p.m ? e.pos[m] : 0;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int tc = t[r] < 0 ? 0 : (t[r] >= e.rope_len ? (int)e.rope_len - 1 : t[r]);
+                    const float *const rope_row = e.rope + (int64_t)tc * EP_D + xbase + li;
+                    cs[r] = rope_row[0];
+                    sn[r] = rope_row[32];
+                }
+            }
+            if (e.resid) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                    const bool ok = m < p.m && head_ok;
+                    const float *const q0 = e.resid + m * e.resid_pitch + (int64_t)head * EP_D + xbase + li;
+                    u0[r] = ok ? q0[0] : 0.0f;
+                    u1[r] = ok ? q0[32] : 0.0f;
+                }
+            }
+        };
+        request(0);
+#pragma unroll // (the accumulators are registers: no run-time index into them)
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int rr = 8 * (r / 4) + 4 * g + (r & 3);
+                const int64_t m = m0 + wm * 128 + i * 32 + rr;
+                float v0 = (float)acc[i][0][r], v1 = (float)acc[i][1][r];
+                if (e.resid) { // state += delta * scale, written back; the updated state is what gets normalised
+                    v0 = u0[r] + v0 * e.resid_scale;
+                    v1 = u1[r] + v1 * e.resid_scale;
+                    if (m < p.m && head_ok) {
+                        float *const q0 = e.resid + m * e.resid_pitch + (int64_t)head * EP_D + xbase + li;
+                        q0[0] = v0;
+                        q0[32] = v1;
+                    }
+                }
+                if (e.pos) {
+                    const float cos_value = turn ? cs[r] : 1.0f;
+                    const float sin_value = turn ? sn[r] * e.rotate_dir : 0.0f;
+                    const float r0 = v0 * cos_value - v1 * sin_value;
+                    const float r1 = v0 * sin_value + v1 * cos_value;
+                    v0 = r0;
+                    v1 = r1;
+                }
+                float *const dst = vals + ((wm * 32 + rr) * HEADS_T + head_t) * PITCH + xbase + li;
+                dst[0] = v0;
+                dst[32] = v1;
+            }
+            if (i + 1 < 4) request(i + 1);
+            __syncthreads();
+            if (tid < PAIRS) { // sum of squares in index order, scale
+                const int rc = tid / HEADS_T, ht = tid % HEADS_T;
+                const int64_t m = m0 + (rc / 32) * 128 + i * 32 + (rc % 32);
+                const int hd = (int)(n0 / EP_D) + ht;
+                const float *const v = vals + tid * PITCH;
+                float sum2 = 0.0f;
+#pragma unroll 4
+                for (int x = 0; x < EP_D; x += 16) { // 16 values per round of LDS reads, added in index order
+                    v4f q[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) q[c] = *(const v4f *)(v + x + 4 * c);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        sum2 = sum2 + q[c].x * q[c].x;
+                        sum2 = sum2 + q[c].y * q[c].y;
+                        sum2 = sum2 + q[c].z * q[c].z;
+                        sum2 = sum2 + q[c].w * q[c].w;
+                    }
+                }
+                float discr = 0.0f, mult = 0.0f;
+                if (sum2 != 0.0f) {
+                    const float sko = (float)sqrt((double)(sum2 / (float)EP_D)); // correctly rounded (see the producer kernel)
+                    discr = sko * e.vec_scale;
+                    mult = 1.0f / discr;
+                }
+                mults[tid] = mult;
+                const int sh = hd - e.scale_head_begin;
+                if (e.scale && m < p.m && hd < e.n_heads && sh >= 0 && sh < e.scale_head_count)
+                    e.scale[sh * e.scale_pitch + m * e.scale_row_stride] = discr * e.scale_mult;
+            }
+            __syncthreads();
+            constexpr int OUT_PER_PAIR = EP_D / 16;
+            for (int j = tid; j < PAIRS * OUT_PER_PAIR; j += GW_THREADS) { // convert and store, 16 bytes per thread and step
+                const int pr = j / OUT_PER_PAIR, x = (j % OUT_PER_PAIR) * 16;
+                const int rc = pr / HEADS_T, ht = pr % HEADS_T;
+                const int64_t m = m0 + (rc / 32) * 128 + i * 32 + (rc % 32);
+                const int hd = (int)(n0 / EP_D) + ht;
+                if (m >= p.m || hd >= e.n_heads) continue;
+                const float mult = mults[pr];
+                uint32_t w[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    w[k] = 0;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float y = vals[pr * PITCH + x + 4 * k + u] * mult;
+                        uint32_t b = mult == 0.0f ? 0u : (uint8_t)float_to_i8(y); // a head of zeros: zero bytes
+                        if (e.relu && (b & 0x80u)) b = 0u;
+                        w[k] |= b << (8 * u);
+                    }
+                }
+                *(v4i *)(e.dst + m * e.dst_pitch + (int64_t)hd * EP_D + x) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+            }
+            __syncthreads(); // before the next block of rows overwrites the values
+        }
+    } else if constexpr (MODE == TSATTN_MM_ADD_SCALED) {
         // state += sum * scale: the 32 old values of a block of rows are requested together, then updated and stored
         // (element by element every store would have to be waited for before the next load, which it might overlap;
         // with one workgroup per compute unit nothing else runs under those waits)
@@ -454,7 +591,7 @@ void launch_mode(const GemmParams &p, hipStream_t st)
         // wide tiles when there are two rounds of them for every compute unit, 128 x 128 tiles otherwise
         const int64_t tiles_n = (p.n + GT_BN - 1) / GT_BN;
         const int64_t wide = ((p.m + GW_BM - 1) / GW_BM) * ((p.n + GW_BN - 1) / GW_BN);
-        if (wide >= 512) hipLaunchKernelGGL((gemm_wide_kernel<MODE>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, p);
+        if (wide >= 512) hipLaunchKernelGGL((gemm_wide_kernel<MODE, 0>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, p);
         else hipLaunchKernelGGL((gemm_tiled_kernel<MODE, 2>), dim3((unsigned)(((p.m + 127) / 128) * tiles_n)), dim3(GT_THREADS), 0, st, p);
         return;
     }
@@ -477,10 +614,14 @@ int split_for(const GemmParams &p, int64_t room_bytes)
 // Once per device, before the first product: the wide-tile kernels use more LDS than a launch may ask for by default.
 hipError_t prepare_matmul_i8()
 {
-    hipError_t e = hipFuncSetAttribute((const void *)gemm_wide_kernel<TSATTN_MM_I32>, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)gemm_wide_kernel<TSATTN_MM_F32>, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
-    if (e == hipSuccess) e = hipFuncSetAttribute((const void *)gemm_wide_kernel<TSATTN_MM_ADD_SCALED>, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
-    return e;
+    const void *kernels[] = {(const void *)gemm_wide_kernel<TSATTN_MM_I32, 0>, (const void *)gemm_wide_kernel<TSATTN_MM_F32, 0>,
+                             (const void *)gemm_wide_kernel<TSATTN_MM_ADD_SCALED, 0>, (const void *)gemm_wide_kernel<TSATTN_MM_I32, 64>,
+                             (const void *)gemm_wide_kernel<TSATTN_MM_I32, 128>};
+    for (const void *k : kernels) {
+        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out)
@@ -494,6 +635,23 @@ hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out
         const int split = split_for(p, (int64_t)16 * p.m * p.n * 4);
         GemmParams q = p;
         q.split_stride = p.m * p.n;
+        if (p.ep_head_dim) {
+            // the producer on the result: in the product's own kernel where the wide tiles are used, else after it
+            q.ep.src = p.out; q.ep.src_pitch = p.n; q.ep.n_rows = p.m; q.ep.n_heads = (int)(p.n / p.ep_head_dim);
+            q.ep.src_planes = split; q.ep.src_plane_stride = p.m * p.n;
+            *planes_out = split;
+            const int64_t wide = ((p.m + GW_BM - 1) / GW_BM) * ((p.n + GW_BN - 1) / GW_BN);
+            if (p.m > 32 * GS_MB && wide >= 512 && p.ep_dst_dtype == TSATTN_I8) {
+                if (p.ep_head_dim == 128) hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 128>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, q);
+                else hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 64>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, q);
+                return hipGetLastError();
+            }
+            if (split == 1) launch_mode<TSATTN_MM_I32>(q, st);
+            else hipLaunchKernelGGL((gemm_skinny_kernel<TSATTN_MM_I32>), dim3((unsigned)((p.n + GS_BN - 1) / GS_BN), (unsigned)split), dim3(GS_THREADS), 0, st, q);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            return launch_rope_normalize(q.ep, p.ep_dst_dtype, p.ep_head_dim, true, st);
+        }
         if (split == 1) launch_mode<TSATTN_MM_I32>(q, st);
         else hipLaunchKernelGGL((gemm_skinny_kernel<TSATTN_MM_I32>), dim3((unsigned)((p.n + GS_BN - 1) / GS_BN), (unsigned)split), dim3(GS_THREADS), 0, st, q);
         *planes_out = split;

@@ -151,6 +151,10 @@ struct GemmParams {
     void *workspace;          // optional room for split-K partial sums (few rows)
     int64_t workspace_bytes;
     int64_t split_stride;     // set by the launcher: elements between the parts' planes
+    // optional last step (ep_head_dim != 0): the producer applied to the int32 result, as launch_rope_normalize would
+    // be with src = the result; src, src_pitch, n_rows, n_heads and the planes are filled in by the launcher
+    ProduceParams ep;
+    int ep_head_dim, ep_dst_dtype;
 };
 
 hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out);

@@ -262,6 +262,24 @@ int TLayerComputer::MulForwardPlanes(int rows, const uint8_t *vec, int k, const 
     return planes;
 }
 
+// MulForward with NormalizeState (and whatever else `a` asks of the producer) as its epilogue: one library call; large
+// products never write their int32 sums, small ones leave them in Planes for the producer's launch
+void TLayerComputer::MulForwardNormalize(int rows, const uint8_t *vec, int k, const int8_t *matr, tsattn_produce_args a, int groups,
+                                         int groupDim, uint8_t *dst, void *stream)
+{
+    a.dst_dtype = TSATTN_I8; a.head_dim = groupDim;
+    a.rotate_dir = 1; a.vec_scale = VEC_SCALE;
+    if (a.scale_mult == 0) a.scale_mult = 1;
+    a.dst = dst; a.dst_pitch = (int64_t)groups * groupDim;
+    tsattn_matmul_args m = {};
+    int planes = 0;
+    m.m = rows; m.n = groups * groupDim; m.k = k;
+    m.a = vec; m.a_pitch = k; m.w = matr; m.w_pitch = k;
+    m.mode = TSATTN_MM_I32_PLANES; m.out = Planes; m.out_pitch = m.n; m.planes_out = &planes;
+    m.epilogue = &a;
+    Check(tsattn_matmul_i8(Handle, &m, stream), "tsattn_matmul_i8");
+}
+
 // NormalizeState on int32 planes or on a float array: per group of groupDim values, to int8 (fields of `a` preset by the
 // caller select rotation, scale output, ReLU, the residual update)
 static void Normalize(tsattn_handle_t handle, tsattn_produce_args a, int rows, const void *src, bool srcI32, int planes, int groups,
@@ -283,6 +301,11 @@ static void Normalize(tsattn_handle_t handle, tsattn_produce_args a, int rows, c
 void TLayerComputer::NormalizeState(int rows, float *state, void *stream)
 {
     const int dim = Dims.Dim;
+    if (NormReadyRows > 0) { // the previous call's last product normalised the updated state as its epilogue
+        TS_VERIFY(rows == NormReadyRows, "the normalised state of %d rows is at hand, this call has %d", NormReadyRows, rows);
+        NormReadyRows = 0;
+        return;
+    }
     if (PendingPlanes > 0) {
         TS_VERIFY(rows == PendingRows, "a state update of %d rows is pending, this call has %d", PendingRows, rows);
         tsattn_produce_args a = {};
@@ -311,20 +334,6 @@ void TLayerComputer::Projections(int rows, const int32_t *pos, const float *rope
     // Matrices that lie one after the other in memory (QK, QV, K, V) are one product; the result rows hold the qk, qv, k
     // and v heads in that order either way.
     const size_t matBytes = (size_t)qsum * dim;
-    int planes = 1;
-    if ((const int8_t *)att.QV == att.QK + matBytes && att.K == att.QV + matBytes && att.V == att.K + matBytes) {
-        planes = MulForwardPlanes(rows, NormState, dim, att.QK, 4 * qsum, stream);
-    } else {
-        const int8_t *mats[4] = {att.QK, att.QV, att.K, att.V};
-        for (int i = 0; i < 4; ++i) {
-            tsattn_matmul_args a = {};
-            a.m = rows; a.n = qsum; a.k = dim;
-            a.a = NormState; a.a_pitch = dim; a.w = mats[i]; a.w_pitch = dim;
-            a.mode = TSATTN_MM_I32; a.out = Planes + (size_t)i * qsum; a.out_pitch = 4 * qsum;
-            a.workspace = Workspace; a.workspace_bytes = WorkspaceBytes;
-            Check(tsattn_matmul_i8(Handle, &a, stream), "tsattn_matmul_i8");
-        }
-    }
     // the cached key scale takes the matrix scale: qvMult *= att.QVScale * VEC_SCALE * CalcDotScale(dim)
     tsattn_produce_args a = {};
     a.pos = pos; a.rope = ropeBuf; a.rope_len = ropeLen; a.rope_heads = 2 * headCount;
@@ -333,7 +342,22 @@ void TLayerComputer::Projections(int rows, const int32_t *pos, const float *rope
     else { a.scale_pitch = 1; a.scale_row_stride = headCount; }                   // [row][head], what the cache append reads
     a.scale_head_begin = headCount; a.scale_head_count = headCount;
     a.scale_mult = att.QVScale * VEC_SCALE * sqrtf(1.0f / (float)dim);
-    Normalize(Handle, a, rows, Planes, true, planes, 4 * headCount, headDim, Q4, stream);
+    if ((const int8_t *)att.QV == att.QK + matBytes && att.K == att.QV + matBytes && att.V == att.K + matBytes) {
+        MulForwardNormalize(rows, NormState, dim, att.QK, a, 4 * headCount, headDim, Q4, stream);
+        return;
+    }
+    {
+        const int8_t *mats[4] = {att.QK, att.QV, att.K, att.V};
+        for (int i = 0; i < 4; ++i) {
+            tsattn_matmul_args mm = {};
+            mm.m = rows; mm.n = qsum; mm.k = dim;
+            mm.a = NormState; mm.a_pitch = dim; mm.w = mats[i]; mm.w_pitch = dim;
+            mm.mode = TSATTN_MM_I32; mm.out = Planes + (size_t)i * qsum; mm.out_pitch = 4 * qsum;
+            mm.workspace = Workspace; mm.workspace_bytes = WorkspaceBytes;
+            Check(tsattn_matmul_i8(Handle, &mm, stream), "tsattn_matmul_i8");
+        }
+    }
+    Normalize(Handle, a, rows, Planes, true, 1, 4 * headCount, headDim, Q4, stream);
 }
 
 // KVProduct (unless the attention call made it), combiner (its AddScaled done by the normalisation that follows:
@@ -348,19 +372,26 @@ void TLayerComputer::AfterAttention(int rows, const TAttentionMatrices &att, boo
                                 (int64_t)qsum * COMBINER_REP, stream), "tsattn_kv_product");
     }
     const int kvDim = qsum * COMBINER_REP;
-    int planes = MulForwardPlanes(rows, Kv, kvDim, att.Combiner, dim, stream);
     {
         tsattn_produce_args a = {};
         a.resid = state; a.resid_pitch = dim; a.resid_scale = att.CombinerScale * VEC_SCALE * sqrtf(1.0f / (float)kvDim);
-        Normalize(Handle, a, rows, Planes, true, planes, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
+        MulForwardNormalize(rows, Kv, kvDim, att.Combiner, a, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
     }
-    planes = MulForwardPlanes(rows, NormState, dim, att.Expand, ReluDim, stream);
     {
         tsattn_produce_args a = {};
         a.relu = 1;
-        Normalize(Handle, a, rows, Planes, true, planes, headCount, ReluDim / headCount, Relu, stream);
+        MulForwardNormalize(rows, NormState, dim, att.Expand, a, headCount, ReluDim / headCount, Relu, stream);
     }
     const float contractScale = att.ContractScale * VEC_SCALE * sqrtf(1.0f / (float)ReluDim);
+    if (deferStateUpdate && rows > 128) {
+        // many rows: the product updates the state and normalises it in its own epilogue; nothing is left pending but
+        // the next call's first normalisation is already done
+        tsattn_produce_args a = {};
+        a.resid = state; a.resid_pitch = dim; a.resid_scale = contractScale;
+        MulForwardNormalize(rows, Relu, ReluDim, att.Contract, a, dim / STATE_NORM_TILE, STATE_NORM_TILE, NormState, stream);
+        NormReadyRows = rows;
+        return;
+    }
     if (deferStateUpdate) {
         PendingPlanes = MulForwardPlanes(rows, Relu, ReluDim, att.Contract, dim, stream);
         PendingScale = contractScale;
@@ -424,7 +455,7 @@ void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, in
 void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
                                             const TAttentionMatrices &att, const int32_t *spanStart, const int32_t *spanFinish,
                                             const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
-                                            void *stream)
+                                            void *stream, bool deferStateUpdate)
 {
     TAttentionVecHistory &kvCache = *pKVCache;
     const int headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
@@ -457,7 +488,7 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
     fa.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; fa.s_head_stride = kvCache.MaxLen;
     fa.cache_len = kvCache.Length; fa.max_len = kvCache.MaxLen;
     Check(tsattn_cache_fill(Handle, &fa, stream), "tsattn_cache_fill");
-    AfterAttention(len, att, false, false, state, stream);
+    AfterAttention(len, att, false, deferStateUpdate, state, stream);
 }
 
 void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const std::vector<TAttentionVecHistory *> &kvCaches,

@@ -167,9 +167,12 @@ class TLayerComputer
     void *Workspace = nullptr;
     int64_t WorkspaceBytes = 0;
     int PendingPlanes = 0, PendingRows = 0; // a deferred state update: the contract product's parts in Planes
+    int NormReadyRows = 0;                  // NormState already holds NormalizeState of the caller's state (that many rows)
     float PendingScale = 0;
 
     int MulForwardPlanes(int rows, const uint8_t *vec, int k, const int8_t *matr, int n, void *stream);
+    void MulForwardNormalize(int rows, const uint8_t *vec, int k, const int8_t *matr, tsattn_produce_args a, int groups, int groupDim,
+                             uint8_t *dst, void *stream);
     void Projections(int rows, const int32_t *pos, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att, bool scalePlanes,
                      float *state, void *stream);
     void AfterAttention(int rows, const TAttentionMatrices &att, bool kvDone, bool deferStateUpdate, float *state, void *stream);
@@ -187,8 +190,10 @@ class TLayerComputer
 
     // t: device int32 [seqCount], the new tokens' positions; ropeBuf: device table of FillRopeBuf with ropeLen rows;
     // state: device [seqCount][Dim] fp32, updated in place; the cache gets the new rows and its lengths grow by one.
-    // deferStateUpdate: leave the layer's last state update (contract's AddScaled) to the first normalisation of the next
-    // call on the same state rows, or to FlushState -- one launch less per layer; until then `state` lacks that update.
+    // deferStateUpdate (layers that follow one another on the same state rows): with few rows the layer's last state
+    // update (contract's AddScaled) is left to the first normalisation of the next call, or to FlushState -- one launch
+    // less per layer; until then `state` lacks that update.  With many rows the last product updates the state and
+    // normalises it for the next call as its epilogue.  Either way finish with FlushState.
     void AddLookupProduct(const int32_t *t, const float *ropeBuf, int64_t ropeLen, const TAttentionMatrices &att,
                           TAttentionVecHistory *pKVCache, float *state, void *stream, bool deferStateUpdate = false);
     // Does a pending state update and returns NormalizeState(state) (device, int8 [rows][Dim]), which is what
@@ -200,7 +205,7 @@ class TLayerComputer
     void AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
                                 const TAttentionMatrices &att, const int32_t *spanStart, const int32_t *spanFinish,
                                 const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
-                                void *stream);
+                                void *stream, bool deferStateUpdate = false);
     const float *GetValLookup() const { return ValLookup; } // [rows][HeadCount*TTDim] of the last call
 };
 
