@@ -316,6 +316,19 @@ def bench_matmul(ctx, steps):
     res["square_8192"] = {"ms": round(ms, 4), "TOP/s": round(2.0 * m2 * m2 * k / ms / 1e9, 2),
                           "frac_of_int8_peak": round(2.0 * m2 * m2 * k / ms / 1e9 / PEAK_I8_TOPS, 4)}
     del a, w2, out
+    # the four projections of the prompt batch as one product with the producer as its epilogue: RoPE on the qk and
+    # qv heads, per-head normalisation, int8 rows and the key scales; the int32 sums are never stored
+    m, kp, npj, H = 32 * 2048, 2048, 4 * 16 * 128, 16
+    a = torch.randint(0, 256, (m, kp), dtype=torch.uint8, device="cuda", generator=g)
+    wp = torch.randint(0, 256, (npj, kp), dtype=torch.uint8, device="cuda", generator=g)
+    rope = ctx.fill_rope_table(128, 2048)
+    pos = torch.arange(2048, dtype=torch.int32, device="cuda").repeat(32)
+    scratch = torch.empty(m * npj, dtype=torch.int32, device="cuda")
+    ms = gpu_time_ms(lambda: ctx.matmul_normalize(a, wp, 4 * H, capi.I8, scratch, pos=pos, rope=rope, scale_mult=0.01, rope_heads=2 * H,
+                                                  scale_heads=(H, H)), max(3, steps // 10), 2)
+    res["prompt_projections_with_producer"] = {"rows": m, "k": kp, "n": npj, "ms": round(ms, 4), "TOP/s": round(2.0 * m * npj * kp / ms / 1e9, 2),
+                                               "frac_of_int8_peak": round(2.0 * m * npj * kp / ms / 1e9 / PEAK_I8_TOPS, 4)}
+    del a, wp, scratch
     m = 32
     a = torch.randint(0, 256, (m, k), dtype=torch.uint8, device="cuda", generator=g)
     state = torch.zeros((m, n), dtype=torch.float32, device="cuda")
