@@ -247,6 +247,12 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
         asm volatile("" ::: "memory");                          \
     } while (0)
     const int n_steps = (int)(p.k / GW_BK);
+    // (with the producer as epilogue: the position of tile row tid, asked for now, so that the epilogue's rope rows do not
+    // wait for it)
+    int row_pos = 0;
+    if constexpr (EP_D != 0) {
+        if (p.ep.pos && tid < GW_BM && m0 + tid < p.m) row_pos = p.ep.pos[m0 + tid];
+    }
     // requests past K fetch bytes that are never computed with (or zeros past the rows' end)
     request(0, gw_lds);
     request(GW_BK, gw_lds + GW_BUF);
@@ -300,30 +306,28 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
         constexpr int HEADS_T = GW_BN / EP_D;  // heads per tile
         constexpr int PAIRS = 64 * HEADS_T;    // (row, head) pairs per block of rows
         constexpr int PITCH = EP_D + 4;        // rows 16 bytes aligned, 16 lanes' 16-byte reads on 64 different banks
-        static_assert((PAIRS * PITCH + PAIRS) * 4 <= GW_LDS_BYTES && PAIRS <= GW_THREADS, "the epilogue's LDS and threads");
+        static_assert((PAIRS * PITCH + PAIRS + GW_BM) * 4 <= GW_LDS_BYTES && PAIRS <= GW_THREADS, "the epilogue's LDS and threads");
         float *const vals = (float *)gw_lds;
         float *const mults = vals + PAIRS * PITCH;
+        int *const tile_pos = (int *)(mults + PAIRS); // positions of the tile's 256 rows
         const ProduceParams &e = p.ep;
         const int head_t = (wn * 64) / EP_D, xbase = (wn * 64) % EP_D;
         const int head = (int)(n0 / EP_D) + head_t;
         const bool head_ok = head < e.n_heads;
         const bool turn = head < e.rope_heads;
         __syncthreads(); // every wave is done with the operand buffers
+        if (tid < GW_BM) tile_pos[tid] = row_pos;
+        __syncthreads();
         // Everything a block of rows needs from memory is requested before any of it is used or stored (row by row, each
         // row's stores would have to be waited for before the next row's loads, which they might overlap), and the next
         // block's requests go out before this block's sums and conversion, which they pass under.
         float cs[16], sn[16], u0[16], u1[16];
         auto request = [&](int i) __attribute__((always_inline)) {
             if (e.pos) {
-                int t[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
-                    t[r] = m < p.m ? e.pos[m] : 0;
-                }
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int tc = t[r] < 0 ? 0 : (t[r] >= e.rope_len ? (int)e.rope_len - 1 : t[r]);
+                    const int t = tile_pos[wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3)];
+                    const int tc = t < 0 ? 0 : (t >= e.rope_len ? (int)e.rope_len - 1 : t);
                     const float *const rope_row = e.rope + (int64_t)tc * EP_D + xbase + li;
                     cs[r] = rope_row[0];
                     sn[r] = rope_row[32];
