@@ -316,19 +316,25 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
         const bool head_ok = head < e.n_heads;
         const bool turn = head < e.rope_heads;
         __syncthreads(); // every wave is done with the operand buffers
-        if (tid < GW_BM) tile_pos[tid] = row_pos;
+        if (tid < GW_BM) tile_pos[tid] = row_pos < 0 ? 0 : (row_pos >= e.rope_len ? (int)e.rope_len - 1 : row_pos);
         __syncthreads();
+        // Addresses inside the tile are 32-bit offsets from a base that is the same for the whole wave (the launcher
+        // checks that the pitches allow it): one add per access instead of a 64-bit multiply.
+        const int rows_here = (int)(p.m - m0 < GW_BM ? p.m - m0 : GW_BM);
+        const bool rotate = e.pos && turn;
+        const char *const rope_base = (const char *)(e.rope + xbase);
+        char *const resid_base = (char *)(e.resid + m0 * e.resid_pitch + (int64_t)head * EP_D + xbase);
+        const uint32_t resid_pitch_bytes = (uint32_t)e.resid_pitch * 4u;
         // Everything a block of rows needs from memory is requested before any of it is used or stored (row by row, each
         // row's stores would have to be waited for before the next row's loads, which they might overlap), and the next
         // block's requests go out before this block's sums and conversion, which they pass under.
         float cs[16], sn[16], u0[16], u1[16];
         auto request = [&](int i) __attribute__((always_inline)) {
-            if (e.pos) {
+            if (rotate) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int t = tile_pos[wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3)];
-                    const int tc = t < 0 ? 0 : (t >= e.rope_len ? (int)e.rope_len - 1 : t);
-                    const float *const rope_row = e.rope + (int64_t)tc * EP_D + xbase + li;
+                    const uint32_t t = (uint32_t)tile_pos[wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3)];
+                    const float *const rope_row = (const float *)(rope_base + (t * (uint32_t)(EP_D * 4) + (uint32_t)li * 4u));
                     cs[r] = rope_row[0];
                     sn[r] = rope_row[32];
                 }
@@ -336,9 +342,9 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
             if (e.resid) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int64_t m = m0 + wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
-                    const bool ok = m < p.m && head_ok;
-                    const float *const q0 = e.resid + m * e.resid_pitch + (int64_t)head * EP_D + xbase + li;
+                    const int row = wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+                    const bool ok = row < rows_here && head_ok;
+                    const float *const q0 = (const float *)(resid_base + ((uint32_t)row * resid_pitch_bytes + (uint32_t)li * 4u));
                     u0[r] = ok ? q0[0] : 0.0f;
                     u1[r] = ok ? q0[32] : 0.0f;
                 }
@@ -350,25 +356,25 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int rr = 8 * (r / 4) + 4 * g + (r & 3);
-                const int64_t m = m0 + wm * 128 + i * 32 + rr;
+                const int row = wm * 128 + i * 32 + rr;
                 float v0 = (float)acc[i][0][r], v1 = (float)acc[i][1][r];
                 if (e.resid) { // state += delta * scale, written back; the updated state is what gets normalised
                     v0 = u0[r] + v0 * e.resid_scale;
                     v1 = u1[r] + v1 * e.resid_scale;
-                    if (m < p.m && head_ok) {
-                        float *const q0 = e.resid + m * e.resid_pitch + (int64_t)head * EP_D + xbase + li;
+                    if (row < rows_here && head_ok) {
+                        float *const q0 = (float *)(resid_base + ((uint32_t)row * resid_pitch_bytes + (uint32_t)li * 4u));
                         q0[0] = v0;
                         q0[32] = v1;
                     }
                 }
-                if (e.pos) {
-                    const float cos_value = turn ? cs[r] : 1.0f;
-                    const float sin_value = turn ? sn[r] * e.rotate_dir : 0.0f;
+                if (rotate) {
+                    const float cos_value = cs[r];
+                    const float sin_value = sn[r] * e.rotate_dir;
                     const float r0 = v0 * cos_value - v1 * sin_value;
                     const float r1 = v0 * sin_value + v1 * cos_value;
                     v0 = r0;
                     v1 = r1;
-                }
+                } // (a head that is not rotated: cos 1 and sin 0 leave the values as they are)
                 float *const dst = vals + ((wm * 32 + rr) * HEADS_T + head_t) * PITCH + xbase + li;
                 dst[0] = v0;
                 dst[32] = v1;
@@ -381,13 +387,13 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
                 const int hd = (int)(n0 / EP_D) + ht;
                 const float *const v = vals + tid * PITCH;
                 float sum2 = 0.0f;
-#pragma unroll 4
-                for (int x = 0; x < EP_D; x += 16) { // 16 values per round of LDS reads, added in index order
-                    v4f q[4];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) q[c] = *(const v4f *)(v + x + 4 * c);
+                for (int x = 0; x < EP_D; x += 32) { // 32 values per round of LDS reads, added in index order
+                    v4f q[8];
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
+                    for (int c = 0; c < 8; ++c) q[c] = *(const v4f *)(v + x + 4 * c);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
                         sum2 = sum2 + q[c].x * q[c].x;
                         sum2 = sum2 + q[c].y * q[c].y;
                         sum2 = sum2 + q[c].z * q[c].z;
@@ -406,27 +412,34 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
                     e.scale[sh * e.scale_pitch + m * e.scale_row_stride] = discr * e.scale_mult;
             }
             __syncthreads();
+            // Convert and store, 16 bytes per thread and step.  Clamping before rounding gives what rounding before
+            // clamping gives (the bounds are whole numbers); adding 1.5 * 2^23 rounds to nearest even and leaves the whole
+            // number, in two's complement, in the low bits of the float.  A head of zeros has mult 0: zero bytes.
             constexpr int OUT_PER_PAIR = EP_D / 16;
-            for (int j = tid; j < PAIRS * OUT_PER_PAIR; j += GW_THREADS) { // convert and store, 16 bytes per thread and step
+            static_assert((PAIRS * OUT_PER_PAIR) % GW_THREADS == 0, "whole steps of the workgroup");
+            const float low = e.relu ? 0.0f : -127.0f;
+            uint8_t *const dst_base = e.dst + m0 * e.dst_pitch + n0;
+#pragma unroll
+            for (int j0 = 0; j0 < PAIRS * OUT_PER_PAIR; j0 += GW_THREADS) {
+                const int j = j0 + tid;
                 const int pr = j / OUT_PER_PAIR, x = (j % OUT_PER_PAIR) * 16;
                 const int rc = pr / HEADS_T, ht = pr % HEADS_T;
-                const int64_t m = m0 + (rc / 32) * 128 + i * 32 + (rc % 32);
-                const int hd = (int)(n0 / EP_D) + ht;
-                if (m >= p.m || hd >= e.n_heads) continue;
+                const int row = (rc / 32) * 128 + i * 32 + (rc % 32);
                 const float mult = mults[pr];
+                v4f q[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) q[k] = *(const v4f *)(vals + pr * PITCH + x + 4 * k);
                 uint32_t w[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    w[k] = 0;
+                    uint32_t b[4];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const float y = vals[pr * PITCH + x + 4 * k + u] * mult;
-                        uint32_t b = mult == 0.0f ? 0u : (uint8_t)float_to_i8(y); // a head of zeros: zero bytes
-                        if (e.relu && (b & 0x80u)) b = 0u;
-                        w[k] |= b << (8 * u);
-                    }
+                    for (int u = 0; u < 4; ++u) b[u] = __float_as_uint(fminf(fmaxf(q[k][u] * mult, low), 127.0f) + 12582912.0f);
+                    // byte 0 of each of the four
+                    w[k] = __builtin_amdgcn_perm(__builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u), __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u), 0x05040100u);
                 }
-                *(v4i *)(e.dst + m * e.dst_pitch + (int64_t)hd * EP_D + x) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+                if (row < rows_here && (int)(n0 / EP_D) + ht < e.n_heads)
+                    *(v4i *)(dst_base + ((uint32_t)row * (uint32_t)e.dst_pitch + (uint32_t)(ht * EP_D + x))) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
             }
             __syncthreads(); // before the next block of rows overwrites the values
         }
@@ -645,7 +658,10 @@ hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out
             q.ep.src_planes = split; q.ep.src_plane_stride = p.m * p.n;
             *planes_out = split;
             const int64_t wide = ((p.m + GW_BM - 1) / GW_BM) * ((p.n + GW_BN - 1) / GW_BN);
-            if (p.m > 32 * GS_MB && wide >= 512 && p.ep_dst_dtype == TSATTN_I8) {
+            // (the epilogue addresses a tile's rows with 32-bit offsets)
+            const bool offsets_fit = q.ep.dst_pitch < (1 << 23) && (!q.ep.resid || q.ep.resid_pitch < (1 << 21)) &&
+                                     (!q.ep.pos || q.ep.rope_len * p.ep_head_dim * 4 < ((int64_t)1 << 31));
+            if (p.m > 32 * GS_MB && wide >= 512 && p.ep_dst_dtype == TSATTN_I8 && offsets_fit) {
                 if (p.ep_head_dim == 128) hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 128>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, q);
                 else hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 64>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, q);
                 return hipGetLastError();
