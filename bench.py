@@ -507,7 +507,8 @@ def bench_prompt_pass(ctx, steps):
             c.cache_len.zero_()
             w = layer["width"]
             _, norm = add_lookup_product_prompt(ctx, layer, c, off, pos, m.rope, state, *spans[w], span_tiles=tiles[w],
-                                                causal_period=m.prompt if w >= m.prompt else 0, norm=norm, want_norm=True)
+                                                causal_period=m.prompt if w >= m.prompt else 0, norm=norm, want_norm=True,
+                                                want_val=False)
     ms = gpu_time_ms(run, 2, 1)
     assert bool(torch.isfinite(state).all()) and int(m.caches[0].cache_len[0]) == m.prompt
     att_flops = sum(prefill_flops(B, m.prompt, H, d, w) for w, _ in m.sched)

@@ -103,6 +103,17 @@ typedef struct tsattn_prefill_args {
                                     sequences under a wide causal window, as the reference's fixed-length
                                     fragments are).  Only the order in which work is launched depends on it,
                                     never the result; a value the kernel cannot use is ignored. */
+    /* Optional fused consumer (kv_out == NULL = off): KVProduct of the result with each token's K vector, as
+     * tsattn_kv_product(k = kv_k, value = out, mult = kv_mult) would make it from an f32 `out` afterwards, bit for
+     * bit (the batch form of cpu_infer.cpp:511, :320-337; on the GPU the reference does it in its own kernel,
+     * gpt/compute/gpt_combiner.cuh:13-37).  dtype must be int8 and out_dtype f32 (TSATTN_ERR_UNSUPPORTED otherwise:
+     * make the two calls); `out` may then be NULL (the result itself is not written) and debug_qk_acc must be. */
+    const void *kv_k;          /* int8 [n_tokens][n_heads*head_dim], row pitch kv_k_pitch bytes, 4-byte aligned */
+    int64_t kv_k_pitch;
+    void *kv_out;              /* int8 [n_tokens][n_heads*kv_rep*head_dim], row pitch kv_out_pitch bytes, 16-byte aligned */
+    int64_t kv_out_pitch;
+    int kv_rep;                /* 1..4 */
+    float kv_mult;
 } tsattn_prefill_args;
 
 int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream);

@@ -370,3 +370,59 @@ def test_prefill_randomised_shapes(ctx, seed):
     assert np.array_equal(outs[0], outs[1]), what
     assert_within_tolerance(outs[0], want, what)
     assert not outs[0][fi < st].any(), what
+
+
+@pytest.mark.parametrize("d,H,seq_lens,window,slope,rep", [
+    (128, 3, [300, 1, 129, 70], 10 ** 6, 0.0, 4),
+    (128, 2, [257], 64, 0.5, 3),
+    (64, 5, [40, 200, 333], 10 ** 6, 0.0, 4),
+    (64, 2, [128, 128], 1, 0.25, 1),
+    (64, 1, [100], 0, 0.0, 2),
+])
+def test_prefill_fused_kv_product_equals_the_separate_call(ctx, d, H, seq_lens, window, slope, rep):
+    """KVProduct as the prefill kernel's last step: the same bytes as tsattn_kv_product on the f32 result of the same
+    launch (which the oracle's KVProduct of that result confirms), with and without the result itself written, with
+    the K rows and the output inside wider rows, and nothing written outside the output's columns."""
+    n = sum(seq_lens)
+    q, qs, k, ks, v, vs = make_qkv(70 + d + rep, n, H, d, capi.I8)
+    st, fi = orc.make_spans(seq_lens, window)
+    rng = np.random.default_rng(5 + rep)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    wide = t(rng.integers(-127, 128, (n, H * d + 64), dtype=np.int8).view(np.uint8))
+    kk = wide[:, 32:32 + H * d]   # 4-byte aligned rows of a wider array
+    mult = 0.37
+    args = (capi.I8, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), slope)
+    room = torch.full((n, H * d * rep + 48), 0x5a, dtype=torch.uint8, device="cuda")
+    kv_out = room[:, 16:16 + H * d * rep]
+    out = ctx.compute_val_lookup(*args, kv_product=(kk, kv_out, rep, mult))
+    plain = ctx.compute_val_lookup(*args)
+    assert torch.equal(out, plain), "the result itself changes with the fused consumer"
+    separate = ctx.kv_product(kk.contiguous(), plain, H, rep, mult)
+    assert torch.equal(kv_out, separate), "fused KVProduct differs from the separate call"
+    want = orc.kv_product(kk.cpu().numpy(), plain.cpu().numpy(), H, rep, mult)
+    assert np.array_equal(kv_out.cpu().numpy().view(np.int8), want)
+    assert (room[:, :16] == 0x5a).all() and (room[:, 16 + H * d * rep:] == 0x5a).all()
+    # without the result, with the span summary and a period hint
+    kv2 = torch.zeros((n, H * d * rep), dtype=torch.uint8, device="cuda")
+    tiles = ctx.build_span_tiles(t(st), t(fi))
+    none = ctx.compute_val_lookup(*args, kv_product=(kk, kv2, rep, mult), want_out=False, span_tiles=tiles, causal_period=seq_lens[0])
+    assert none is None and torch.equal(kv2, separate)
+
+
+def test_prefill_fused_kv_product_argument_checks(ctx):
+    n, H, d = 64, 1, 64
+    q, qs, k, ks, v, vs = make_qkv(3, n, H, d, capi.E4M3)
+    st, fi = orc.make_spans([n], 10 ** 6)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    kk = torch.zeros((n, H * d), dtype=torch.uint8, device="cuda")
+    kv = torch.zeros((n, H * d * 4), dtype=torch.uint8, device="cuda")
+    with pytest.raises(capi.TsattnError):      # e4m3 attention: no fused consumer
+        ctx.compute_val_lookup(capi.E4M3, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), 0.0, kv_product=(kk, kv, 4, 1.0))
+    q, qs, k, ks, v, vs = make_qkv(3, n, H, d, capi.I8)
+    args = (capi.I8, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), 0.0)
+    with pytest.raises(capi.TsattnError):      # f16 result
+        ctx.compute_val_lookup(*args, out_f16=True, kv_product=(kk, kv, 4, 1.0))
+    with pytest.raises(capi.TsattnError):      # rep out of range
+        ctx.compute_val_lookup(*args, kv_product=(kk, kv, 5, 1.0))
+    with pytest.raises(capi.TsattnError):      # output rows too short
+        ctx.compute_val_lookup(*args, kv_product=(kk, kv[:, :H * d * 2].contiguous(), 4, 1.0))

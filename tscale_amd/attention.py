@@ -276,17 +276,21 @@ class AttentionContext:
     # ---- prefill --------------------------------------------------------------------------------
     def compute_val_lookup(self, dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, span_start, span_finish,
                            alibi_slope, out=None, out_f16=False, sum_weight_log=None, k_global_scale=None,
-                           debug_qk_acc=None, causal_period=0, span_tiles=None):
+                           debug_qk_acc=None, causal_period=0, span_tiles=None, kv_product=None, want_out=True):
         """q,k,v: uint8 [n_tokens, n_heads*d] (row pitch = stride(0)); scales f32 [n_heads, n_tokens] or numbers.
         causal_period: launch-order hint for batches of equal-length sequences under a wide causal window (the
-        common sequence length); never changes the result.  span_tiles: what build_span_tiles made of these spans."""
+        common sequence length); never changes the result.  span_tiles: what build_span_tiles made of these spans.
+        kv_product = (k, kv_out, rep, mult): KVProduct of the f32 result with the tokens' K vectors, written by the same
+        launch (k uint8 [n_tokens, H*d], kv_out uint8 [n_tokens, H*rep*d]); with want_out=False the result itself is
+        not written and None is returned."""
         n_tokens, hd = q.shape
         d = hd // n_heads
-        if out is None:
+        assert want_out or kv_product is not None
+        if out is None and want_out:
             out = torch.empty((n_tokens, hd), dtype=torch.float16 if out_f16 else torch.float32, device=q.device)
         a = capi.PrefillArgs()
         a.dtype = dtype
-        a.out_dtype = capi.OUT_F16 if out.dtype == torch.float16 else capi.OUT_F32
+        a.out_dtype = capi.OUT_F16 if (out is not None and out.dtype == torch.float16) else capi.OUT_F32
         a.n_tokens, a.n_heads, a.head_dim = n_tokens, n_heads, d
         a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
         a.q_pitch, a.k_pitch, a.v_pitch = q.stride(0), k.stride(0), v.stride(0)
@@ -299,10 +303,17 @@ class AttentionContext:
         a.k_global_scale = _ptr(k_global_scale)
         a.span_start, a.span_finish = _ptr(span_start), _ptr(span_finish)
         a.alibi_slope = float(alibi_slope)
-        a.out, a.out_pitch = _ptr(out), out.stride(0) * out.element_size()
+        if out is not None:
+            a.out, a.out_pitch = _ptr(out), out.stride(0) * out.element_size()
         a.sum_weight_log = _ptr(sum_weight_log)
         if debug_qk_acc is not None:
             a.debug_qk_acc, a.debug_pitch = _ptr(debug_qk_acc), debug_qk_acc.stride(1)
+        if kv_product is not None:
+            kv_k, kv_out, kv_rep, kv_mult = kv_product
+            assert kv_k.stride(1) == 1 and kv_out.stride(1) == 1
+            a.kv_k, a.kv_k_pitch = _ptr(kv_k), kv_k.stride(0)
+            a.kv_out, a.kv_out_pitch = _ptr(kv_out), kv_out.stride(0)
+            a.kv_rep, a.kv_mult = int(kv_rep), float(kv_mult)
         a.causal_period = int(causal_period)
         a.span_tiles = _ptr(span_tiles)
         capi.check(self.lib.tsattn_prefill(self.handle, ctypes.byref(a), _stream_ptr()))
@@ -420,13 +431,14 @@ def flush_state(ctx, pending, state):
 
 
 def add_lookup_product_prompt(ctx, layer, cache, seq_offset, pos, rope, state, span_start, span_finish, span_tiles=None,
-                              causal_period=0, norm=None, want_norm=False):
+                              causal_period=0, norm=None, want_norm=False, want_val=True):
     """The same layer for a whole batch of prompt tokens at once (sequences concatenated, seq_offset int32 [B+1], pos
     int32 [n_tokens] = each token's position in its sequence): every token's attention over the earlier tokens of its
     sequence is one tsattn_prefill launch, and the tokens' key and value rows go into the cache in one
     tsattn_cache_fill.  Token by token through add_lookup_product gives the same cache and the same states (a token's
     layer input does not depend on other tokens' outputs of the same layer).  state: f32 [n_tokens, dim], updated in
-    place; the spans are those of the layer's width (build_spans).  Returns the attention output.
+    place; the spans are those of the layer's width (build_spans).  Returns the attention output (None with
+    want_val=False: KVProduct is the attention kernel's last step and nothing else reads the output).
     norm: NormalizeState(state) where the caller has it (the previous layer's second result); want_norm=True returns
     (attention output, NormalizeState(new state)), which the layer's last product then makes as its epilogue."""
     n, dim = state.shape
@@ -443,10 +455,12 @@ def add_lookup_product_prompt(ctx, layer, cache, seq_offset, pos, rope, state, s
     q4, qv_scale = ctx.matmul_normalize(norm, layer["proj"], 4 * H, capi.I8, room, pos=pos, rope=rope, scale_mult=key_mult,
                                         rope_heads=2 * H, scale_heads=(H, H))      # scales as [head][token] planes
     qk, qv, k, v = q4[:, :qsum], q4[:, qsum:2 * qsum], q4[:, 2 * qsum:3 * qsum], q4[:, 3 * qsum:]
+    # attention with KVProduct as its last step: the result itself is written only for a caller who wants it
+    kv = torch.empty((n, qsum * COMBINER_REP), dtype=torch.uint8, device=state.device)
     val = ctx.compute_val_lookup(capi.I8, H, qk, qv, v, VEC_SCALE, qv_scale, VEC_SCALE, span_start, span_finish, layer["slope"],
-                                 span_tiles=span_tiles, causal_period=causal_period)
+                                 span_tiles=span_tiles, causal_period=causal_period, kv_product=(k, kv, COMBINER_REP, 1.0),
+                                 want_out=want_val)
     cache.fill_from_prefill(seq_offset, qv, qv_scale, v)       # value scales: the cache's constant VEC_SCALE
-    kv = ctx.kv_product(k, val, H, COMBINER_REP)
     norm, _ = ctx.matmul_normalize(kv, layer["combiner"], groups, capi.I8, room, resid=state,
                                    resid_scale=float(f32(layer["combiner_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(qsum * COMBINER_REP)))))
     del kv

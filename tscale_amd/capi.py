@@ -42,6 +42,8 @@ class PrefillArgs(_c.Structure):
         ("span_finish", _c.c_void_p), ("alibi_slope", _c.c_float), ("out", _c.c_void_p),
         ("out_pitch", _c.c_int64), ("sum_weight_log", _c.c_void_p), ("debug_qk_acc", _c.c_void_p),
         ("debug_pitch", _c.c_int64), ("span_tiles", _c.c_void_p), ("causal_period", _c.c_int64),
+        ("kv_k", _c.c_void_p), ("kv_k_pitch", _c.c_int64), ("kv_out", _c.c_void_p), ("kv_out_pitch", _c.c_int64),
+        ("kv_rep", _c.c_int), ("kv_mult", _c.c_float),
     ]
 
 

@@ -124,20 +124,35 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     if (a->n_tokens < 0 || a->n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: n_tokens %lld n_heads %d", (long long)a->n_tokens, a->n_heads);
     if (a->n_tokens > 0x7fffffff - 256) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: n_tokens too large");
     if (a->n_tokens == 0) return TSATTN_OK;
-    if (!a->q || !a->k || !a->v || !a->out || !a->span_start || !a->span_finish)
+    if (!a->q || !a->k || !a->v || (!a->out && !a->kv_out) || !a->span_start || !a->span_finish)
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: null data pointer");
     const int64_t row = (int64_t)a->n_heads * a->head_dim;
     if (a->q_pitch < row || a->k_pitch < row || a->v_pitch < row || (a->q_pitch | a->k_pitch | a->v_pitch) % 16)
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: input pitch must be >= %lld and a multiple of 16", (long long)row);
     const int64_t out_row = row * (a->out_dtype == TSATTN_OUT_F16 ? 2 : 4);
-    if (a->out_pitch < out_row || a->out_pitch % 16) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: out_pitch must be >= %lld and a multiple of 16", (long long)out_row);
+    if (a->out && (a->out_pitch < out_row || a->out_pitch % 16)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: out_pitch must be >= %lld and a multiple of 16", (long long)out_row);
     if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out))
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: q, k, v, out must be 16-byte aligned");
     if ((a->q_scale || a->k_scale || a->v_scale || a->sum_weight_log) && a->scale_pitch < a->n_tokens)
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: scale_pitch %lld < n_tokens", (long long)a->scale_pitch);
     if (a->debug_qk_acc && a->debug_pitch < a->n_tokens) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: debug_pitch < n_tokens");
 
-    tsattn::PrefillParams p;
+    if (a->kv_out) {
+        if (!a->kv_k) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: the fused KVProduct needs kv_k");
+        if (a->out_dtype != TSATTN_OUT_F32 || a->dtype != TSATTN_I8)
+            return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_prefill: the fused KVProduct goes with int8 attention and takes the f32 result (out_dtype f32)");
+        if (a->debug_qk_acc) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_prefill: no fused KVProduct together with debug_qk_acc");
+        if (a->kv_rep < 1 || a->kv_rep > 4) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: kv_rep %d (1..4)", a->kv_rep);
+        if (((uintptr_t)a->kv_k & 3) || a->kv_k_pitch % 4 || a->kv_k_pitch < row || !aligned16(a->kv_out) || a->kv_out_pitch % 16 ||
+            a->kv_out_pitch < row * a->kv_rep)
+            return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: kv_k must be 4-byte aligned, kv_out 16-byte aligned (pitches too) and the kv pitches must cover a row");
+    }
+
+    tsattn::PrefillParams p = {};
+    if (a->kv_out) {
+        p.kv_k = (const uint8_t *)a->kv_k; p.kv_k_pitch = a->kv_k_pitch; p.kv_out = (uint8_t *)a->kv_out; p.kv_out_pitch = a->kv_out_pitch;
+        p.kv_rep = a->kv_rep; p.kv_mult = a->kv_mult;
+    }
     p.q = (const uint8_t *)a->q; p.k = (const uint8_t *)a->k; p.v = (const uint8_t *)a->v;
     p.q_pitch = a->q_pitch; p.k_pitch = a->k_pitch; p.v_pitch = a->v_pitch;
     p.qs = a->q_scale; p.ks = a->k_scale; p.vs = a->v_scale;

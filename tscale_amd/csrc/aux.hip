@@ -191,35 +191,69 @@ hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st
 }
 
 // Bulk form of the append: the K/V rows of a prefill batch ([token][head*d]) go to the planar cache.
-// A workgroup handles 64 consecutive tokens of one head: reads are 16 bytes per lane with the lanes of a
-// row adjacent, writes cover whole cache rows back to back.
+// A workgroup handles 16 consecutive tokens with all their heads: a wave reads 1 KiB of a row at a time, four
+// requests of K and four of V per thread are out before the first store, and every token is looked up in the
+// sequence offsets once, not once per thread.
+constexpr int FILL_TOKENS = 16;
+
 __global__ __launch_bounds__(256) void cache_fill_kernel(FillParams p)
 {
-    const int chunks = p.head_dim / 16;
-    const int rows_per_block = 256 / chunks;
-    const int head = blockIdx.y;
-    const int c = threadIdx.x % chunks;
-    const int64_t tok = (int64_t)blockIdx.x * rows_per_block + threadIdx.x / chunks;
-    if (tok >= p.n_tokens) return;
-    // sequence of this token: last s with seq_offset[s] <= tok
-    int lo = 0, hi = p.n_seqs;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (p.seq_offset[mid] <= tok) lo = mid; else hi = mid;
+    __shared__ int s_seq[FILL_TOKENS];
+    __shared__ int64_t s_pos[FILL_TOKENS]; // -1: nothing to write for this token
+    const int64_t tok0 = (int64_t)blockIdx.x * FILL_TOKENS;
+    if (threadIdx.x < FILL_TOKENS) {
+        const int64_t tok = tok0 + threadIdx.x;
+        int seq = 0;
+        int64_t pos = -1;
+        if (tok < p.n_tokens) {
+            // sequence of this token: last s with seq_offset[s] <= tok
+            int lo = 0, hi = p.n_seqs;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (p.seq_offset[mid] <= tok) lo = mid; else hi = mid;
+            }
+            seq = lo;
+            const int64_t first = p.seq_offset[seq];
+            if (tok >= first && tok < p.seq_offset[seq + 1]) {
+                pos = (int64_t)p.cache_len[seq] + (tok - first);
+                if (pos < 0 || pos >= p.max_len) pos = -1;
+            }
+        }
+        s_seq[threadIdx.x] = seq;
+        s_pos[threadIdx.x] = pos;
     }
-    const int seq = lo;
-    const int64_t first = p.seq_offset[seq];
-    if (tok < first || tok >= p.seq_offset[seq + 1]) return;
-    const int64_t pos = (int64_t)p.cache_len[seq] + (tok - first);
-    if (pos < 0 || pos >= p.max_len) return;
-    const int64_t src = tok * p.pitch + head * p.head_dim + c * 16;
-    const int64_t dst = (int64_t)seq * p.seq_stride + (int64_t)head * p.head_stride + pos * p.tok_stride + c * 16;
-    *(v4i *)(p.k + dst) = *(const v4i *)(p.k_src + src);
-    *(v4i *)(p.v + dst) = *(const v4i *)(p.v_src + src);
-    if (c == 0) {
-        const int64_t sd = (int64_t)seq * p.s_seq_stride + (int64_t)head * p.s_head_stride + pos;
-        if (p.ks_src) p.ks[sd] = p.ks_src[(int64_t)head * p.scale_pitch + tok];
-        if (p.vs_src) p.vs[sd] = p.vs_src[(int64_t)head * p.scale_pitch + tok];
+    __syncthreads();
+    const int chunks_head = p.head_dim / 16, chunks_row = p.n_heads * chunks_head;
+    const int total = FILL_TOKENS * chunks_row;
+    for (int base = 0; base < total; base += 4 * 256) {
+        v4i kk[4], vv[4];
+        int64_t dst[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int id = base + u * 256 + (int)threadIdx.x;
+            const int t = id / chunks_row, c = id % chunks_row;
+            dst[u] = -1;
+            if (id < total && s_pos[t] >= 0) {
+                const int head = c / chunks_head, within = c % chunks_head;
+                const int64_t src = (tok0 + t) * p.pitch + c * 16;
+                dst[u] = (int64_t)s_seq[t] * p.seq_stride + (int64_t)head * p.head_stride + s_pos[t] * p.tok_stride + within * 16;
+                kk[u] = *(const v4i *)(p.k_src + src);
+                vv[u] = *(const v4i *)(p.v_src + src);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (dst[u] >= 0) {
+                *(v4i *)(p.k + dst[u]) = kk[u];
+                *(v4i *)(p.v + dst[u]) = vv[u];
+            }
+    }
+    for (int id = threadIdx.x; id < FILL_TOKENS * p.n_heads; id += 256) { // scales: consecutive lanes, consecutive tokens
+        const int head = id / FILL_TOKENS, t = id % FILL_TOKENS;
+        if (s_pos[t] < 0) continue;
+        const int64_t sd = (int64_t)s_seq[t] * p.s_seq_stride + (int64_t)head * p.s_head_stride + s_pos[t];
+        if (p.ks_src) p.ks[sd] = p.ks_src[(int64_t)head * p.scale_pitch + tok0 + t];
+        if (p.vs_src) p.vs[sd] = p.vs_src[(int64_t)head * p.scale_pitch + tok0 + t];
     }
 }
 
@@ -236,9 +270,7 @@ __global__ void cache_len_add_kernel(int32_t *cache_len, const int32_t *seq_offs
 hipError_t launch_cache_fill(const FillParams &p, hipStream_t st)
 {
     if (p.n_seqs == 0 || p.n_tokens == 0) return hipSuccess;
-    const int rows_per_block = 256 / (p.head_dim / 16);
-    hipLaunchKernelGGL(cache_fill_kernel, dim3((unsigned)((p.n_tokens + rows_per_block - 1) / rows_per_block), (unsigned)p.n_heads),
-                       dim3(256), 0, st, p);
+    hipLaunchKernelGGL(cache_fill_kernel, dim3((unsigned)((p.n_tokens + FILL_TOKENS - 1) / FILL_TOKENS)), dim3(256), 0, st, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(cache_len_add_kernel, dim3((unsigned)((p.n_seqs + 255) / 256)), dim3(256), 0, st, p.cache_len, p.seq_offset,

@@ -70,6 +70,21 @@ __device__ inline int8_t float_to_i8(float x)
     return (int8_t)(int)r;
 }
 
+// Four floats to four int8 in one word (first value in the low byte): what float_to_i8 gives for each, with the lower
+// bound a parameter (-127, or 0 where negative results are dropped).  Clamping before rounding gives what rounding
+// before clamping gives, the bounds being whole numbers (one median-of-three instruction; a NaN comes out as the lower
+// bound, as it does from fmaxf/fminf); adding 1.5 * 2^23 rounds to nearest even and leaves the whole number, in two's
+// complement, in the low bits of the float.
+__device__ inline uint32_t pack_i8x4(float y0, float y1, float y2, float y3, float low)
+{
+    const uint32_t b0 = __float_as_uint(__builtin_amdgcn_fmed3f(y0, low, 127.0f) + 12582912.0f);
+    const uint32_t b1 = __float_as_uint(__builtin_amdgcn_fmed3f(y1, low, 127.0f) + 12582912.0f);
+    const uint32_t b2 = __float_as_uint(__builtin_amdgcn_fmed3f(y2, low, 127.0f) + 12582912.0f);
+    const uint32_t b3 = __float_as_uint(__builtin_amdgcn_fmed3f(y3, low, 127.0f) + 12582912.0f);
+    // byte 0 of each
+    return __builtin_amdgcn_perm(__builtin_amdgcn_perm(b3, b2, 0x0c0c0400u), __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u), 0x05040100u);
+}
+
 // Butterfly exchange inside a wave through DPP where the pattern allows it.
 template <int CTRL>
 __device__ inline int dpp_mov(int v)

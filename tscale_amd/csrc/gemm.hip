@@ -185,6 +185,9 @@ __global__ __launch_bounds__(GT_THREADS, 2) void gemm_tiled_kernel(GemmParams p)
 constexpr int GW_THREADS = 512, GW_BM = 256, GW_BN = 256, GW_BK = 64, GW_NBUF = 4;
 constexpr int GW_BUF = (GW_BM + GW_BN) * GW_BK;
 constexpr int GW_LDS_BYTES = GW_NBUF * GW_BUF;
+// with the producer as epilogue: the floats of 128 rows (row pitch head width + 4), a multiplier per (row, head), 256 positions
+constexpr int ep_lds_bytes(int head_dim) { return head_dim == 0 ? 0 : (128 * (GW_BN / head_dim) * (head_dim + 4) + 128 * (GW_BN / head_dim) + GW_BM) * 4; }
+constexpr int gw_lds_bytes(int head_dim) { return ep_lds_bytes(head_dim) > GW_LDS_BYTES ? ep_lds_bytes(head_dim) : GW_LDS_BYTES; }
 
 template <int MODE, int EP_D>
 __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
@@ -298,15 +301,18 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
     if constexpr (EP_D != 0) {
         // The producer as the product's epilogue (the reference's projection kernels end the same way,
         // TStoreRowTileNormalizeRope, gpt/compute/gpt_rope.cuh:4-66): the int32 sums never go to memory.  The tile's
-        // 256 columns are whole heads of EP_D; 64 of its rows at a time (block i of both row halves) go through LDS as
-        // floats -- after the residual update and the rotation, which are lane-local: a wave's 64 columns are one
-        // rotation block, x in acc[.][0] and x + 32 in acc[.][1] -- so that one thread per (row, head) can add up the
-        // squares in index order, as the producer kernel and the CPU path do.  Every float operation as written there.
+        // 256 columns are whole heads of EP_D; 128 of its rows at a time (blocks 2 s and 2 s + 1 of both row halves) go
+        // through LDS as floats -- after the residual update or the rotation, which are lane-local: a wave's 64 columns
+        // are one rotation block, x in acc[.][0] and x + 32 in acc[.][1] -- so that one thread per (row, head) can add up
+        // the squares in index order, as the producer kernel and the CPU path do (that chain of additions is the longest
+        // wait of the epilogue: the more pairs a step has, the more threads walk their chains side by side).  Every
+        // float operation as written there.  A residual update and a rotation in one call are left to the producer
+        // kernel by the launcher.
 #pragma clang fp contract(off)
         constexpr int HEADS_T = GW_BN / EP_D;  // heads per tile
-        constexpr int PAIRS = 64 * HEADS_T;    // (row, head) pairs per block of rows
+        constexpr int PAIRS = 128 * HEADS_T;   // (row, head) pairs per step
         constexpr int PITCH = EP_D + 4;        // rows 16 bytes aligned, 16 lanes' 16-byte reads on 64 different banks
-        static_assert((PAIRS * PITCH + PAIRS + GW_BM) * 4 <= GW_LDS_BYTES && PAIRS <= GW_THREADS, "the epilogue's LDS and threads");
+        static_assert(ep_lds_bytes(EP_D) == (PAIRS * PITCH + PAIRS + GW_BM) * 4 && PAIRS <= GW_THREADS, "the epilogue's LDS and threads");
         float *const vals = (float *)gw_lds;
         float *const mults = vals + PAIRS * PITCH;
         int *const tile_pos = (int *)(mults + PAIRS); // positions of the tile's 256 rows
@@ -327,63 +333,67 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
         const uint32_t resid_pitch_bytes = (uint32_t)e.resid_pitch * 4u;
         // Everything a block of rows needs from memory is requested before any of it is used or stored (row by row, each
         // row's stores would have to be waited for before the next row's loads, which they might overlap), and the next
-        // block's requests go out before this block's sums and conversion, which they pass under.
-        float cs[16], sn[16], u0[16], u1[16];
-        auto request = [&](int i) __attribute__((always_inline)) {
-            if (rotate) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const uint32_t t = (uint32_t)tile_pos[wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3)];
-                    const float *const rope_row = (const float *)(rope_base + (t * (uint32_t)(EP_D * 4) + (uint32_t)li * 4u));
-                    cs[r] = rope_row[0];
-                    sn[r] = rope_row[32];
-                }
-            }
+        // step's requests go out before this step's sums and conversion, which they pass under.  Per block two values
+        // per row and lane: the old state's, or cos and sin.
+        float xa[2][16], xb[2][16];
+        auto request = [&](int i, int set) __attribute__((always_inline)) {
             if (e.resid) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int row = wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
                     const bool ok = row < rows_here && head_ok;
                     const float *const q0 = (const float *)(resid_base + ((uint32_t)row * resid_pitch_bytes + (uint32_t)li * 4u));
-                    u0[r] = ok ? q0[0] : 0.0f;
-                    u1[r] = ok ? q0[32] : 0.0f;
+                    xa[set][r] = ok ? q0[0] : 0.0f;
+                    xb[set][r] = ok ? q0[32] : 0.0f;
+                }
+            } else if (rotate) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const uint32_t t = (uint32_t)tile_pos[wm * 128 + i * 32 + 8 * (r / 4) + 4 * g + (r & 3)];
+                    const float *const rope_row = (const float *)(rope_base + (t * (uint32_t)(EP_D * 4) + (uint32_t)li * 4u));
+                    xa[set][r] = rope_row[0];
+                    xb[set][r] = rope_row[32];
                 }
             }
         };
-        request(0);
+        request(0, 0);
+        request(1, 1);
 #pragma unroll // (the accumulators are registers: no run-time index into them)
-        for (int i = 0; i < 4; ++i) {
+        for (int s = 0; s < 2; ++s) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int rr = 8 * (r / 4) + 4 * g + (r & 3);
-                const int row = wm * 128 + i * 32 + rr;
-                float v0 = (float)acc[i][0][r], v1 = (float)acc[i][1][r];
-                if (e.resid) { // state += delta * scale, written back; the updated state is what gets normalised
-                    v0 = u0[r] + v0 * e.resid_scale;
-                    v1 = u1[r] + v1 * e.resid_scale;
-                    if (row < rows_here && head_ok) {
-                        float *const q0 = (float *)(resid_base + ((uint32_t)row * resid_pitch_bytes + (uint32_t)li * 4u));
-                        q0[0] = v0;
-                        q0[32] = v1;
-                    }
+            for (int b = 0; b < 2; ++b) {
+                const int i = 2 * s + b;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int rr = 8 * (r / 4) + 4 * g + (r & 3);
+                    const int row = wm * 128 + i * 32 + rr;
+                    float v0 = (float)acc[i][0][r], v1 = (float)acc[i][1][r];
+                    if (e.resid) { // state += delta * scale, written back; the updated state is what gets normalised
+                        v0 = xa[b][r] + v0 * e.resid_scale;
+                        v1 = xb[b][r] + v1 * e.resid_scale;
+                        if (row < rows_here && head_ok) {
+                            float *const q0 = (float *)(resid_base + ((uint32_t)row * resid_pitch_bytes + (uint32_t)li * 4u));
+                            q0[0] = v0;
+                            q0[32] = v1;
+                        }
+                    } else if (rotate) {
+                        const float cos_value = xa[b][r];
+                        const float sin_value = xb[b][r] * e.rotate_dir;
+                        const float r0 = v0 * cos_value - v1 * sin_value;
+                        const float r1 = v0 * sin_value + v1 * cos_value;
+                        v0 = r0;
+                        v1 = r1;
+                    } // (a head that is not rotated: cos 1 and sin 0 leave the values as they are)
+                    float *const dst = vals + ((b * 64 + wm * 32 + rr) * HEADS_T + head_t) * PITCH + xbase + li;
+                    dst[0] = v0;
+                    dst[32] = v1;
                 }
-                if (rotate) {
-                    const float cos_value = cs[r];
-                    const float sin_value = sn[r] * e.rotate_dir;
-                    const float r0 = v0 * cos_value - v1 * sin_value;
-                    const float r1 = v0 * sin_value + v1 * cos_value;
-                    v0 = r0;
-                    v1 = r1;
-                } // (a head that is not rotated: cos 1 and sin 0 leave the values as they are)
-                float *const dst = vals + ((wm * 32 + rr) * HEADS_T + head_t) * PITCH + xbase + li;
-                dst[0] = v0;
-                dst[32] = v1;
+                if (s == 0) request(2 + b, b);
             }
-            if (i + 1 < 4) request(i + 1);
             __syncthreads();
             if (tid < PAIRS) { // sum of squares in index order, scale
                 const int rc = tid / HEADS_T, ht = tid % HEADS_T;
-                const int64_t m = m0 + (rc / 32) * 128 + i * 32 + (rc % 32);
+                const int64_t m = m0 + ((rc % 64) / 32) * 128 + (2 * s + rc / 64) * 32 + (rc % 32);
                 const int hd = (int)(n0 / EP_D) + ht;
                 const float *const v = vals + tid * PITCH;
                 float sum2 = 0.0f;
@@ -412,9 +422,7 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
                     e.scale[sh * e.scale_pitch + m * e.scale_row_stride] = discr * e.scale_mult;
             }
             __syncthreads();
-            // Convert and store, 16 bytes per thread and step.  Clamping before rounding gives what rounding before
-            // clamping gives (the bounds are whole numbers); adding 1.5 * 2^23 rounds to nearest even and leaves the whole
-            // number, in two's complement, in the low bits of the float.  A head of zeros has mult 0: zero bytes.
+            // Convert and store, 16 bytes per thread and step.  A head of zeros has mult 0: zero bytes.
             constexpr int OUT_PER_PAIR = EP_D / 16;
             static_assert((PAIRS * OUT_PER_PAIR) % GW_THREADS == 0, "whole steps of the workgroup");
             const float low = e.relu ? 0.0f : -127.0f;
@@ -424,24 +432,18 @@ __global__ __launch_bounds__(GW_THREADS, 1) void gemm_wide_kernel(GemmParams p)
                 const int j = j0 + tid;
                 const int pr = j / OUT_PER_PAIR, x = (j % OUT_PER_PAIR) * 16;
                 const int rc = pr / HEADS_T, ht = pr % HEADS_T;
-                const int row = (rc / 32) * 128 + i * 32 + (rc % 32);
+                const int row = ((rc % 64) / 32) * 128 + (2 * s + rc / 64) * 32 + (rc % 32);
                 const float mult = mults[pr];
                 v4f q[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) q[k] = *(const v4f *)(vals + pr * PITCH + x + 4 * k);
                 uint32_t w[4];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    uint32_t b[4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) b[u] = __float_as_uint(fminf(fmaxf(q[k][u] * mult, low), 127.0f) + 12582912.0f);
-                    // byte 0 of each of the four
-                    w[k] = __builtin_amdgcn_perm(__builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u), __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u), 0x05040100u);
-                }
+                for (int k = 0; k < 4; ++k) w[k] = pack_i8x4(q[k].x * mult, q[k].y * mult, q[k].z * mult, q[k].w * mult, low);
                 if (row < rows_here && (int)(n0 / EP_D) + ht < e.n_heads)
                     *(v4i *)(dst_base + ((uint32_t)row * (uint32_t)e.dst_pitch + (uint32_t)(ht * EP_D + x))) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
             }
-            __syncthreads(); // before the next block of rows overwrites the values
+            __syncthreads(); // before the next step overwrites the values
         }
     } else if constexpr (MODE == TSATTN_MM_ADD_SCALED) {
         // state += sum * scale: the 32 old values of a block of rows are requested together, then updated and stored
@@ -631,11 +633,16 @@ int split_for(const GemmParams &p, int64_t room_bytes)
 // Once per device, before the first product: the wide-tile kernels use more LDS than a launch may ask for by default.
 hipError_t prepare_matmul_i8()
 {
-    const void *kernels[] = {(const void *)gemm_wide_kernel<TSATTN_MM_I32, 0>, (const void *)gemm_wide_kernel<TSATTN_MM_F32, 0>,
-                             (const void *)gemm_wide_kernel<TSATTN_MM_ADD_SCALED, 0>, (const void *)gemm_wide_kernel<TSATTN_MM_I32, 64>,
-                             (const void *)gemm_wide_kernel<TSATTN_MM_I32, 128>};
-    for (const void *k : kernels) {
-        const hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS_BYTES);
+    const struct {
+        const void *kernel;
+        int lds;
+    } kernels[] = {{(const void *)gemm_wide_kernel<TSATTN_MM_I32, 0>, gw_lds_bytes(0)},
+                   {(const void *)gemm_wide_kernel<TSATTN_MM_F32, 0>, gw_lds_bytes(0)},
+                   {(const void *)gemm_wide_kernel<TSATTN_MM_ADD_SCALED, 0>, gw_lds_bytes(0)},
+                   {(const void *)gemm_wide_kernel<TSATTN_MM_I32, 64>, gw_lds_bytes(64)},
+                   {(const void *)gemm_wide_kernel<TSATTN_MM_I32, 128>, gw_lds_bytes(128)}};
+    for (const auto &k : kernels) {
+        const hipError_t e = hipFuncSetAttribute(k.kernel, hipFuncAttributeMaxDynamicSharedMemorySize, k.lds);
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -661,9 +668,10 @@ hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out
             // (the epilogue addresses a tile's rows with 32-bit offsets)
             const bool offsets_fit = q.ep.dst_pitch < (1 << 23) && (!q.ep.resid || q.ep.resid_pitch < (1 << 21)) &&
                                      (!q.ep.pos || q.ep.rope_len * p.ep_head_dim * 4 < ((int64_t)1 << 31));
-            if (p.m > 32 * GS_MB && wide >= 512 && p.ep_dst_dtype == TSATTN_I8 && offsets_fit) {
-                if (p.ep_head_dim == 128) hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 128>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, q);
-                else hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 64>), dim3((unsigned)wide), dim3(GW_THREADS), GW_LDS_BYTES, st, q);
+            const bool one_operand = !(q.ep.resid && q.ep.pos); // (registers for the old state or for cos and sin)
+            if (p.m > 32 * GS_MB && wide >= 512 && p.ep_dst_dtype == TSATTN_I8 && offsets_fit && one_operand) {
+                if (p.ep_head_dim == 128) hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 128>), dim3((unsigned)wide), dim3(GW_THREADS), gw_lds_bytes(128), st, q);
+                else hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 64>), dim3((unsigned)wide), dim3(GW_THREADS), gw_lds_bytes(64), st, q);
                 return hipGetLastError();
             }
             if (split == 1) launch_mode<TSATTN_MM_I32>(q, st);

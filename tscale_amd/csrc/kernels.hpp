@@ -65,6 +65,13 @@ struct PrefillParams {
     int n_tokens;
     int n_heads;
     int period_tiles; // query tiles per period of equal span structure, 0 = unknown (launch order only)
+    // optional fused consumer (kv_out != nullptr): KVProduct of the f32 result with the rows of kv_k; out may then be null
+    const uint8_t *kv_k;
+    int64_t kv_k_pitch;
+    uint8_t *kv_out;
+    int64_t kv_out_pitch;
+    int kv_rep;
+    float kv_mult;
     WgMap map;        // set by the launcher: how workgroup ids map to (head, query tile)
 };
 

@@ -201,6 +201,8 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
     // the common-tile loop with ALiBi only where it fits into the registers without spilling
     constexpr bool FAST_LOOP = !DUMP && (!SLOPE || (D == 128 && DTYPE == TSATTN_E4M3));
     constexpr int LDS_BYTES = (HAS_SHORT && SHORT_BYTES > LOOP_BYTES) ? SHORT_BYTES : LOOP_BYTES;
+    // the fused KVProduct exists where the reference has one: behind int8 attention with an f32 result (cpu_infer.cpp:509-511)
+    constexpr bool KV_FUSED = DTYPE == TSATTN_I8 && !OUT_F16 && !DUMP;
     __shared__ __attribute__((aligned(16))) uint8_t lds_raw[LDS_BYTES];
     auto k_lds = [&](int b) -> uint8_t * { return lds_raw + b * L::K_BYTES; };
     auto v_lds = [&](int b) -> uint8_t * { return lds_raw + 2 * L::K_BYTES + b * L::V_BYTES; };
@@ -804,7 +806,71 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
     float l_all = l + __shfl_xor(l, 32, WAVE);
     l_all += fast_exp2(-m_ref);
     const float inv = 1.0f / l_all;
-    if (row_ok) {
+    if constexpr (KV_FUSED) if (p.kv_out) {
+        // Fused consumer: KVProduct (gpt/train/cpu_infer.cpp:320-337) of the result, which is in registers, with the
+        // rows of kv_k: kv[head][blk][x] = int8((k[x ^ blk] * value[x]) * mult).  x ^ blk stays inside an aligned group
+        // of four and a lane holds such groups, so the products are lane-local.  The bytes of two blk at a time go
+        // through this wave's corner of LDS (32 rows x D bytes each) so that they leave as whole rows of D bytes,
+        // 16 bytes per lane.
+        constexpr int KV_PITCH = D + 16;
+        static_assert(PF_WAVES * 2 * 32 * KV_PITCH <= LDS_BYTES, "the KVProduct rows of all waves fit into the tiles' LDS");
+        __syncthreads(); // every wave is done with the K and V tiles
+        // (what follows is computed from these copies, which the compiler cannot trace back: nothing of it is
+        // prepared before the tile loop and kept in registers through it)
+        int qi = lane & 31, g = lane >> 5, q0 = tile * PF_BM + wave * 32;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "+v"(qi), "+v"(g), "+v"(q0));
+#endif
+        const int from = q0 + qi;
+        const bool row_ok = from < p.n_tokens;
+        uint8_t *const stage = lds_raw + (q0 / 32 % PF_WAVES) * (2 * 32 * KV_PITCH);
+        uint32_t kw[DT][4];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4)
+                kw[dt][c4] = row_ok ? *(const uint32_t *)(p.kv_k + (int64_t)from * p.kv_k_pitch + hoff + dt * 32 + 8 * c4 + 4 * g) : 0u;
+        for (int hb = 0; 2 * hb < p.kv_rep; ++hb) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                for (int c4 = 0; c4 < 4; ++c4) {
+                    float o[4], key[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        o[j] = o_acc[dt][c4 * 4 + j] * inv;
+                        key[j] = (float)(int8_t)((kw[dt][c4] >> (8 * j)) & 0xff);
+                    }
+#pragma unroll
+                    for (int bb = 0; bb < 2; ++bb) {
+                        const int blk = 2 * hb + bb; // (x ^ blk) % 4 = j ^ bb ^ 2 hb
+                        const float *const kx = key;
+                        const int s0 = (0 ^ bb), s1 = (1 ^ bb), s2 = (2 ^ bb), s3 = (3 ^ bb);
+                        uint32_t word;
+                        if (hb == 0)
+                            word = pack_i8x4((kx[s0] * o[0]) * p.kv_mult, (kx[s1] * o[1]) * p.kv_mult, (kx[s2] * o[2]) * p.kv_mult,
+                                             (kx[s3] * o[3]) * p.kv_mult, -127.0f);
+                        else
+                            word = pack_i8x4((kx[s0 ^ 2] * o[0]) * p.kv_mult, (kx[s1 ^ 2] * o[1]) * p.kv_mult, (kx[s2 ^ 2] * o[2]) * p.kv_mult,
+                                             (kx[s3 ^ 2] * o[3]) * p.kv_mult, -127.0f);
+                        if (blk < p.kv_rep) *(uint32_t *)(stage + (bb * 32 + qi) * KV_PITCH + dt * 32 + 8 * c4 + 4 * g) = word;
+                    }
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's bytes are in LDS (nobody else reads them)
+#pragma unroll
+            for (int it = 0; it < 2 * 32 * CHUNKS / WAVE; ++it) {
+                const int id = it * WAVE + g * 32 + qi;
+                const int c = id % CHUNKS, r = (id / CHUNKS) % 32, bb = id / (CHUNKS * 32);
+                const int blk = 2 * hb + bb;
+                const v4i w = *(const v4i *)(stage + (bb * 32 + r) * KV_PITCH + c * 16);
+                if (q0 + r < p.n_tokens && blk < p.kv_rep)
+                    *(v4i *)(p.kv_out + (int64_t)(q0 + r) * p.kv_out_pitch + ((int64_t)head * p.kv_rep + blk) * D + c * 16) = w;
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read before the next two blk overwrite it
+        }
+    }
+    if (row_ok && p.out) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -820,10 +886,8 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
                 }
             }
         }
-        if (p.sum_weight_log && g == 0) {
-            p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m_ref + __log2f(l_all);
-        }
     }
+    if (row_ok && p.sum_weight_log && g == 0) p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m_ref + __log2f(l_all);
 }
 
 template <int DTYPE, int D, bool OUT_F16>

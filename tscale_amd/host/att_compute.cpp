@@ -473,7 +473,10 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
     pa.scale_pitch = len;
     pa.span_start = spanStart; pa.span_finish = spanFinish; pa.span_tiles = spanTiles; pa.causal_period = causalPeriod;
     pa.alibi_slope = att.AlibiSlope;
-    pa.out = ValLookup; pa.out_pitch = (int64_t)qsum * 4;
+    pa.out = WriteValLookup ? ValLookup : nullptr; pa.out_pitch = (int64_t)qsum * 4;
+    // KVProduct (cpu_infer.cpp:511) as the attention kernel's last step
+    pa.kv_k = Q4 + 2 * (size_t)qsum; pa.kv_k_pitch = pitch4; pa.kv_out = Kv; pa.kv_out_pitch = (int64_t)qsum * COMBINER_REP;
+    pa.kv_rep = COMBINER_REP; pa.kv_mult = 1.0f;
     Check(tsattn_prefill(Handle, &pa, stream), "tsattn_prefill");
     // kvCache.AddVectors for every token at once
     tsattn_fill_args fa = {};
@@ -488,7 +491,7 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
     fa.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; fa.s_head_stride = kvCache.MaxLen;
     fa.cache_len = kvCache.Length; fa.max_len = kvCache.MaxLen;
     Check(tsattn_cache_fill(Handle, &fa, stream), "tsattn_cache_fill");
-    AfterAttention(len, att, false, deferStateUpdate, state, stream);
+    AfterAttention(len, att, true, deferStateUpdate, state, stream);
 }
 
 void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const std::vector<TAttentionVecHistory *> &kvCaches,

@@ -207,6 +207,9 @@ class TLayerComputer
                                 const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
                                 void *stream, bool deferStateUpdate = false);
     const float *GetValLookup() const { return ValLookup; } // [rows][HeadCount*TTDim] of the last call
+    // false: AddLookupProductPrompt does not write the attention output (its KVProduct, made by the same kernel, is all
+    // the layer reads); GetValLookup() is then stale after that call
+    bool WriteValLookup = true;
 };
 
 // The model around the layers: TCPUModelParams of the reference (gpt/train/cpu_infer.cpp:58-86), device copies.
