@@ -360,12 +360,12 @@ class Int8Layers:
     MODEL_DISCR_SCALE = 1/32), one KV cache per layer for B = 32 sequences.  Embedding, final layer and sampling are
     not part of it."""
 
-    def __init__(self, ctx, cache_len, seed):
+    def __init__(self, ctx, cache_len, seed, n_new=64):
         import torch
         from tscale_amd import KVCache, capi
         from tscale_amd.attention import alibi_layer_schedule, VEC_SCALE
         self.ctx = ctx
-        self.B, self.H, self.d, self.dim, self.depth, self.prompt, self.n_new = 32, 16, 128, 2048, 24, 2048, 64
+        self.B, self.H, self.d, self.dim, self.depth, self.prompt, self.n_new = 32, 16, 128, 2048, 24, 2048, n_new
         self.L = self.prompt + self.n_new
         qsum = self.H * self.d
         g = torch.Generator(device="cuda").manual_seed(seed)
@@ -485,6 +485,97 @@ def bench_generate_model(ctx, steps):
             "weight_bytes": m.weight_bytes + head_bytes, "choices_changed": bool((labels != first).any())}
 
 
+def bench_prompt_then_generate(ctx, n_new=256):
+    """The whole of the last configuration in one timed region: 32 prompts of 2048 random token ids (uniform over the
+    vocabulary) through the embedding and the 24 layers in batch form, the final layer on each prompt's last token,
+    then greedy generation of n_new tokens, one HIP graph replay per token (recorded beforehand, outside the timed
+    region).  Nothing is reused between the phases but the KV caches the prompt pass filled."""
+    import numpy as np
+    import torch
+    from tscale_amd import capi
+    from tscale_amd.attention import add_lookup_product, add_lookup_product_prompt, flush_state, VEC_SCALE
+    m = Int8Layers(ctx, cache_len=0, seed=1313 + 12, n_new=n_new)
+    B, H, d, dim, qsum = m.B, m.H, m.d, m.dim, m.H * m.d
+    vocab = 50257
+    def matrix(n, k):
+        return (torch.randn((n, k), device="cuda", generator=m.g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
+    embed, final = matrix(vocab, dim), matrix(vocab, dim)
+    bias = torch.randn(vocab, device="cuda", generator=m.g) * 0.1
+    f32 = np.float32
+    final_scale = float(f32(np.sqrt(f32(1.0) / f32(dim))) * (f32(1.0) / f32(0.693147)) * f32(0.03) * f32(VEC_SCALE))
+    n = B * m.prompt
+    ids = torch.randint(0, vocab, (n,), dtype=torch.int32, device="cuda", generator=m.g)
+    off = torch.arange(0, n + 1, m.prompt, dtype=torch.int32, device="cuda")
+    pos = torch.arange(m.prompt, dtype=torch.int32, device="cuda").repeat(B)
+    last = (off[1:] - 1).long()
+    spans = {w: ctx.build_spans(off, n, w) for w in {w for w, _ in m.sched}}
+    tiles = {w: ctx.build_span_tiles(*sp) for w, sp in spans.items()}
+    prompt_state = torch.empty((n, dim), dtype=torch.float32, device="cuda")
+    labels = torch.zeros((B,), dtype=torch.int32, device="cuda")
+    state = torch.empty((B, dim), dtype=torch.float32, device="cuda")
+    t = torch.full((B,), m.prompt, dtype=torch.int32, device="cuda")
+    room = torch.empty(16 * 4 * B * max(dim, qsum), dtype=torch.uint8, device="cuda")
+    planes = torch.empty(16 * B * vocab, dtype=torch.int32, device="cuda")
+    keep = {}
+    def choose(norm):
+        logits = ctx.matmul_i8(norm, final, mode=capi.MM_I32_PLANES, out=planes)
+        ctx.softmax_rows(logits, final_scale, bias, want_prob=False, argmax=labels)
+    def prompt_phase():
+        ctx.embed_rows(ids, embed, 0.03, out=prompt_state)
+        norm = None
+        for layer, c in zip(m.layers, m.caches):
+            w = layer["width"]
+            _, norm = add_lookup_product_prompt(ctx, layer, c, off, pos, m.rope, prompt_state, *spans[w], span_tiles=tiles[w],
+                                                causal_period=m.prompt if w >= m.prompt else 0, norm=norm, want_norm=True,
+                                                want_val=False)
+        choose(norm[last].contiguous())   # NormalizeState of each prompt's last token, made by the last product
+    def step():
+        ctx.embed_rows(labels, embed, 0.03, out=state)
+        pending = None
+        for layer, c in zip(m.layers, m.caches):
+            _, pending = add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep, pending=pending, defer=True)
+        choose(flush_state(ctx, pending, state))
+        t.add_(1)
+    def rewind():
+        for c in m.caches:
+            c.cache_len.zero_()
+        t.fill_(m.prompt)
+    # once untimed: the prompt (so that a step sees caches of the right length), a step eagerly, the graph of a step
+    prompt_phase()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    torch.cuda.synchronize()
+    rewind()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+    torch.cuda.synchronize()
+    ev[0].record()
+    prompt_phase()
+    ev[1].record()
+    chosen = [labels.clone()]
+    for _ in range(n_new - 1):
+        graph.replay()
+        chosen.append(labels.clone())
+    ev[2].record()
+    torch.cuda.synchronize()
+    ms_prompt, ms_gen = ev[0].elapsed_time(ev[1]), ev[1].elapsed_time(ev[2])
+    chosen = torch.stack(chosen)
+    assert int(m.caches[0].cache_len[0]) == m.prompt + n_new - 1 and int(chosen.min()) >= 0 and int(chosen.max()) < vocab
+    assert bool(torch.isfinite(state).all())
+    return {"config": "B32: 2048-token prompts (random ids over 50257) through embedding + 24 int8 layers + final layer, then greedy "
+                      "generation of %d tokens (the first from the prompt pass, the others one HIP graph replay each); int8 KV cache" % n_new,
+            "ms_total": round(ms_prompt + ms_gen, 2), "ms_prompt_to_first_token": round(ms_prompt, 2),
+            "ms_per_generated_token": round(ms_gen / (n_new - 1), 4),
+            "generated_tokens_per_s": round(B * n_new / (ms_prompt + ms_gen) * 1e3, 1),
+            "distinct_tokens_chosen": int(torch.unique(chosen).numel())}
+
+
 def bench_prompt_pass(ctx, steps):
     """The prompt of the same configuration through the same 24 layers in batch form (add_lookup_product_prompt):
     32 x 2048 tokens, per layer one prefill attention launch, one cache fill, seven matrix products in four calls, each
@@ -600,6 +691,9 @@ def run_only(ctx, args):
     if name == "prompt-pass":
         print(json.dumps({"only": name, **bench_prompt_pass(ctx, args.steps)}))
         return
+    if name == "prompt-then-generate":
+        print(json.dumps({"only": name, **bench_prompt_then_generate(ctx)}))
+        return
     if name == "token-step":
         print(json.dumps({"only": name, **bench_token_step(ctx, args.steps)}))
         return
@@ -637,7 +731,7 @@ def main():
     ap.add_argument("--extra", action="store_true",
                     help="also time the 1.5B-style prefill shapes and the attention share of the 1.5B-style generation run")
     ap.add_argument("--only", default=None,
-                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step", "prompt-pass", "generate-model"],
+                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step", "prompt-pass", "generate-model", "prompt-then-generate"],
                     help="profiling aid: run just this launch --steps times and print its timing")
     ap.add_argument("--calibrate", action="store_true",
                     help="with --only: first run three 256 MiB device copies (counter calibration)")
@@ -726,6 +820,8 @@ def main():
         result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
         result["prompt_pass_24_layers"] = bench_prompt_pass(ctx, args.steps)
         result["generate_whole_model"] = bench_generate_model(ctx, args.steps)
+        torch.cuda.empty_cache()
+        result["prompt_then_generate_256"] = bench_prompt_then_generate(ctx)
     print(json.dumps(result))
 
 
