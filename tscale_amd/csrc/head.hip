@@ -38,8 +38,10 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(HeadParams p)
 
 // One workgroup per row.  w[k] = vec[k] * scale + bias[k]; M = max(0, max w) (the buffer's maximum starts at 0,
 // cpu_infer.cpp:226-244); p[k] = 2^(w[k] - M) / sum (base 2: the scale carries 1/ln 2).  The choice is the first k of
-// the largest w.
-constexpr int SM_THREADS = 256;
+// the largest w.  A row is 200 KB of sums and as much bias for one workgroup: 1024 threads, eight independent
+// requests per thread and round, so that a pass is a handful of memory round trips and not two hundred.
+constexpr int SM_THREADS = 1024;
+constexpr int SM_U = 8;
 
 __device__ inline float softmax_logit(const HeadParams &p, int64_t row, int64_t k)
 {
@@ -59,9 +61,16 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
     // pass 1: maximum and where it is first reached
     float best = -INFINITY;
     int arg = 0x7fffffff;
-    for (int64_t k = tid; k < p.n; k += SM_THREADS) {
-        const float w = softmax_logit(p, row, k);
-        if (w > best) { best = w; arg = (int)k; }
+    for (int64_t k0 = tid; k0 < p.n; k0 += SM_U * SM_THREADS) {
+        float w[SM_U];
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = k0 + u * SM_THREADS;
+            w[u] = k < p.n ? softmax_logit(p, row, k) : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) // (ascending k: the first of equal values stays)
+            if (w[u] > best) { best = w[u]; arg = (int)(k0 + u * SM_THREADS); }
     }
     for (int o = 32; o > 0; o >>= 1) {
         const float ob = __shfl_xor(best, o, WAVE);
@@ -79,7 +88,17 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
     const float M = fmaxf(0.0f, best);
     // pass 2: sum of the weights
     float sum = 0.0f;
-    for (int64_t k = tid; k < p.n; k += SM_THREADS) sum += fast_exp2(fmaxf(softmax_logit(p, row, k) - M, -127.0f));
+    for (int64_t k0 = tid; k0 < p.n; k0 += SM_U * SM_THREADS) {
+        float w[SM_U];
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = k0 + u * SM_THREADS;
+            w[u] = k < p.n ? softmax_logit(p, row, k) : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u)
+            if (k0 + u * SM_THREADS < p.n) sum += fast_exp2(fmaxf(w[u] - M, -127.0f));
+    }
     for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, WAVE);
     if (lane == 0) s_sum[wave] = sum;
     __syncthreads();
@@ -87,7 +106,19 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
     for (int w = 0; w < SM_THREADS / WAVE; ++w) sum += s_sum[w];
     const float inv = 1.0f / sum;
     // pass 3: the probabilities
-    for (int64_t k = tid; k < p.n; k += SM_THREADS) p.prob[row * p.prob_pitch + k] = fast_exp2(fmaxf(softmax_logit(p, row, k) - M, -127.0f)) * inv;
+    for (int64_t k0 = tid; k0 < p.n; k0 += SM_U * SM_THREADS) {
+        float w[SM_U];
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = k0 + u * SM_THREADS;
+            w[u] = k < p.n ? softmax_logit(p, row, k) : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = k0 + u * SM_THREADS;
+            if (k < p.n) p.prob[row * p.prob_pitch + k] = fast_exp2(fmaxf(w[u] - M, -127.0f)) * inv;
+        }
+    }
 }
 
 
