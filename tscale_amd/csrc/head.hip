@@ -38,10 +38,13 @@ __global__ __launch_bounds__(256) void embed_rows_kernel(HeadParams p)
 
 // One workgroup per row.  w[k] = vec[k] * scale + bias[k]; M = max(0, max w) (the buffer's maximum starts at 0,
 // cpu_infer.cpp:226-244); p[k] = 2^(w[k] - M) / sum (base 2: the scale carries 1/ln 2).  The choice is the first k of
-// the largest w.  A row is 200 KB of sums and as much bias for one workgroup: 1024 threads, eight independent
-// requests per thread and round, so that a pass is a handful of memory round trips and not two hundred.
+// the largest w.  A row is 200 KB of sums and as much bias for one CU, and what a CU gets per microsecond is what it
+// has in flight: 1024 threads, four requests of 16 bytes (rows start at any multiple of 4 bytes) per thread and round,
+// so that a pass is two rounds of memory latency and not two hundred.
 constexpr int SM_THREADS = 1024;
-constexpr int SM_U = 8;
+constexpr int SM_U = 4;
+typedef int v4i_any __attribute__((ext_vector_type(4), aligned(4)));
+typedef float v4f_any __attribute__((ext_vector_type(4), aligned(4)));
 
 __device__ inline float softmax_logit(const HeadParams &p, int64_t row, int64_t k)
 {
@@ -51,6 +54,41 @@ __device__ inline float softmax_logit(const HeadParams &p, int64_t row, int64_t 
     return p.bias ? w + p.bias[k] : w;
 }
 
+// the same for k .. k + 3
+__device__ inline v4f softmax_logit4(const HeadParams &p, int64_t row, int64_t k)
+{
+    v4i v = *(const v4i_any *)(p.src + row * p.src_pitch + k);
+    for (int pl = 1; pl < p.src_planes; ++pl) v += *(const v4i_any *)(p.src + pl * p.src_plane_stride + row * p.src_pitch + k);
+    v4f w = v4f{(float)v.x * p.scale, (float)v.y * p.scale, (float)v.z * p.scale, (float)v.w * p.scale};
+    if (p.bias) {
+        const v4f b = *(const v4f_any *)(p.bias + k);
+        w = v4f{w.x + b.x, w.y + b.y, w.z + b.z, w.w + b.w};
+    }
+    return w;
+}
+
+// Walks a row: groups of four from the front, SM_U requests per thread out before the first is used (none under a
+// branch: a group past the end asks for the last whole group again), then the up to three values that are left.
+template <typename F>
+__device__ inline void softmax_walk(const HeadParams &p, int64_t row, int tid, F &&f)
+{
+    const int64_t n4 = p.n & ~(int64_t)3;
+    for (int64_t base = 0; base < n4; base += 4 * SM_THREADS * SM_U) {
+        v4f w[SM_U];
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = base + 4 * (tid + (int64_t)u * SM_THREADS);
+            w[u] = softmax_logit4(p, row, k < n4 ? k : n4 - 4);
+        }
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = base + 4 * (tid + (int64_t)u * SM_THREADS);
+            if (k < n4) { f(k, w[u].x); f(k + 1, w[u].y); f(k + 2, w[u].z); f(k + 3, w[u].w); }
+        }
+    }
+    if (n4 + tid < p.n) f(n4 + tid, softmax_logit(p, row, n4 + tid));
+}
+
 __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
 {
     __shared__ float s_max[SM_THREADS / WAVE];
@@ -58,20 +96,12 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
     __shared__ float s_sum[SM_THREADS / WAVE];
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
-    // pass 1: maximum and where it is first reached
+    // pass 1: maximum and where it is first reached (a thread sees its k in ascending order)
     float best = -INFINITY;
     int arg = 0x7fffffff;
-    for (int64_t k0 = tid; k0 < p.n; k0 += SM_U * SM_THREADS) {
-        float w[SM_U];
-#pragma unroll
-        for (int u = 0; u < SM_U; ++u) {
-            const int64_t k = k0 + u * SM_THREADS;
-            w[u] = k < p.n ? softmax_logit(p, row, k) : -INFINITY;
-        }
-#pragma unroll
-        for (int u = 0; u < SM_U; ++u) // (ascending k: the first of equal values stays)
-            if (w[u] > best) { best = w[u]; arg = (int)(k0 + u * SM_THREADS); }
-    }
+    softmax_walk(p, row, tid, [&](int64_t k, float w) {
+        if (w > best) { best = w; arg = (int)k; }
+    });
     for (int o = 32; o > 0; o >>= 1) {
         const float ob = __shfl_xor(best, o, WAVE);
         const int oa = __shfl_xor(arg, o, WAVE);
@@ -88,17 +118,7 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
     const float M = fmaxf(0.0f, best);
     // pass 2: sum of the weights
     float sum = 0.0f;
-    for (int64_t k0 = tid; k0 < p.n; k0 += SM_U * SM_THREADS) {
-        float w[SM_U];
-#pragma unroll
-        for (int u = 0; u < SM_U; ++u) {
-            const int64_t k = k0 + u * SM_THREADS;
-            w[u] = k < p.n ? softmax_logit(p, row, k) : -INFINITY;
-        }
-#pragma unroll
-        for (int u = 0; u < SM_U; ++u)
-            if (k0 + u * SM_THREADS < p.n) sum += fast_exp2(fmaxf(w[u] - M, -127.0f));
-    }
+    softmax_walk(p, row, tid, [&](int64_t, float w) { sum += fast_exp2(fmaxf(w - M, -127.0f)); });
     for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, WAVE);
     if (lane == 0) s_sum[wave] = sum;
     __syncthreads();
@@ -106,19 +126,8 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(HeadParams p)
     for (int w = 0; w < SM_THREADS / WAVE; ++w) sum += s_sum[w];
     const float inv = 1.0f / sum;
     // pass 3: the probabilities
-    for (int64_t k0 = tid; k0 < p.n; k0 += SM_U * SM_THREADS) {
-        float w[SM_U];
-#pragma unroll
-        for (int u = 0; u < SM_U; ++u) {
-            const int64_t k = k0 + u * SM_THREADS;
-            w[u] = k < p.n ? softmax_logit(p, row, k) : -INFINITY;
-        }
-#pragma unroll
-        for (int u = 0; u < SM_U; ++u) {
-            const int64_t k = k0 + u * SM_THREADS;
-            if (k < p.n) p.prob[row * p.prob_pitch + k] = fast_exp2(fmaxf(w[u] - M, -127.0f)) * inv;
-        }
-    }
+    float *const prob = p.prob + row * p.prob_pitch;
+    softmax_walk(p, row, tid, [&](int64_t k, float w) { prob[k] = fast_exp2(fmaxf(w - M, -127.0f)) * inv; });
 }
 
 
