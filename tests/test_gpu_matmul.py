@@ -112,6 +112,7 @@ def test_matmul_planes_sum_to_the_product(ctx, m, n, k):
 @pytest.mark.parametrize("m,n,k,d,variant", [
     (4096, 8192, 256, 128, "rope"), (8192, 4096, 128, 128, "resid"), (4100, 8192, 192, 64, "rope"), (16384, 2048, 64, 128, "relu"),
     (8000, 4224, 128, 64, "resid"),                                       # the product's kernel normalises its own tiles
+    (4096, 8192, 128, 128, "both"),                                       # rotation and residual update: two launches again
     (300, 512, 256, 128, "rope"), (32, 2048, 1024, 128, "resid"), (5, 256, 128, 64, "relu"),   # two launches
 ])
 def test_matmul_with_the_producer_as_its_epilogue(ctx, m, n, k, d, variant):
@@ -121,23 +122,23 @@ def test_matmul_with_the_producer_as_its_epilogue(ctx, m, n, k, d, variant):
     H = n // d
     a, w = dev(rand_i8(rng, (m, k)).view(np.uint8)), dev(rand_i8(rng, (n, k)).view(np.uint8))
     kw = {}
-    if variant == "rope":
+    if variant in ("rope", "both"):
         rope = dev(orc.fill_rope(d, 64))
         pos = dev(rng.integers(-1, 70, m).astype(np.int32))              # out-of-table positions are clamped
         kw = dict(pos=pos, rope=rope, scale_mult=0.37, rope_heads=max(1, H // 2), scale_heads=(H // 4, max(1, H // 4)))
     elif variant == "relu":
         kw = dict(relu=True, row_major_scale=True)
     resid0 = rng.standard_normal((m, n)).astype(np.float32)
-    if variant == "resid":
+    if variant in ("resid", "both"):
         r1, r2 = dev(resid0), dev(resid0)
-        kw = dict(resid=r1, resid_scale=0.011)
+        kw = dict(kw, resid=r1, resid_scale=0.011)
     got_q, got_s = ctx.matmul_normalize(a, w, H, capi.I8, **kw)
     sums = ctx.matmul_i8(a, w, mode=capi.MM_I32_PLANES)
-    if variant == "resid":
-        kw = dict(resid=r2, resid_scale=0.011)
+    if variant in ("resid", "both"):
+        kw = dict(kw, resid=r2, resid_scale=0.011)
     want_q, want_s = ctx.rope_normalize_rows(sums, H, capi.I8, **kw)
     torch.cuda.synchronize()
     assert torch.equal(got_q, want_q)
     assert torch.equal(got_s, want_s)
-    if variant == "resid":
+    if variant in ("resid", "both"):
         assert torch.equal(r1, r2)
