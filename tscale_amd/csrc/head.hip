@@ -152,11 +152,39 @@ __global__ __launch_bounds__(SM_THREADS) void sample_rows_kernel(HeadParams p)
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     float best = -1e38f;
     int arg = 0x7fffffff;
-    for (int64_t k = tid; k < p.n; k += SM_THREADS) {
-        const uint32_t r = p.rnd ? p.rnd[row * p.rnd_pitch + k] : mix32(p.seed, p.offset + (uint64_t)(row * p.n + k));
+    auto take = [&](int64_t k, float prob, uint32_t r) {
         const double u = ((double)r + 0.5) * (1.0 / 4294967296.0);
-        const float score = (float)((double)(logf(p.prob[row * p.prob_pitch + k]) / p.temperature) - log(-log(u)));
+        const float score = (float)((double)(logf(prob) / p.temperature) - log(-log(u)));
         if (score > best) { best = score; arg = (int)k; }
+    };
+    // groups of four from the front (16-byte requests, all of a round out before the first is used; a thread sees its k
+    // in ascending order), then the up to three values that are left
+    const float *const prob = p.prob + row * p.prob_pitch;
+    const uint32_t *const rnd = p.rnd ? p.rnd + row * p.rnd_pitch : nullptr;
+    const int64_t n4 = p.n & ~(int64_t)3;
+    for (int64_t base = 0; base < n4; base += 4 * SM_THREADS * SM_U) {
+        v4f q[SM_U];
+        v4i r[SM_U];
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = base + 4 * (tid + (int64_t)u * SM_THREADS), kc = k < n4 ? k : n4 - 4;
+            q[u] = *(const v4f_any *)(prob + kc);
+            r[u] = rnd ? (v4i)*(const v4i_any *)(rnd + kc) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < SM_U; ++u) {
+            const int64_t k = base + 4 * (tid + (int64_t)u * SM_THREADS);
+            if (k >= n4) continue;
+            const float qq[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+            const int rr[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                take(k + j, qq[j], rnd ? (uint32_t)rr[j] : mix32(p.seed, p.offset + (uint64_t)(row * p.n + k + j)));
+        }
+    }
+    if (n4 + tid < p.n) {
+        const int64_t k = n4 + tid;
+        take(k, prob[k], rnd ? rnd[k] : mix32(p.seed, p.offset + (uint64_t)(row * p.n + k)));
     }
     for (int o = 32; o > 0; o >>= 1) {
         const float ob = __shfl_xor(best, o, WAVE);
