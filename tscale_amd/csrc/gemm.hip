@@ -530,15 +530,21 @@ __global__ __launch_bounds__(GS_THREADS) void gemm_skinny_kernel(GemmParams p)
 #pragma unroll
     for (int j = 0; j < GS_MB; ++j) acc[j] = v16i{0};
 
-    for (int kb = k_begin; kb < k_end; kb += GS_SLAB) {
-        const int slab = min(GS_SLAB, k_end - kb); // bytes of K in this slab, a multiple of 64
-        const bool in_slab = 16 * lane < slab;
-        v4i rw[GS_LD];
+    // the weights of a slab are requested while the slab before it is being multiplied
+    auto request_w = [&](int kb, v4i (&dst)[GS_LD]) __attribute__((always_inline)) {
+        const bool in_slab = 16 * lane < min(GS_SLAB, k_end - kb);
 #pragma unroll
         for (int i = 0; i < GS_LD; ++i) {
             const int row = 4 * i + wave;
-            rw[i] = in_slab ? __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, row * (int)p.w_pitch + 16 * lane, kb, 0)) : v4i{0, 0, 0, 0};
+            dst[i] = in_slab ? __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, row * (int)p.w_pitch + 16 * lane, kb, 0)) : v4i{0, 0, 0, 0};
         }
+    };
+    v4i rw[GS_LD], rw_next[GS_LD];
+    if (k_begin < k_end) request_w(k_begin, rw);
+    for (int kb = k_begin; kb < k_end; kb += GS_SLAB) {
+        const int slab = min(GS_SLAB, k_end - kb); // bytes of K in this slab, a multiple of 64
+        const bool in_slab = 16 * lane < slab;
+        const bool more = kb + GS_SLAB < k_end;
 #pragma unroll
         for (int j = 0; j < GS_MB; ++j) {
             if (j < n_mb) { // uniform
@@ -548,6 +554,7 @@ __global__ __launch_bounds__(GS_THREADS) void gemm_skinny_kernel(GemmParams p)
                     const int row = 32 * j + 4 * i + wave;
                     rx[i] = in_slab ? __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ar, row * (int)p.a_pitch + 16 * lane, kb, 0)) : v4i{0, 0, 0, 0};
                 }
+                if (j == 0 && more) request_w(kb + GS_SLAB, rw_next);
                 __syncthreads(); // the previous block's reads of x_lds (and, for j == 0, of w_lds) are done
                 if (j == 0) {
 #pragma unroll
@@ -569,6 +576,10 @@ __global__ __launch_bounds__(GS_THREADS) void gemm_skinny_kernel(GemmParams p)
                     }
                 }
             }
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < GS_LD; ++i) rw[i] = rw_next[i];
         }
     }
     // sum the waves' shares in LDS; register r of block j: weight row n0 + 8*(r/4) + 4*g + r%4, activation row 32*j + li
