@@ -45,13 +45,15 @@
  *   tso_matmul_i8          train/cpu_infer.cpp:294-316   pinned: numpy int64 matrix product (a library routine), +-127
  *                                                         extremes; the scaled forms against the same product in
  *                                                         float64
- *   tso_add_lookup_product train/cpu_infer.cpp:465-527   a composition of the functions above in the reference's order;
- *                                                         pinned as a whole only by invariants (the input state's
- *                                                         scale does not matter to the attention half, zero combiner and contract matrices
- *                                                         leave the state alone, the first token sees no keys, the
- *                                                         update is linear in the two matrix scales): the order of
- *                                                         the steps and which scale goes where were checked by
- *                                                         reading -- parity unpinned beyond its parts
+ *   tso_add_lookup_product train/cpu_infer.cpp:465-527   pinned: the same layer in float64 with nothing rounded to
+ *                                                         int8 (division by rms * VEC_SCALE, complex rotation, an
+ *                                                         ordinary softmax with one zero key, real-valued KV cache;
+ *                                                         what the reference's own Check does, :625-685) agrees over
+ *                                                         several tokens to within the int8 rounding, and does not
+ *                                                         with k and v exchanged in KVProduct, the key scale's
+ *                                                         CalcDotScale taken of the head width, a VEC_SCALE dropped,
+ *                                                         or the ReLU in front of the normalisation; plus invariants
+ *                                                         (state scale, zero matrices, first token, linearity)
  *   tso_embed_rows         train/cpu_infer.cpp:559-565   pinned: numpy gather and sum
  *   tso_softmax_rows       train/cpu_infer.cpp:340-355   pinned: scipy's softmax on ln 2 * w (a library routine), rows
  *                                                         sum to 1, adding a constant to the bias changes nothing

@@ -85,3 +85,119 @@ def test_updates_are_linear_in_the_matrix_scales():
     b, _, _ = run(only_ffn, (0.03, 0.0, 0.04), state, [3, 4, 5])
     assert np.abs((b - state) - 2 * (a - state)).max() < 1e-5 * np.abs(a - state).max() + 1e-6
     assert np.abs(a - state).max() > 1e-3
+
+
+# ---- the composition as a whole --------------------------------------------------------------------------------------
+# The reference checks its int8 layer against its real-valued model (NCPUInfer::Check, gpt/train/cpu_infer.cpp:625-685):
+# int8 values times their scales are approximations of real vectors, and every rounding step can be left out.  What
+# follows is that real-valued layer in float64, written from gpt/train/cpu_infer.cpp:465-527 with NormalizeState
+# (:358-391) as a division by rms * VEC_SCALE, ApplyRope (gpt/att/rope.cpp:28-46) as a complex rotation, the attention
+# (:413-460) as an ordinary softmax with one zero key, KVProduct (:320-337) as a product of k shuffled by z ^ blk with the
+# attention output, MulForward / AddScaled (:294-316) as matrix products.  Nothing is rounded to int8 anywhere, and the
+# KV cache holds real vectors.  The oracle must agree with it to within the rounding of its int8 vectors -- and a layer
+# with k and v exchanged, a scale computed from the wrong width, a dropped VEC_SCALE or the ReLU in front of the
+# normalisation must not.
+VS = 1.0 / 24
+LOG2 = 0.693147
+
+
+def _rms_norm(x, groups):
+    g = x.reshape(groups, -1)
+    rms = np.sqrt((g * g).mean(axis=1, keepdims=True))
+    return (g / (rms * VS)).reshape(-1), (rms[:, 0] * VS)
+
+
+def _rotate(x, rope_row, d):
+    out = x.copy().reshape(-1, d)
+    for blk in range(0, d, 64):
+        z = out[:, blk:blk + 32] + 1j * out[:, blk + 32:blk + 64]
+        z = z * (rope_row[blk:blk + 32] + 1j * rope_row[blk + 32:blk + 64])
+        out[:, blk:blk + 32], out[:, blk + 32:blk + 64] = z.real, z.imag
+    return out.reshape(-1)
+
+
+def real_layer(mats, scales, width, slope, t, rope, state, cache, mutate=None):
+    """One token of one sequence.  cache: list of (qv vector [H*D], v vector [H*D]) of the rows before it."""
+    W = {n: m.astype(np.float64) for n, m in mats.items()}
+    qv_scale, comb_scale, contr_scale = scales
+    dim = state.size
+    n, _ = _rms_norm(state, dim // 128)
+    qk, qv, k, v = W["qk"] @ n, W["qv"] @ n, W["k"] @ n, W["v"] @ n
+    qk, qv = _rotate(qk, rope[t], D), _rotate(qv, rope[t], D)
+    qk, _ = _rms_norm(qk, H)
+    k, _ = _rms_norm(k, H)
+    v, _ = _rms_norm(v, H)
+    # the cache keeps qv itself (the int8 path: its normalised form and the scale that undoes the normalisation)
+    key_mult = qv_scale * VS * np.sqrt(1.0 / (D if mutate == "dot_scale_of_head" else dim))
+    if mutate == "drop_vec_scale":
+        key_mult = qv_scale * np.sqrt(1.0 / dim)
+    cache.append((qv * key_mult, v))
+    cur = len(cache) - 1
+    keys = [cur] if width == 0 else list(range(cur - 1, cur - 1 - min(cur, width), -1))
+    att_scale = np.sqrt(1.0 / D) * (0.5 / LOG2)
+    val = np.zeros(H * D)
+    for h in range(H):
+        sl = slice(h * D, (h + 1) * D)
+        logits = np.array([0.0] + [qk[sl] @ cache[to][0][sl] * att_scale * VS - slope * (cur - to) for to in keys])
+        w = np.exp2(logits - logits.max())
+        w /= w.sum()
+        for z, to in enumerate(keys):
+            val[sl] += w[z + 1] * VS * cache[to][1][sl]
+    a, b = (v, k) if mutate == "swap_k_v" else (k, v)
+    del b
+    kv = np.empty(H * D * 4)
+    for h in range(H):
+        for blk in range(4):
+            z = np.arange(D)
+            kv[(h * 4 + blk) * D:(h * 4 + blk + 1) * D] = a[h * D + (z ^ blk)] * val[h * D + z]
+    state = state + (W["combiner"] @ kv) * (comb_scale * VS * np.sqrt(1.0 / kv.size))
+    n2, _ = _rms_norm(state, dim // 128)
+    relu_src = W["expand"] @ n2
+    if mutate == "relu_before_norm":
+        relu, _ = _rms_norm(np.maximum(relu_src, 0.0), H)
+    else:
+        relu = np.maximum(_rms_norm(relu_src, H)[0], 0.0)
+    state = state + (W["contract"] @ relu) * (contr_scale * VS * np.sqrt(1.0 / relu.size))
+    return state, val
+
+
+def _run_both(mutate, n_tokens=6, width=100, slope=0.0, seed=21):
+    """n_tokens tokens of B sequences through the oracle (one shared cache object, as the reference keeps it) and through
+    the real-valued layer; both start every token from the oracle's state, so rounding does not pile up over tokens.
+    Returns the largest differences of the new state's update and of the attention output, relative to their rms."""
+    mats = make_layer(seed)
+    scales = (0.04, 0.03, 0.05)
+    rng = np.random.default_rng(seed + 1)
+    state = rng.standard_normal((B, DIM)).astype(np.float32)
+    k = np.zeros((B, H, MAXLEN, D), dtype=np.uint8)
+    v = np.zeros((B, H, MAXLEN, D), dtype=np.uint8)
+    ks = np.zeros((B, H, MAXLEN), dtype=np.float32)
+    cl = np.zeros(B, dtype=np.int32)
+    rope = orc.fill_rope(D, 64)
+    caches = [[] for _ in range(B)]
+    worst_state, worst_val = 0.0, 0.0
+    for tok in range(n_tokens):
+        t = np.full(B, tok, dtype=np.int32)
+        new_state, val = orc.add_lookup_product(mats, scales, width, slope, H, D, t, rope, state, k, v, ks, cl)
+        for b in range(B):
+            want_state, want_val = real_layer(mats, scales, width, slope, tok, rope.astype(np.float64), state[b].astype(np.float64),
+                                              caches[b], mutate)
+            upd, want_upd = new_state[b] - state[b], want_state - state[b]
+            worst_state = max(worst_state, np.abs(upd - want_upd).max() / np.sqrt((want_upd ** 2).mean()))
+            if tok > 0:
+                worst_val = max(worst_val, np.abs(val[b] - want_val).max() / (np.sqrt((want_val ** 2).mean()) + 1e-30))
+        state = new_state
+    return worst_state, worst_val
+
+
+def test_layer_agrees_with_its_real_valued_form():
+    for width, slope in ((100, 0.0), (2, 0.5), (0, 0.0)):
+        ws, wv = _run_both(None, width=width, slope=slope)
+        assert ws < 0.15 and wv < 0.15, (width, slope, ws, wv)
+
+
+@pytest.mark.parametrize("mutate", ["swap_k_v", "dot_scale_of_head", "drop_vec_scale", "relu_before_norm"])
+def test_a_wrong_composition_does_not(mutate):
+    good_s, good_v = _run_both(None)
+    bad_s, bad_v = _run_both(mutate)
+    assert max(bad_s / good_s, bad_v / good_v) > 4.0, (mutate, good_s, good_v, bad_s, bad_v)
