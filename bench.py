@@ -2,14 +2,18 @@
 """Benchmark of the quantized attention path on one MI355X.
 
 A "step" is one pass of the hot path over one batch of synthetic input, inputs resident in HBM:
-  prefill (the headline `value`): the 125M-style configuration -- batch 16, seq 1024, 12 heads,
-      head_dim 64, e4m3 Q/K/V with per-row fp32 scales, 12 layers alternating (window 64, slope 0.5)
-      and (full causal window, slope 0) -- one step = the 12 attention launches of one forward pass,
-      each layer on its own Q/K/V buffers.
-  decode (reported in the same line under "decode"): batch 64, one bf16 query per sequence, int8 KV
-      cache of 4096 rows, 16 heads x 128, per-row scales; one step = one decode launch pair
-      (split kernel + merge), rotating over 4 caches so that no launch finds its cache in the
-      Infinity Cache.
+  prefill (the headline `value`): the 1.5B-style configuration, the largest prefill shape of the five -- batch 8,
+      seq 4096, 16 heads, head_dim 128, e4m3 Q/K/V with per-row fp32 scales, layers alternating (window 256, slope 0.5)
+      and (full causal window, slope 0) -- one step = one pair of such layers (two launches, 616.19 GFLOP), each layer
+      on its own Q/K/V buffers.
+  "prefill_125M_style": batch 16, seq 1024, 12 heads x 64, e4m3, 12 layers alternating window 64 / full -- one pass
+      of 12 launches.
+  "decode": batch 64, one bf16 query per sequence, int8 KV cache of 4096 rows, 16 heads x 128, per-row scales; one
+      step = one decode launch, rotating over 4 caches so that no launch finds its cache in the Infinity Cache.
+  "generation_1p5B_style": the attention calls of the random-init 1.5B-style generation run at their shapes (24 layers
+      on the InitAlibi schedule, int8, batch 32, 2048-token prompt, 256 generated tokens).
+  "cpu_reference_config": batch 1, seq 1024, 12 heads x 64, int8, full causal window, fp32 output: the shape the
+      reference's CPU path is quoted on; the CPU leg of it runs on int8, as that configuration says.
 Algorithmic work: FLOPs = 4*d*sum_rows min(row, W) per (sequence, head) (masked tiles count zero,
 the zero vector adds none); decode bytes = K + V planes + both scale planes + q + out.
 
@@ -28,10 +32,42 @@ PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA
 PEAK_I8_TOPS = 5000.0
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; KiB per dispatch, scaled
-# by what the same counters read for a copy kernel of known size).  None until measured; the numbers
-# and commands are in profiles/.
-MEASURED_TRAFFIC = {"prefill_c2": 71.4e6, "decode_c3": 1108.0e6}  # bytes per launch (profiles/*.md)
+
+
+def profile_facts():
+    """HBM bytes per launch and matrix-pipe utilisation as rocprofv3 measured them (profiles/*.md: FETCH_SIZE and
+    WRITE_SIZE in KiB per dispatch scaled by what the same counters read for a copy of known size; MfmaUtil).  Each
+    summary carries its figures once more as a `<!-- facts {...} -->` line together with the first 16 hex digits of the
+    sha256 of the kernel source they were measured on; figures of a source that has changed since are not reported."""
+    import glob
+    import hashlib
+    import re
+    out = {}
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        for m in re.finditer(r"<!-- facts (.*?) -->", open(path).read()):
+            try:
+                f = json.loads(m.group(1))
+                src = os.path.join(ROOT, "tscale_amd", "csrc", f["source"])
+                if hashlib.sha256(open(src, "rb").read()).hexdigest()[:16] != f["source_sha16"]:
+                    continue
+                for k, v in f["launches"].items():
+                    out[k] = dict(v, profile=os.path.basename(path))
+            except (KeyError, ValueError, OSError):
+                continue
+    return out
+
+
+def roofline(kernel, bound, achieved, flops_or_bytes, launch_ms, fact):
+    peak, unit = (PEAK_FP8_TFLOPS, "TFLOP/s") if bound == "mfma" else (PEAK_HBM_GBPS, "GB/s")
+    r = {"kernel": kernel, "bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+         "frac": round(achieved / peak, 5), "traffic": None, "launch_ms": round(launch_ms, 5)}
+    r["flops_per_launch" if bound == "mfma" else "bytes_per_launch"] = flops_or_bytes
+    if fact:
+        r["traffic"] = fact.get("traffic_bytes")
+        if "mfma_util" in fact:
+            r["mfma_util"] = fact["mfma_util"]
+        r["traffic_from"] = fact["profile"]
+    return r
 
 
 def pairs(S, W):
@@ -223,7 +259,11 @@ def bench_generation(ctx, steps):
     res["prefill"] = {"layer_ms": {f"W={w}": round(t, 5) for w, t in pre_ms.items()},
                       "pass_ms": round(total_ms, 4), "TOP/s": round(total_flops / total_ms / 1e9, 2),
                       "full_layer_TOP/s": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9, 2),
-                      "full_layer_frac_of_int8_peak": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9 / PEAK_I8_TOPS, 5)}
+                      "full_layer_frac_of_int8_peak": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9 / PEAK_I8_TOPS, 5),
+                      "roofline": {"kernel": "prefill_kernel<int8, d128>, full causal window over the prompt", "bound": "mfma",
+                                   "achieved": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9, 2), "peak": PEAK_I8_TOPS,
+                                   "unit": "TOP/s", "frac": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9 / PEAK_I8_TOPS, 5),
+                                   "traffic": None, "launch_ms": round(pre_ms[wide], 5), "flops_per_launch": gw.prefill_flops(first[wide])}}
     fill_ms = gpu_time_ms(gw.fill_caches, 2, 1)
     n = gw.B * gw.prompt
     fill_bytes = len(gw.caches) * 2 * (n * gw.H * gw.d * 2 + n * gw.H * 4 * 2)   # read + write of K, V and both scales
@@ -256,7 +296,11 @@ def bench_generation(ctx, steps):
     res["generate"] = {"ms_256_tokens": round(gen_ms, 3), "ms_per_token": round(gen_ms / gw.n_new, 4),
                        "us_per_layer_step": round(gen_ms / gw.n_new / len(gw.sched) * 1e3, 2),
                        "GB/s": round(nbytes / gen_ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / gen_ms / 1e6 / PEAK_HBM_GBPS, 4),
-                       "bytes": nbytes, "launch": "HIP graph of one step (24 x decode with fused append), replayed per token"}
+                       "bytes": nbytes, "launch": "HIP graph of one step (24 x decode with fused append), replayed per token",
+                       "roofline": {"kernel": "decode_split_kernel<int8, d128> with fused append, 24 launches per token (+ 10 merges)",
+                                    "bound": "hbm", "achieved": round(nbytes / gen_ms / 1e6, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                                    "frac": round(nbytes / gen_ms / 1e6 / PEAK_HBM_GBPS, 4), "traffic": None,
+                                    "bytes_per_token": nbytes // gw.n_new}}
     return res
 
 
@@ -610,7 +654,7 @@ def bench_prompt_pass(ctx, steps):
             "TOP/s": round((mm_ops + att_flops) / ms / 1e9, 1), "frac_of_int8_peak": round((mm_ops + att_flops) / ms / 1e9 / PEAK_I8_TOPS, 4)}
 
 
-def cpu_baseline_prefill(wl, n_seq_sample):
+def cpu_baseline_prefill(wl, n_seq_sample, layers=None, repeat=1):
     """The oracle (a port of the reference's CPU attention) on the same quantised inputs: the first
     `n_seq_sample` sequences of every layer of the pass, all host threads; plus one sequence of one
     full-window layer on a single thread (the reference's CPU path has no threading)."""
@@ -622,16 +666,17 @@ def cpu_baseline_prefill(wl, n_seq_sample):
     flops = 0.0
     t_total = 0.0
     layers_done = 0
-    for li in range(len(wl.layers)):
+    for li in (layers if layers is not None else range(len(wl.layers))):
         (q, qs), (k, ks), (v, vs) = wl.inputs[li]
         W, slope = wl.layers[li]
         hq, hk, hv = (x[:n].cpu().numpy() for x in (q, k, v))
         hqs, hks, hvs = (np.ascontiguousarray(x[:, :n].cpu().numpy()) for x in (qs, ks, vs))
         st, fi = orc.make_spans([S] * n_seq_sample, W)
         t0 = time.perf_counter()
-        orc.prefill_q8(wl.dtype, hq, hk, hv, H, hqs, hks, hvs, st, fi, slope, n_threads=threads)
+        for _ in range(repeat):
+            orc.prefill_q8(wl.dtype, hq, hk, hv, H, hqs, hks, hvs, st, fi, slope, n_threads=threads)
         t_total += time.perf_counter() - t0
-        flops += prefill_flops(n_seq_sample, S, H, d, W)
+        flops += repeat * prefill_flops(n_seq_sample, S, H, d, W)
         layers_done += 1
         if t_total > 20.0 and layers_done % 2 == 0:
             break
@@ -644,8 +689,8 @@ def cpu_baseline_prefill(wl, n_seq_sample):
     t1 = time.perf_counter() - t0
     return {
         "value": flops / t_total / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-        "sample": f"{n_seq_sample} of {wl.B} sequences, {layers_done} of {len(wl.layers)} layers, "
-                  f"{threads} OpenMP threads, {t_total:.2f} s",
+        "sample": f"{n_seq_sample} of {wl.B} sequences, {layers_done} of {len(wl.layers)} layers"
+                  + (f" x {repeat} repetitions" if repeat > 1 else "") + f", {threads} OpenMP threads, {t_total:.2f} s",
         "single_thread_value": prefill_flops(1, S, H, d, S) / t1 / 1e12,
         "single_thread_sample": f"1 sequence, one full-window layer, 1 thread, {t1:.2f} s",
     }
@@ -729,7 +774,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--extra", action="store_true",
-                    help="also time the 1.5B-style prefill shapes and the attention share of the 1.5B-style generation run")
+                    help="also time the producer, KVProduct, the int8 matrix products, the token step, the prompt pass and "
+                         "generation with the whole int8 model")
     ap.add_argument("--only", default=None,
                     choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step", "prompt-pass", "generate-model", "prompt-then-generate"],
                     help="profiling aid: run just this launch --steps times and print its timing")
@@ -750,32 +796,69 @@ def main():
         run_only(ctx, args)
         return
 
-    # ---- prefill, 125M-style -----------------------------------------------------------------
-    B, S, H, d, NL = 16, 1024, 12, 64, 12
-    wl = PrefillWorkload(ctx, capi.E4M3, B, S, H, d, NL, seed=1313 + 2)
+    facts = profile_facts()
+    # ---- prefill, 1.5B-style: the headline -----------------------------------------------------
+    B, S, H, d = 8, 4096, 16, 128
+    wl = PrefillWorkload(ctx, capi.E4M3, B, S, H, d, 2, seed=1313 + 4, short=256)
     ms = gpu_time_ms(wl.step, args.steps, args.warmup)
     tflops = wl.flops / (ms * 1e-3) / 1e12
-    ms_short = gpu_time_ms(lambda: wl.run_layer(0), args.steps, 2)
-    ms_wide = gpu_time_ms(lambda: wl.run_layer(1), args.steps, 2)
-    launch_ms = ms / NL
-    ach = (wl.flops / NL) / (launch_ms * 1e-3) / 1e12
+    lsteps = max(10, args.steps // 2)
+    ms_short = gpu_time_ms(lambda: wl.run_layer(0), lsteps, 2)
+    ms_wide = gpu_time_ms(lambda: wl.run_layer(1), lsteps, 2)
+    ach = wl.flops_layer[1] / (ms_wide * 1e-3) / 1e12
     result = {
         "metric": "prefill attn TFLOP/s + decode attn HBM GB/s (% of MI355X peak), 1 GPU",
         "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "e4m3 (fp32 accumulate; f16 P.V)", "data": "synthetic",
-        "config": {"workload": "prefill-125M-style: B16 S1024 H12 d64 e4m3 + per-row f32 scales, 12 layers "
-                               "alternating (W=64, slope 0.5)/(W=1024, slope 0), f16 out; 173.18 GFLOP per step",
-                   "layer_ms": {"window64": round(ms_short, 5), "full": round(ms_wide, 5)},
-                   "layer_tflops": {"window64": round(wl.flops_layer[0] / ms_short / 1e9, 2),
+        "config": {"workload": "prefill-1.5B-style: B8 S4096 H16 d128 e4m3 + per-row f32 scales, one pair of layers "
+                               "(W=256, slope 0.5) + (W=4096, slope 0), f16 out; 616.19 GFLOP per step",
+                   "frac_of_fp8_peak": round(tflops / PEAK_FP8_TFLOPS, 5),
+                   "layer_ms": {"window256": round(ms_short, 5), "full": round(ms_wide, 5)},
+                   "layer_tflops": {"window256": round(wl.flops_layer[0] / ms_short / 1e9, 2),
                                     "full": round(wl.flops_layer[1] / ms_wide / 1e9, 2)}},
-        "roofline": {"kernel": "prefill_kernel<e4m3, d64>", "bound": "mfma", "achieved": round(ach, 3),
-                     "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_FP8_TFLOPS, 5),
-                     "traffic": MEASURED_TRAFFIC["prefill_c2"],
-                     "launch_ms": round(launch_ms, 5), "flops_per_launch": wl.flops / NL},
+        # the dominant kernel: the full-window launch (549.62 of the step's 616.19 GFLOP), timed back to back on its own
+        "roofline": roofline("prefill_kernel<e4m3, d128>, full causal window", "mfma", ach, wl.flops_layer[1], ms_wide,
+                             facts.get("prefill_c4_full")),
+        "roofline_window256": roofline("prefill_kernel<e4m3, d128, slope>, window 256", "mfma",
+                                       wl.flops_layer[0] / (ms_short * 1e-3) / 1e12, wl.flops_layer[0], ms_short,
+                                       facts.get("prefill_c4_short")),
     }
     if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline_prefill(wl, 16)
+        result["cpu_baseline"] = cpu_baseline_prefill(wl, 2)
+    del wl
+    torch.cuda.empty_cache()
+
+    # ---- prefill, 125M-style -----------------------------------------------------------------
+    B, S, H, d, NL = 16, 1024, 12, 64, 12
+    wl = PrefillWorkload(ctx, capi.E4M3, B, S, H, d, NL, seed=1313 + 2)
+    ms = gpu_time_ms(wl.step, args.steps, args.warmup)
+    ms_short = graph_time_ms(lambda: wl.run_layer(0), 20, max(3, args.steps // 5))
+    ms_wide = graph_time_ms(lambda: wl.run_layer(1), 20, max(3, args.steps // 5))
+    c2 = {"value": round(wl.flops / (ms * 1e-3) / 1e12, 3), "unit": "TFLOP/s", "ms_per_step": round(ms, 5), "steps": args.steps,
+          "config": {"workload": "prefill-125M-style: B16 S1024 H12 d64 e4m3 + per-row f32 scales, 12 layers alternating "
+                                 "(W=64, slope 0.5)/(W=1024, slope 0), f16 out; 173.18 GFLOP per step",
+                     "layer_ms": {"window64": round(ms_short, 5), "full": round(ms_wide, 5)}},
+          "roofline": roofline("prefill_kernel<e4m3, d64>, full causal window", "mfma", wl.flops_layer[1] / (ms_wide * 1e-3) / 1e12,
+                               wl.flops_layer[1], ms_wide, facts.get("prefill_c2_full")),
+          "roofline_window64": roofline("prefill_kernel<e4m3, d64, slope>, window 64", "mfma",
+                                        wl.flops_layer[0] / (ms_short * 1e-3) / 1e12, wl.flops_layer[0], ms_short,
+                                        facts.get("prefill_c2_short"))}
+    c2["roofline_window64"]["hbm_GB/s"] = round(65.3e6 / (ms_short * 1e-3) / 1e9, 1)   # 65.3 MB of inputs and output per launch
+    if not args.no_cpu:
+        c2["cpu_baseline"] = cpu_baseline_prefill(wl, 16)
+    result["prefill_125M_style"] = c2
+    del wl
+    torch.cuda.empty_cache()
+
+    # ---- the CPU-reference configuration (int8, B1) ------------------------------------------------
+    wl = PrefillWorkload(ctx, capi.I8, 1, 1024, 12, 64, 2, seed=1313 + 1)
+    ms1 = graph_time_ms(lambda: wl.run_layer(1), 20, max(3, args.steps // 5))
+    c1 = {"config": {"workload": "B1 S1024 H12 d64 int8 + per-row f32 scales, full causal window; 1.609 GFLOP"},
+          "gpu_ms": round(ms1, 5), "gpu_TOP/s": round(wl.flops_layer[1] / ms1 / 1e9, 3)}
+    if not args.no_cpu:
+        c1["cpu_baseline"] = cpu_baseline_prefill(wl, 1, layers=[1], repeat=8)
+    result["cpu_reference_config"] = c1
     del wl
     torch.cuda.empty_cache()
 
@@ -788,31 +871,18 @@ def main():
         dec = {"value": round(gbps, 2), "unit": "GB/s", "ms_per_step": round(dms, 5), "steps": dsteps, "dtype": "int8",
                "config": {"workload": "decode: B64, 1 bf16 query/seq, int8 KV cache L=4096, H16 d128, per-row f32 scales; "
                                       "1108.08 MB per step; 4 caches in rotation"},
-               "roofline": {"kernel": "decode_split_kernel<int8, d128>", "bound": "hbm", "achieved": round(gbps, 2),
-                            "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": round(gbps / PEAK_HBM_GBPS, 5),
-                            "traffic": MEASURED_TRAFFIC["decode_c3"], "bytes_per_launch": dw.bytes}}
+               "roofline": roofline("decode_split_kernel<int8, d128>", "hbm", gbps, dw.bytes, dms, facts.get("decode_c3"))}
         if not args.no_cpu:
             dec["cpu_baseline"] = cpu_baseline_decode(dw, 64, 200)
         result["decode"] = dec
         del dw
         torch.cuda.empty_cache()
+        # ---- the attention calls of the 1.5B-style generation run ---------------------------------
+        result["generation_1p5B_style"] = bench_generation(ctx, args.steps)
+        torch.cuda.empty_cache()
 
     # ---- optional: 1.5B-style prefill shapes ---------------------------------------------------------
     if args.extra:
-        B, S, H, d = 8, 4096, 16, 128
-        wl = PrefillWorkload(ctx, capi.E4M3, B, S, H, d, 2, seed=1313 + 4, short=256)
-        steps = max(10, args.steps // 5)
-        ms_s = gpu_time_ms(lambda: wl.run_layer(0), steps, 2)
-        ms_w = gpu_time_ms(lambda: wl.run_layer(1), steps, 2)
-        result["prefill_1p5B_style"] = {
-            "config": "B8 S4096 H16 d128 e4m3, W=256 (slope 0.5) / full (slope 0)",
-            "layer_ms": {"window256": round(ms_s, 5), "full": round(ms_w, 5)},
-            "layer_tflops": {"window256": round(wl.flops_layer[0] / ms_s / 1e9, 2), "full": round(wl.flops_layer[1] / ms_w / 1e9, 2)},
-            "frac_of_fp8_peak_full": round(wl.flops_layer[1] / ms_w / 1e9 / PEAK_FP8_TFLOPS, 5)}
-        del wl
-        torch.cuda.empty_cache()
-        result["generation_1p5B_style"] = bench_generation(ctx, args.steps)
-        torch.cuda.empty_cache()
         result["producer"] = bench_producer(ctx, args.steps)
         torch.cuda.empty_cache()
         result["kv_product"] = bench_kv_product(ctx, args.steps)
