@@ -173,6 +173,20 @@ typedef struct tsattn_decode_args {
 
 int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream);
 
+/* tsattn_decode for callers that cannot allocate device memory: code under HIP graph capture that has no handle yet,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same
+ * kernels and the same results as tsattn_decode, but no handle: the split partials and arrival counters live in an array
+ * that is part of the library's device image (about 8.1 MiB per GPU the library runs on, held until the process ends),
+ * and the call -- the first one on a device included -- makes no hipMalloc / hipFree or other allocating call.  It runs
+ * on the calling thread's current device; `stream` must belong to it.
+ * Limits (TSATTN_ERR_SCRATCH beyond them): n_seqs <= TSATTN_STATIC_MAX_SEQS and n_seqs * n_heads * splits <=
+ * TSATTN_STATIC_MAX_PARTS, where splits is n_splits, or with n_splits == 0 what the library chooses (never more than
+ * fits).  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race;
+ * order them. */
+#define TSATTN_STATIC_MAX_PARTS 16384
+#define TSATTN_STATIC_MAX_SEQS 1024
+int tsattn_decode_static(const tsattn_decode_args *a, void *stream);
+
 /* Append one token per sequence to the cache at row cache_len[seq], then increment cache_len[seq]
  * on the device.  Replaces TAttentionVecHistory::AddVectors, gpt/train/cpu_infer.cpp:403-408
  * (call :506).  k_new, v_new: [n_seqs][n_heads*head_dim] 8-bit; *_scale_new: [n_seqs][n_heads]. */

@@ -321,11 +321,12 @@ class AttentionContext:
 
     # ---- decode ---------------------------------------------------------------------------------
     def compute_val_lookup_decode(self, cache, q, q_scale, window, alibi_slope, out=None, n_splits=0,
-                                  debug_qk_acc=None, max_len=None, append=None, kv_product=None):
+                                  debug_qk_acc=None, max_len=None, append=None, kv_product=None, static_scratch=False):
         """q: uint8 [B, H*d] with q_scale f32 [B, H] (or a number), or bfloat16 [B, H*d] (quantised in the kernel).
         append = (k_new, k_scale_new, v_new, v_scale_new): KVCache.add_vectors fused into the same launches.
         kv_product = (k, kv_out, rep, mult): KVProduct of the result with the token's K vector, written by the same
-        launches (k uint8 [B, H*d], kv_out uint8 [B, H*rep*d])."""
+        launches (k uint8 [B, H*d], kv_out uint8 [B, H*rep*d]).
+        static_scratch: go through tsattn_decode_static, the entry point that needs no handle and allocates nothing."""
         B, H, d = cache.n_seqs, cache.n_heads, cache.head_dim
         if out is None:
             out = torch.empty((B, H * d), dtype=torch.float32, device=q.device)
@@ -357,7 +358,10 @@ class AttentionContext:
             kk, kv_out, rep, mult = kv_product
             a.kv_k, a.kv_k_pitch, a.kv_out, a.kv_out_pitch = _ptr(kk), kk.stride(0), _ptr(kv_out), kv_out.stride(0)
             a.kv_rep, a.kv_mult = int(rep), float(mult)
-        capi.check(self.lib.tsattn_decode(self.handle, ctypes.byref(a), _stream_ptr()))
+        if static_scratch:
+            capi.check(self.lib.tsattn_decode_static(ctypes.byref(a), _stream_ptr()))
+        else:
+            capi.check(self.lib.tsattn_decode(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
 
 

@@ -5,6 +5,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
+#include <mutex>
+
 #include "../../include/tsattn.h"
 #include "kernels.hpp"
 
@@ -14,6 +17,24 @@ struct tsattn_ctx {
     float *part_acc;
     float *part_ml;
     int32_t *seq_done;
+};
+
+// Scratch of the entry point that allocates nothing (tsattn_decode_static): split partials [pair][split][d] f32, their
+// (max, sum) pairs, per-sequence arrival counters.  One copy per GPU the library runs on, held until the process ends.
+constexpr int64_t STATIC_ACC_BYTES = (int64_t)TSATTN_STATIC_MAX_PARTS * 128 * sizeof(float);
+constexpr int64_t STATIC_ML_BYTES = (int64_t)TSATTN_STATIC_MAX_PARTS * 2 * sizeof(float);
+constexpr int64_t STATIC_CNT_BYTES = (int64_t)TSATTN_STATIC_MAX_SEQS * sizeof(int32_t);
+static __device__ __align__(256) uint8_t g_decode_scratch[STATIC_ACC_BYTES + STATIC_ML_BYTES + STATIC_CNT_BYTES];
+constexpr int STATIC_MAX_DEVICES = 64;
+static uint8_t *g_static_ptr[STATIC_MAX_DEVICES]; // this device's copy of the array, from hipGetSymbolAddress
+static std::mutex g_static_mutex;
+
+struct DecodeScratch {
+    int max_seqs, max_head_dim, max_splits;
+    int64_t max_pairs, max_parts; // (sequence, head) pairs; pairs x splits
+    float *part_acc, *part_ml;
+    int32_t *seq_done;
+    bool clear_counters;
 };
 
 namespace {
@@ -43,6 +64,85 @@ bool dtype_ok(int t) { return t == TSATTN_I8 || t == TSATTN_E4M3; }
 bool aligned16(const void *p) { return (((uintptr_t)p) & 15) == 0; }
 
 } // namespace
+
+// The body of both decode entry points; `lim` says what the scratch behind part_acc / part_ml / seq_done was sized for.
+static int decode_with_scratch(const DecodeScratch &lim, const tsattn_decode_args *a, void *stream)
+{
+    if (!dtype_ok(a->dtype)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: dtype %d", a->dtype);
+    if (a->q_dtype != TSATTN_Q_8BIT && a->q_dtype != TSATTN_Q_BF16) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: q_dtype %d", a->q_dtype);
+    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: head_dim %d (64 or 128 supported)", a->head_dim);
+    if (a->n_seqs < 0 || a->n_heads <= 0 || a->max_len < 0 || a->window < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: negative size");
+    if (a->n_seqs == 0) return TSATTN_OK;
+    if (!a->q || !a->k_cache || !a->v_cache || !a->cache_len || !a->out) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: null data pointer");
+    const int qbytes = a->q_dtype == TSATTN_Q_BF16 ? 2 : 1;
+    if (a->q_pitch < (int64_t)a->n_heads * a->head_dim * qbytes || a->q_pitch % 16) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: q_pitch");
+    if (a->tok_stride < a->head_dim || a->tok_stride % 16 || a->head_stride % 16 || a->seq_stride % 16)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: cache strides must be multiples of 16 bytes, tok_stride >= head_dim");
+    if (!aligned16(a->q) || !aligned16(a->k_cache) || !aligned16(a->v_cache)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: q and caches must be 16-byte aligned");
+    if (a->debug_qk_acc && a->debug_pitch < a->max_len) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: debug_pitch < max_len");
+    if (a->n_seqs > lim.max_seqs || a->head_dim > lim.max_head_dim || (int64_t)a->n_seqs * a->n_heads > lim.max_pairs)
+        return fail(TSATTN_ERR_SCRATCH, "tsattn_decode: %d seqs x %d heads x d%d exceeds the scratch's %d seqs, %lld (seq, head) pairs, d%d", a->n_seqs,
+                    a->n_heads, a->head_dim, lim.max_seqs, (long long)lim.max_pairs, lim.max_head_dim);
+    const int max_splits = (int)std::min<int64_t>(lim.max_splits, lim.max_parts / ((int64_t)a->n_seqs * a->n_heads));
+    int splits = a->n_splits;
+    if (splits < 0 || splits > max_splits) return fail(TSATTN_ERR_SCRATCH, "tsattn_decode: n_splits %d exceeds the scratch's %d for this batch", splits, max_splits);
+    if (splits == 0) {
+        // One workgroup streams its rows fast enough that one or two per compute unit reach the memory's rate, and every
+        // split beyond that only adds to the merge: about 384 workgroups in all (measured best at 4096 rows: 1 split from
+        // 256 (sequence, head) pairs up, 4 at 128, 8 at 32 and below), and at least 512 cache rows per split
+        const int64_t pairs = (int64_t)a->n_seqs * a->n_heads;
+        int64_t want = 384 / pairs;
+        int64_t rows = a->max_len;   // rows one query can see
+        if (a->window < rows) rows = a->window > 0 ? a->window : 1;
+        int64_t by_len = (rows + 511) / 512;
+        if (want > by_len) want = by_len;
+        if (want < 1) want = 1;
+        if (want > max_splits) want = max_splits;
+        splits = (int)want;
+    }
+    tsattn::DecodeParams p = {};
+    p.q = (const uint8_t *)a->q; p.q_pitch = a->q_pitch; p.q_scale = a->q_scale; p.q_scale_const = a->q_scale_const;
+    p.k = (const uint8_t *)a->k_cache; p.v = (const uint8_t *)a->v_cache;
+    p.seq_stride = a->seq_stride; p.head_stride = a->head_stride; p.tok_stride = a->tok_stride;
+    p.ks = a->k_scale; p.vs = a->v_scale; p.s_seq_stride = a->s_seq_stride; p.s_head_stride = a->s_head_stride;
+    p.ks_const = a->k_scale_const; p.vs_const = a->v_scale_const;
+    p.cache_len = a->cache_len; p.window = a->window; p.slope = a->alibi_slope;
+    p.n_heads = a->n_heads; p.n_splits = splits;
+    p.part_acc = lim.part_acc; p.part_ml = lim.part_ml;
+    p.dbg = a->debug_qk_acc; p.dbg_pitch = a->debug_pitch;
+    p.out = a->out;
+    p.k_new = (const uint8_t *)a->k_new; p.v_new = (const uint8_t *)a->v_new; p.new_pitch = a->new_pitch;
+    p.ks_new = a->k_scale_new; p.vs_new = a->v_scale_new;
+    p.cache_len_rw = const_cast<int32_t *>(a->cache_len); p.max_len = a->max_len;
+    p.seq_done = lim.seq_done;
+    if (a->kv_out) {
+        if (!a->kv_k) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: the fused KVProduct needs kv_k");
+        if (a->dtype != TSATTN_I8) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: the fused KVProduct is defined for int8 keys");
+        if (a->kv_rep < 1 || a->kv_rep > 4) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: kv_rep %d (1..4)", a->kv_rep);
+        if (((uintptr_t)a->kv_k & 3) || a->kv_k_pitch % 4 || a->kv_k_pitch < (int64_t)a->n_heads * a->head_dim ||
+            a->kv_out_pitch < (int64_t)a->n_heads * a->head_dim * a->kv_rep)
+            return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: kv_k must be 4-byte aligned and the kv pitches must cover a row");
+        p.kv_k = (const uint8_t *)a->kv_k; p.kv_k_pitch = a->kv_k_pitch; p.kv_out = (uint8_t *)a->kv_out; p.kv_out_pitch = a->kv_out_pitch;
+        p.kv_rep = a->kv_rep; p.kv_mult = a->kv_mult;
+    }
+    if (a->k_new || a->v_new) {
+        if (!a->k_new || !a->v_new) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: fused append needs both k_new and v_new");
+        if (a->window == 0) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: fused append is not available with window 0; call tsattn_cache_append first");
+        if (a->new_pitch % 16 || a->new_pitch < (int64_t)a->n_heads * a->head_dim || !aligned16(a->k_new) || !aligned16(a->v_new))
+            return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: k_new/v_new must be 16-byte aligned with a pitch that covers a row");
+        if ((a->k_scale_new && !a->k_scale) || (a->v_scale_new && !a->v_scale)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: new scales given without scale planes");
+    }
+    if (lim.clear_counters && a->k_new) {
+        // the arrival counters of the single-split fused append start at zero: a launch leaves them so, but this scratch is
+        // shared by every caller on the device (a fill kernel, not a memset: callers may be capturing a graph)
+        hipError_t ez = tsattn::launch_zero_i32(lim.seq_done, a->n_seqs, (hipStream_t)stream);
+        if (ez != hipSuccess) return hip_fail(ez, "counter clear launch");
+    }
+    hipError_t e = tsattn::launch_decode(p, a->dtype, a->head_dim, a->q_dtype == TSATTN_Q_BF16, a->n_seqs, a->out, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "decode launch");
+    return TSATTN_OK;
+}
+
 
 extern "C" {
 
@@ -175,72 +275,43 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
 int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
 {
     if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: null argument");
-    if (!dtype_ok(a->dtype)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: dtype %d", a->dtype);
-    if (a->q_dtype != TSATTN_Q_8BIT && a->q_dtype != TSATTN_Q_BF16) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: q_dtype %d", a->q_dtype);
-    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: head_dim %d (64 or 128 supported)", a->head_dim);
-    if (a->n_seqs < 0 || a->n_heads <= 0 || a->max_len < 0 || a->window < 0) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: negative size");
-    if (a->n_seqs == 0) return TSATTN_OK;
-    if (!a->q || !a->k_cache || !a->v_cache || !a->cache_len || !a->out) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: null data pointer");
-    const int qbytes = a->q_dtype == TSATTN_Q_BF16 ? 2 : 1;
-    if (a->q_pitch < (int64_t)a->n_heads * a->head_dim * qbytes || a->q_pitch % 16) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: q_pitch");
-    if (a->tok_stride < a->head_dim || a->tok_stride % 16 || a->head_stride % 16 || a->seq_stride % 16)
-        return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: cache strides must be multiples of 16 bytes, tok_stride >= head_dim");
-    if (!aligned16(a->q) || !aligned16(a->k_cache) || !aligned16(a->v_cache)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: q and caches must be 16-byte aligned");
-    if (a->debug_qk_acc && a->debug_pitch < a->max_len) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: debug_pitch < max_len");
-    if (a->n_seqs > h->max_seqs || a->n_heads > h->max_heads || a->head_dim > h->max_head_dim)
-        return fail(TSATTN_ERR_SCRATCH, "tsattn_decode: %d seqs x %d heads x d%d exceeds the handle's %d x %d x d%d", a->n_seqs, a->n_heads,
-                    a->head_dim, h->max_seqs, h->max_heads, h->max_head_dim);
-    int splits = a->n_splits;
-    if (splits < 0 || splits > h->max_splits) return fail(TSATTN_ERR_SCRATCH, "tsattn_decode: n_splits %d exceeds the handle's %d", splits, h->max_splits);
-    if (splits == 0) {
-        // One workgroup streams its rows fast enough that one or two per compute unit reach the memory's rate, and every
-        // split beyond that only adds to the merge: about 384 workgroups in all (measured best at 4096 rows: 1 split from
-        // 256 (sequence, head) pairs up, 4 at 128, 8 at 32 and below), and at least 512 cache rows per split
-        const int64_t pairs = (int64_t)a->n_seqs * a->n_heads;
-        int64_t want = 384 / pairs;
-        int64_t rows = a->max_len;   // rows one query can see
-        if (a->window < rows) rows = a->window > 0 ? a->window : 1;
-        int64_t by_len = (rows + 511) / 512;
-        if (want > by_len) want = by_len;
-        if (want < 1) want = 1;
-        if (want > h->max_splits) want = h->max_splits;
-        splits = (int)want;
+    DecodeScratch lim;
+    lim.max_seqs = h->max_seqs; lim.max_head_dim = h->max_head_dim; lim.max_splits = h->max_splits;
+    lim.max_pairs = (int64_t)h->max_seqs * h->max_heads;
+    lim.max_parts = lim.max_pairs * h->max_splits;
+    lim.part_acc = h->part_acc; lim.part_ml = h->part_ml; lim.seq_done = h->seq_done;
+    lim.clear_counters = false;
+    return decode_with_scratch(lim, a, stream);
+}
+
+int tsattn_decode_static(const tsattn_decode_args *a, void *stream)
+{
+    if (!a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode_static: null argument");
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= STATIC_MAX_DEVICES) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode_static: device %d (ordinals below %d)", dev, STATIC_MAX_DEVICES);
+    uint8_t *base;
+    {
+        // Set-up, once per device and with that device current: the array's name is a host-side stand-in; the address of
+        // this device's copy comes from the runtime and is what every use below goes through.
+        std::lock_guard<std::mutex> lock(g_static_mutex);
+        if (!g_static_ptr[dev]) {
+            void *ptr = nullptr;
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_decode_scratch));
+            if (e != hipSuccess || !ptr) return hip_fail(e, "hipGetSymbolAddress(decode scratch)");
+            g_static_ptr[dev] = (uint8_t *)ptr;
+        }
+        base = g_static_ptr[dev];
     }
-    tsattn::DecodeParams p = {};
-    p.q = (const uint8_t *)a->q; p.q_pitch = a->q_pitch; p.q_scale = a->q_scale; p.q_scale_const = a->q_scale_const;
-    p.k = (const uint8_t *)a->k_cache; p.v = (const uint8_t *)a->v_cache;
-    p.seq_stride = a->seq_stride; p.head_stride = a->head_stride; p.tok_stride = a->tok_stride;
-    p.ks = a->k_scale; p.vs = a->v_scale; p.s_seq_stride = a->s_seq_stride; p.s_head_stride = a->s_head_stride;
-    p.ks_const = a->k_scale_const; p.vs_const = a->v_scale_const;
-    p.cache_len = a->cache_len; p.window = a->window; p.slope = a->alibi_slope;
-    p.n_heads = a->n_heads; p.n_splits = splits;
-    p.part_acc = h->part_acc; p.part_ml = h->part_ml;
-    p.dbg = a->debug_qk_acc; p.dbg_pitch = a->debug_pitch;
-    p.out = a->out;
-    p.k_new = (const uint8_t *)a->k_new; p.v_new = (const uint8_t *)a->v_new; p.new_pitch = a->new_pitch;
-    p.ks_new = a->k_scale_new; p.vs_new = a->v_scale_new;
-    p.cache_len_rw = const_cast<int32_t *>(a->cache_len); p.max_len = a->max_len;
-    p.seq_done = h->seq_done;
-    if (a->kv_out) {
-        if (!a->kv_k) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: the fused KVProduct needs kv_k");
-        if (a->dtype != TSATTN_I8) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: the fused KVProduct is defined for int8 keys");
-        if (a->kv_rep < 1 || a->kv_rep > 4) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: kv_rep %d (1..4)", a->kv_rep);
-        if (((uintptr_t)a->kv_k & 3) || a->kv_k_pitch % 4 || a->kv_k_pitch < (int64_t)a->n_heads * a->head_dim ||
-            a->kv_out_pitch < (int64_t)a->n_heads * a->head_dim * a->kv_rep)
-            return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: kv_k must be 4-byte aligned and the kv pitches must cover a row");
-        p.kv_k = (const uint8_t *)a->kv_k; p.kv_k_pitch = a->kv_k_pitch; p.kv_out = (uint8_t *)a->kv_out; p.kv_out_pitch = a->kv_out_pitch;
-        p.kv_rep = a->kv_rep; p.kv_mult = a->kv_mult;
-    }
-    if (a->k_new || a->v_new) {
-        if (!a->k_new || !a->v_new) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: fused append needs both k_new and v_new");
-        if (a->window == 0) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_decode: fused append is not available with window 0; call tsattn_cache_append first");
-        if (a->new_pitch % 16 || a->new_pitch < (int64_t)a->n_heads * a->head_dim || !aligned16(a->k_new) || !aligned16(a->v_new))
-            return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: k_new/v_new must be 16-byte aligned with a pitch that covers a row");
-        if ((a->k_scale_new && !a->k_scale) || (a->v_scale_new && !a->v_scale)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode: new scales given without scale planes");
-    }
-    hipError_t e = tsattn::launch_decode(p, a->dtype, a->head_dim, a->q_dtype == TSATTN_Q_BF16, a->n_seqs, a->out, (hipStream_t)stream);
-    if (e != hipSuccess) return hip_fail(e, "decode launch");
-    return TSATTN_OK;
+    DecodeScratch lim;
+    lim.max_seqs = TSATTN_STATIC_MAX_SEQS; lim.max_head_dim = 128; lim.max_splits = DEFAULT_MAX_SPLITS;
+    lim.max_pairs = TSATTN_STATIC_MAX_PARTS; lim.max_parts = TSATTN_STATIC_MAX_PARTS;
+    lim.part_acc = (float *)base;
+    lim.part_ml = (float *)(base + STATIC_ACC_BYTES);
+    lim.seq_done = (int32_t *)(base + STATIC_ACC_BYTES + STATIC_ML_BYTES);
+    lim.clear_counters = true;
+    return decode_with_scratch(lim, a, stream);
 }
 
 int tsattn_cache_append(tsattn_handle_t h, const tsattn_append_args *a, void *stream)

@@ -179,6 +179,19 @@ __global__ void cache_len_bump_kernel(int32_t *cache_len, int n_seqs, int max_le
     if (i < n_seqs && cache_len[i] >= 0 && cache_len[i] < max_len) cache_len[i] += 1;
 }
 
+__global__ void zero_i32_kernel(int32_t *p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+hipError_t launch_zero_i32(int32_t *p, int n, hipStream_t st)
+{
+    if (n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(zero_i32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, p, n);
+    return hipGetLastError();
+}
+
 hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st)
 {
     if (n_seqs == 0) return hipSuccess;

@@ -107,6 +107,9 @@ struct AppendParams {
 
 hipError_t launch_cache_append(const AppendParams &p, int n_seqs, hipStream_t st);
 
+// n int32 at p become zero (a kernel: memset nodes are avoided in code a caller may capture into a graph)
+hipError_t launch_zero_i32(int32_t *p, int n, hipStream_t st);
+
 struct ProduceParams {
     const void *src;
     int64_t src_pitch; // elements per row
