@@ -5,7 +5,8 @@
  * All data pointers are DEVICE pointers unless stated otherwise.  Every call that takes a stream is
  * asynchronous on that stream (pass the hipStream_t as void*, NULL = the default stream), never
  * synchronises, never allocates and never reads device data on the host, so it can be captured
- * into a HIP graph.  A handle belongs to one device and one host thread at a time.
+ * into a HIP graph.  A handle belongs to one device and one host thread at a time, and calls on one handle must not
+ * overlap on the device (one stream, or ordered streams): decode keeps split partials and arrival counters in it.
  *
  * Reference lines are given relative to the reference's code/ directory.
  *
@@ -397,6 +398,10 @@ int tsattn_quantize_rows(tsattn_handle_t h, int src_dtype, int dst_dtype, const 
 int tsattn_build_spans(tsattn_handle_t h, int n_seqs, const int32_t *seq_offset, int64_t n_tokens,
                        const uint8_t *doc_start_flag, int64_t window, int32_t *span_start,
                        int32_t *span_finish, void *stream);
+
+/* Diagnostic: copies the handle's per-sequence arrival counters (used by the single-split fused append of tsattn_decode;
+ * every launch leaves them at zero) into dst, a device array of n int32, on the stream.  For tests of graph replays. */
+int tsattn_debug_read_counters(tsattn_handle_t h, int32_t *dst, int n, void *stream);
 
 /* Library build identification (kernel set and target), for logs. */
 const char *tsattn_version(void);

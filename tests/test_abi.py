@@ -19,6 +19,7 @@ STRUCTS = {
     "tsattn_append_args": capi.AppendArgs,
     "tsattn_fill_args": capi.FillArgs,
     "tsattn_produce_args": capi.ProduceArgs,
+    "tsattn_matmul_args": capi.MatmulArgs,
 }
 
 

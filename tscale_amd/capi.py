@@ -109,7 +109,7 @@ class FillArgs(_c.Structure):
 
 
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_decode_static", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_embed_rows", "tsattn_softmax_rows", "tsattn_sample_rows", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_version"]
+           "tsattn_decode", "tsattn_decode_static", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_embed_rows", "tsattn_softmax_rows", "tsattn_sample_rows", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_debug_read_counters", "tsattn_version"]
 
 _lib = None
 
@@ -135,6 +135,8 @@ def load():
         L.tsattn_prefill.argtypes = [_c.c_void_p, _c.POINTER(PrefillArgs), _c.c_void_p]
         L.tsattn_decode.restype = _c.c_int
         L.tsattn_decode.argtypes = [_c.c_void_p, _c.POINTER(DecodeArgs), _c.c_void_p]
+        L.tsattn_debug_read_counters.restype = _c.c_int
+        L.tsattn_debug_read_counters.argtypes = [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p]
         L.tsattn_decode_static.restype = _c.c_int
         L.tsattn_decode_static.argtypes = [_c.POINTER(DecodeArgs), _c.c_void_p]
         L.tsattn_cache_append.restype = _c.c_int

@@ -284,6 +284,15 @@ int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)
     return decode_with_scratch(lim, a, stream);
 }
 
+int tsattn_debug_read_counters(tsattn_handle_t h, int32_t *dst, int n, void *stream)
+{
+    if (!h || !dst || n < 0 || n > h->max_seqs) return fail(TSATTN_ERR_BAD_ARG, "tsattn_debug_read_counters: bad argument");
+    if (n == 0) return TSATTN_OK;
+    hipError_t e = hipMemcpyAsync(dst, h->seq_done, (size_t)n * sizeof(int32_t), hipMemcpyDeviceToDevice, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "counter copy");
+    return TSATTN_OK;
+}
+
 int tsattn_decode_static(const tsattn_decode_args *a, void *stream)
 {
     if (!a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_decode_static: null argument");
