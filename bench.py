@@ -25,6 +25,8 @@ import os
 import sys
 import time
 
+import numpy as np
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
@@ -400,9 +402,12 @@ def bench_matmul(ctx, steps):
 class Int8Layers:
     """24 layers of the int8 inference path (AddLookupProduct, gpt/train/cpu_infer.cpp:465-527) at the 1.5B-style
     attention shape: model width 2048, 16 heads x 128, feed-forward width 2048, per-layer attention width and slope
-    from InitAlibi's schedule, random int8 weights of rms 32 (what the reference's matrix conversion leaves,
-    MODEL_DISCR_SCALE = 1/32), one KV cache per layer for B = 32 sequences.  Embedding, final layer and sampling are
-    not part of it."""
+    from InitAlibi's schedule (tscale_amd/host/model_init.cpp), weights as the reference's random model has them:
+    InitMatrixNormal's table-of-normals values times 0.5 for every matrix -- combiner and contract included
+    (COMBINER_INIT_RANDOM: with the zero start of create_model() the attention output would never reach the result,
+    gpt/train/main_gpt.cpp:274) -- converted by ConvertMatrix (int8 of rms 32, scale = rms / 32), the matrix scales what
+    that conversion returned; one KV cache per layer for B = 32 sequences.  Embedding, final layer and sampling are not
+    part of it."""
 
     def __init__(self, ctx, cache_len, seed, n_new=64):
         import torch
@@ -414,14 +419,22 @@ class Int8Layers:
         qsum = self.H * self.d
         g = torch.Generator(device="cuda").manual_seed(seed)
         self.g = g
-        def matrix(n, k):
-            return (torch.randn((n, k), device="cuda", generator=g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
-        self.sched = alibi_layer_schedule(self.depth, self.L)
+        from tscale_amd import model_init
+        self.seed = seed
+        def matrices(count, n, k, salt):
+            q, sc = model_init.random_int8_matrices(seed * 1000 + salt, count, n, k)
+            return torch.from_numpy(q.view(np.uint8).reshape(count * n, k)).cuda(), sc
+        self.sched = model_init.init_alibi(self.depth, self.L)
+        assert self.sched == [(w, float(np.float32(sl))) for w, sl in alibi_layer_schedule(self.depth, self.L)]
         self.layers, self.caches = [], []
-        for w, slope in self.sched:
-            self.layers.append({"proj": matrix(4 * qsum, self.dim), "combiner": matrix(self.dim, qsum * 4),
-                                "expand": matrix(qsum, self.dim), "contract": matrix(self.dim, qsum),
-                                "qv_scale": 0.03, "combiner_scale": 0.03, "contract_scale": 0.03, "width": w, "slope": slope})
+        for li, (w, slope) in enumerate(self.sched):
+            proj, psc = matrices(4, qsum, self.dim, 10 * li)             # QK, QV, K, V one after the other
+            comb, csc = matrices(1, self.dim, qsum * 4, 10 * li + 1)
+            expand, _ = matrices(1, qsum, self.dim, 10 * li + 2)
+            contract, tsc = matrices(1, self.dim, qsum, 10 * li + 3)
+            self.layers.append({"proj": proj, "combiner": comb, "expand": expand, "contract": contract,
+                                "qv_scale": float(psc[1]), "combiner_scale": float(csc[0]), "contract_scale": float(tsc[0]),
+                                "width": w, "slope": slope})
             c = KVCache(ctx, capi.I8, self.B, self.H, self.L, self.d)
             if cache_len > 0:   # a cache that already holds a prompt: random rows
                 c.k.copy_((torch.randn(c.k.shape, device="cuda", generator=g) * 24).round().clamp(-127, 127).to(torch.int8).view(torch.uint8))
@@ -433,6 +446,18 @@ class Int8Layers:
         self.rope = ctx.fill_rope_table(self.d, self.L)
         self.weight_bytes = sum(sum(v.numel() for v in layer.values() if isinstance(v, torch.Tensor)) for layer in self.layers)
         self.matmul_ops_per_token = 2.0 * sum(sum(v.numel() for v in layer.values() if isinstance(v, torch.Tensor)) for layer in self.layers)
+
+
+def model_ends(m, vocab, dim):
+    """Embedding and final layer of the random model (InitEmbedMatrix: table values as they are, the first 32 labels' rows
+    zero; InitMatrixNormal with sko 1 for the final layer; gpt/model_params/model_params.cpp:47-66, 135-143), converted."""
+    import torch
+    from tscale_amd import model_init
+    e = model_init.init_matrix_normal(m.seed * 1000 + 900, 2.0, vocab, dim)
+    e[:32] = 0
+    eq, es = model_init.convert_matrix(e)
+    fq, fs = model_init.random_int8_matrices(m.seed * 1000 + 901, 1, vocab, dim)
+    return torch.from_numpy(eq.view(np.uint8)).cuda(), es, torch.from_numpy(fq[0].view(np.uint8)).cuda(), float(fs[0])
 
 
 def bench_token_step(ctx, steps):
@@ -487,12 +512,10 @@ def bench_generate_model(ctx, steps):
     m = Int8Layers(ctx, cache_len=2048, seed=1313 + 11)
     B, H, d, dim, qsum = m.B, m.H, m.d, m.dim, m.H * m.d
     vocab = 50257
-    def matrix(n, k):
-        return (torch.randn((n, k), device="cuda", generator=m.g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
-    embed, final = matrix(vocab, dim), matrix(vocab, dim)
+    embed, embed_scale, final, final_layer_scale = model_ends(m, vocab, dim)
     bias = torch.randn(vocab, device="cuda", generator=m.g) * 0.1
     f32 = np.float32
-    final_scale = float(f32(np.sqrt(f32(1.0) / f32(dim))) * (f32(1.0) / f32(0.693147)) * f32(0.03) * f32(VEC_SCALE))
+    final_scale = float(f32(np.sqrt(f32(1.0) / f32(dim))) * (f32(1.0) / f32(0.693147)) * f32(final_layer_scale) * f32(VEC_SCALE))
     labels = torch.randint(0, vocab, (B,), dtype=torch.int32, device="cuda", generator=m.g)
     state = torch.empty((B, dim), dtype=torch.float32, device="cuda")
     t = torch.full((B,), m.prompt, dtype=torch.int32, device="cuda")
@@ -500,7 +523,7 @@ def bench_generate_model(ctx, steps):
     planes = torch.empty(16 * B * vocab, dtype=torch.int32, device="cuda")
     keep = {}
     def step():
-        ctx.embed_rows(labels, embed, 0.03, out=state)
+        ctx.embed_rows(labels, embed, embed_scale, out=state)
         pending = None
         for layer, c in zip(m.layers, m.caches):
             _, pending = add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep, pending=pending, defer=True)
@@ -541,12 +564,10 @@ def bench_prompt_then_generate(ctx, n_new=256):
     m = Int8Layers(ctx, cache_len=0, seed=1313 + 12, n_new=n_new)
     B, H, d, dim, qsum = m.B, m.H, m.d, m.dim, m.H * m.d
     vocab = 50257
-    def matrix(n, k):
-        return (torch.randn((n, k), device="cuda", generator=m.g) * 32).round().clamp(-127, 127).to(torch.int8).view(torch.uint8)
-    embed, final = matrix(vocab, dim), matrix(vocab, dim)
+    embed, embed_scale, final, final_layer_scale = model_ends(m, vocab, dim)
     bias = torch.randn(vocab, device="cuda", generator=m.g) * 0.1
     f32 = np.float32
-    final_scale = float(f32(np.sqrt(f32(1.0) / f32(dim))) * (f32(1.0) / f32(0.693147)) * f32(0.03) * f32(VEC_SCALE))
+    final_scale = float(f32(np.sqrt(f32(1.0) / f32(dim))) * (f32(1.0) / f32(0.693147)) * f32(final_layer_scale) * f32(VEC_SCALE))
     n = B * m.prompt
     ids = torch.randint(0, vocab, (n,), dtype=torch.int32, device="cuda", generator=m.g)
     off = torch.arange(0, n + 1, m.prompt, dtype=torch.int32, device="cuda")
@@ -565,7 +586,7 @@ def bench_prompt_then_generate(ctx, n_new=256):
         logits = ctx.matmul_i8(norm, final, mode=capi.MM_I32_PLANES, out=planes)
         ctx.softmax_rows(logits, final_scale, bias, want_prob=False, argmax=labels)
     def prompt_phase():
-        ctx.embed_rows(ids, embed, 0.03, out=prompt_state)
+        ctx.embed_rows(ids, embed, embed_scale, out=prompt_state)
         norm = None
         for layer, c in zip(m.layers, m.caches):
             w = layer["width"]
@@ -574,7 +595,7 @@ def bench_prompt_then_generate(ctx, n_new=256):
                                                 want_val=False)
         choose(norm[last].contiguous())   # NormalizeState of each prompt's last token, made by the last product
     def step():
-        ctx.embed_rows(labels, embed, 0.03, out=state)
+        ctx.embed_rows(labels, embed, embed_scale, out=state)
         pending = None
         for layer, c in zip(m.layers, m.caches):
             _, pending = add_lookup_product(ctx, layer, c, t, m.rope, state, workspace=room, scratch=keep, pending=pending, defer=True)

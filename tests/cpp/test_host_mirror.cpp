@@ -178,7 +178,7 @@ static int RunCase(int dtype, int window, float slope)
 static int RunLayerCase(int width, float slope, int headDim, bool oneProjectionMatrix)
 {
     const int B = 5, H = 4, d = headDim, dim = 512, steps = 7, maxLen = 16;
-    const int qsum = H * d, kvDim = qsum * 4, reluDim = H * d;
+    const int qsum = H * d, kvDim = qsum * 4, reluDim = H * 128; // GetReluDim(): 128 per head whatever the head width
     TModelDims dims;
     dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim;
     unsigned seed = 99u + width * 3 + headDim;
@@ -298,7 +298,7 @@ struct TLayerData {
 
     TLayerData(const TModelDims &dims, int width, float slope, unsigned &seed)
     {
-        const int dim = dims.Dim, qsum = dims.GetQSum(), kvDim = qsum * 4, reluDim = qsum;
+        const int dim = dims.Dim, qsum = dims.GetQSum(), kvDim = qsum * 4, reluDim = dims.GetReluDim();
         auto randMatrix = [&](size_t n) {
             std::vector<int8_t> m(n);
             for (auto &x : m) x = tso_float_to_i8(Gauss(seed) * 32.0f);

@@ -55,6 +55,8 @@ struct TModelDims {
     int QDim = 128;
     int TTDim = 128;
     int HeadCount = 1;
+    int ReluMult = 1; // feed-forward width in units of 128 per head (gpt/model_params/model_dim.h:66)
+    int GetReluDim() const { return HeadCount * 128 * ReluMult; }
     int GetQSum() const { return QDim * HeadCount; }
     int GetTTSum() const { return TTDim * HeadCount; }
 };
@@ -153,7 +155,7 @@ constexpr int COMBINER_REP = 4;        // gpt/model_params/model_dim.h:12
 // per token call: the four projections are one product when QK, QV, K and V lie one after the other in memory, the
 // normalisations that follow them are one call, K-split products leave their parts for the consumer to add up, and the
 // combiner's AddScaled is done by the normalisation after it.  QDim == TTDim == 64 or 128; the feed-forward width is
-// reluDim = HeadCount * QDim (ReluMult 1 at QDim 128).
+// reluDim = HeadCount * 128 * ReluMult with ReluMult 1.
 struct TInferModel; // below
 
 class TLayerComputer
