@@ -45,6 +45,12 @@ static float Gauss(unsigned &s)
     return u - 6.0f;
 }
 
+static unsigned Rand(unsigned &s)
+{
+    s = s * 1664525u + 1013904223u;
+    return s >> 8;
+}
+
 static int RunCase(int dtype, int window, float slope)
 {
     const int H = 2, d = 128;
@@ -573,9 +579,150 @@ static int RunPredictionCase()
     return fails;
 }
 
+// TComputeContext, the forward half of the reference's IComputeContext: a batch of two fragments built with
+// TNodesBatch::AddSample (one span list per attention width, some nodes with two embedding labels), Init, then
+// ComputeFragmentPredictions / ComputeScore / ComputeFinalStateVectors against the oracle's token-by-token pass of the
+// same three layers (each fragment on its own cache rows; a node's position is its index in the batch).
+static int RunContextCase(int firstLayer, int nLayers)
+{
+    const int B = 2, H = 2, d = 128, dim = 256, vocab = 512, maxLen = 64;
+    const int fragLen[B] = {24, 40};
+    const int len = fragLen[0] + fragLen[1];
+    TModelDims dims;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim;
+    unsigned seed = 20252u;
+    tsattn_config cfg = {};
+    cfg.device = 0; cfg.max_seqs = B; cfg.max_heads = H; cfg.max_head_dim = d;
+    tsattn_handle_t handle = nullptr;
+    if (tsattn_create(&cfg, &handle) != TSATTN_OK) { printf("tsattn_create: %s\n", tsattn_last_error()); return 1; }
+    int fails = 0;
+    {
+        const int widths[3] = {1, 4, 1000};
+        const float slopes[3] = {0.0f, 0.5f, 0.0f};
+        std::vector<std::unique_ptr<TLayerData>> layers;
+        std::vector<TCpuCache> cpuCaches;
+        TInferModel model;
+        std::vector<int> widthId;
+        for (int l = firstLayer; l < firstLayer + nLayers; ++l) {
+            layers.emplace_back(new TLayerData(dims, widths[l], slopes[l], seed));
+            cpuCaches.emplace_back(B, H, maxLen, d);
+            model.LayerArr.push_back(layers.back()->Att);
+            widthId.push_back(l);
+        }
+        std::vector<int8_t> embed((size_t)vocab * dim), finalLayer((size_t)vocab * dim);
+        for (auto &x : embed) x = tso_float_to_i8(Gauss(seed) * 32.0f);
+        for (auto &x : finalLayer) x = tso_float_to_i8(Gauss(seed) * 32.0f);
+        std::vector<float> bias(vocab);
+        for (auto &x : bias) x = Gauss(seed) * 0.5f;
+        int8_t *embedDev = ToDevice(embed), *finalDev = ToDevice(finalLayer);
+        float *biasDev = ToDevice(bias);
+        model.LabelEmbed = embedDev; model.LabelEmbedScale = 0.04f; model.LabelCount = vocab;
+        model.FinalLayer = finalDev; model.FinalLayerScale = 0.08f; model.VocabSize = vocab; model.Bias = biasDev;
+
+        TComputeContext ctx(handle, dims, model, widthId, 3, 128, 2);
+        // the batch: every node's labels, spans for each of the three widths, the next token as its target
+        TNodesBatch &nodes = ctx.GetNodes(0);
+        nodes.Init(3);
+        std::vector<int32_t> labels((size_t)len * 2, -1); // the same as rows of two slots, for the oracle
+        std::vector<int32_t> token(len);
+        for (int i = 0; i < len; ++i) token[i] = (int32_t)(Rand(seed) % vocab);
+        for (int b = 0, ptr = 0; b < B; ptr += fragLen[b], ++b) {
+            TAttentionInfo att[3];
+            for (int k = 0; k < 3; ++k) {
+                att[k].Init();
+                AddWindowSpans(ptr, fragLen[b], widths[k], nullptr, &att[k]);
+            }
+            for (int i = 0; i < fragLen[b]; ++i) {
+                const int node = ptr + i;
+                std::vector<int32_t> nodeLabels = {token[node]};
+                if (i % 5 == 0) nodeLabels.push_back((int32_t)(1 + (node * 7) % (vocab - 1))); // a second label on some nodes
+                for (size_t j = 0; j < nodeLabels.size(); ++j) labels[(size_t)node * 2 + j] = nodeLabels[j];
+                std::vector<std::vector<TAttentionSpan>> spans(3);
+                for (int k = 0; k < 3; ++k)
+                    for (int j = att[k].SpanPtr[i]; j < att[k].SpanPtr[i + 1]; ++j) spans[k].push_back(att[k].Spans[j]);
+                nodes.AddSample(node, nodeLabels, spans);
+                if (i + 1 < fragLen[b]) nodes.Target.push_back(TNodeTarget(node, token[node + 1]));
+            }
+        }
+        ctx.Init(0, TComputeContext::INIT_TEST);
+        std::vector<std::vector<float>> pred, finalState;
+        ctx.ComputeFragmentPredictions(&pred);
+        std::vector<float> targetProb;
+        ctx.ComputeFragmentPredictions(&targetProb);
+        const float score = ctx.ComputeScore();
+        ctx.ComputeFinalStateVectors(&finalState);
+
+        // the oracle's pass
+        std::vector<float> rope((size_t)128 * d), state((size_t)len * dim), want((size_t)len * vocab);
+        tsattn_fill_rope_table(d, 128, rope.data());
+        tso_embed_rows(len, dim, labels.data(), 2, embed.data(), vocab, model.LabelEmbedScale, state.data());
+        for (int l = 0; l < nLayers; ++l) {
+            TCpuCache &cpu = cpuCaches[l];
+            for (int b = 0, ptr = 0; b < B; ptr += fragLen[b], ++b) {
+                for (int i = 0; i < fragLen[b]; ++i) {
+                    int32_t t = ptr + i;
+                    const size_t off = (size_t)b * H * maxLen;
+                    tso_add_lookup_product(&layers[l]->L, 1, &t, rope.data(), &state[(size_t)t * dim], cpu.K.data() + off * d, cpu.V.data() + off * d,
+                                           (int64_t)H * maxLen * d, (int64_t)maxLen * d, d, cpu.KScale.data() + off, (int64_t)H * maxLen, maxLen,
+                                           &cpu.Len[b], maxLen, nullptr, 4);
+                }
+            }
+        }
+        std::vector<uint8_t> norm((size_t)len * dim);
+        std::vector<float> tileScale(dim / STATE_NORM_TILE);
+        for (int r = 0; r < len; ++r) tso_normalize_heads(TSO_I8, &state[(size_t)r * dim], dim, dim / STATE_NORM_TILE, VEC_SCALE, &norm[(size_t)r * dim], tileScale.data());
+        std::vector<int32_t> logits((size_t)len * vocab), wantChoice(len);
+        tso_matmul_i8((const int8_t *)norm.data(), dim, finalLayer.data(), dim, len, vocab, dim, 0, 0.0f, logits.data(), vocab);
+        const float finalScale = sqrtf(1.0f / (float)dim) * (1.0f / 0.693147f) * model.FinalLayerScale * VEC_SCALE;
+        tso_softmax_rows(len, vocab, logits.data(), finalScale, bias.data(), 0, want.data(), wantChoice.data());
+
+        double maxProb = 0, meanProb = 0, maxState = 0, rmsState = 0, rms = 0, wantScore = 0;
+        for (float x : state) rms += (double)x * x;
+        rms = sqrt(rms / state.size());
+        if ((int)pred.size() != len || (int)finalState.size() != len || (int)targetProb.size() != len) { printf("  result sizes\n"); ++fails; }
+        for (int r = 0; r < len && !fails; ++r) {
+            double sum = 0;
+            for (int k = 0; k < vocab; ++k) {
+                const double e = fabs((double)pred[r][k] - want[(size_t)r * vocab + k]) / (want[(size_t)r * vocab + k] + 1e-3);
+                maxProb = fmax(maxProb, e);
+                meanProb += e / ((double)len * vocab);
+                sum += pred[r][k];
+            }
+            if (fabs(sum - 1) > 1e-4) { printf("  probabilities of node %d sum to %.6f\n", r, sum); ++fails; }
+            for (int x = 0; x < dim; ++x) {
+                const double e = fabs((double)finalState[r][x] - state[(size_t)r * dim + x]) / rms;
+                maxState = fmax(maxState, e);
+                rmsState += e * e / ((double)len * dim);
+            }
+        }
+        for (const TNodeTarget &nt : nodes.Target) {
+            wantScore += log(want[(size_t)nt.Node * vocab + nt.TargetId]);
+            if (!fails && targetProb[nt.Node] != pred[nt.Node][nt.TargetId]) { printf("  target probability of node %d\n", (int)nt.Node); ++fails; }
+        }
+        wantScore /= (double)nodes.Target.size();
+        rmsState = sqrt(rmsState);
+        // The batch form against the token form: the attention outputs differ within the prefill tolerance (f16 weights),
+        // which flips single int8 roundings of KVProduct and of the normalisations that follow; every further layer
+        // amplifies what it is given and adds its own flips.  The states here are small (the embedding of one or two
+        // labels, rms 1.3), so a flip weighs more than in the prompt-layer cases above.  Bounds at about twice what is
+        // measured (one layer: probabilities 0.17 / 5e-3, state 3.4e-2 / 6e-3; three: 0.23 / 1.1e-2, 8e-2 / 1.9e-2); the
+        // score, the quantity the reference's own check compares (cpu_infer.cpp:625-685), within 1e-2.
+        const double widen = nLayers == 1 ? 1.0 : 2.5;
+        if (maxProb > 0.3 * widen || meanProb > 1e-2 * widen || maxState > 7e-2 * widen || rmsState > 1.2e-2 * widen || fabs(score - wantScore) > 1e-2) ++fails;
+        printf("TComputeContext: %d nodes in %d fragments, %d layer(s) from width %d, vocabulary %d: |p - p_oracle| / (p_oracle + 1e-3) max %.2e mean %.2e, "
+               "final state error / rms max %.2e rms %.2e, score %.4f (oracle %.4f)  %s\n", len, B, nLayers, widths[firstLayer], vocab, maxProb, meanProb,
+               maxState, rmsState, score, wantScore, fails ? "FAIL" : "ok");
+        for (void *p : {(void *)embedDev, (void *)finalDev, (void *)biasDev}) HIP_OK(hipFree(p));
+    }
+    tsattn_destroy(handle);
+    return fails;
+}
+
 int main()
 {
     int fails = 0;
+    for (int l = 0; l < 3; ++l) fails += RunContextCase(l, 1);
+    fails += RunContextCase(0, 3);
     fails += RunPromptLayerCase(1000, 0.0f, 128);
     fails += RunPromptLayerCase(64, 0.5f, 128);
     fails += RunPromptLayerCase(1, 0.0f, 64);

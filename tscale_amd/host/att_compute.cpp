@@ -1,6 +1,8 @@
 #include "att_compute.h"
 
 #include <hip/hip_runtime.h>
+
+#include <algorithm>
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -27,6 +29,8 @@ static void CheckHip(hipError_t e, const char *what)
 {
     TS_VERIFY(e == hipSuccess, "%s failed: %s", what, hipGetErrorString(e));
 }
+
+static int FlattenSpans(const TAttentionInfo &attInfo, std::vector<int32_t> *pStart, std::vector<int32_t> *pFinish);
 
 void AddWindowSpans(int ptr, int len, int limitWindow, const uint8_t *docStartFlag, TAttentionInfo *pAtt)
 {
@@ -80,40 +84,9 @@ void TAttentionComputer::SetAttention(const TAttentionInfo &attInfo, void *strea
 {
     int len = (int)attInfo.GetSampleCount();
     TS_VERIFY(len <= MaxLen, "%d samples exceed the context's %d", len, MaxLen);
-    std::vector<int32_t> st(len), fi(len);
-    for (int t = 0; t < len; ++t) {
-        int a = attInfo.SpanPtr[t], b = attInfo.SpanPtr[t + 1];
-        TS_VERIFY(b - a <= 1, "row %d has %d spans; one span per row is supported", t, b - a);
-        if (b > a) {
-            st[t] = attInfo.Spans[a].Start;
-            fi[t] = attInfo.Spans[a].Finish;
-        } else {
-            st[t] = t;
-            fi[t] = t - 1;
-        }
-    }
+    std::vector<int32_t> st, fi;
+    CausalPeriod = FlattenSpans(attInfo, &st, &fi); // (and the launch-order hint)
     Len = len;
-    // Launch-order hint: rows without keys mark sequence starts; if they are equally spaced, cover the batch and
-    // the window is wide (the last row of a sequence sees at least half of it), the batch has a causal period.
-    CausalPeriod = 0;
-    {
-        int period = 0, last = -1;
-        bool regular = len > 0 && fi[0] < st[0];
-        for (int t = 0; t < len && regular; ++t) {
-            if (fi[t] < st[t]) {
-                if (last >= 0) {
-                    if (period == 0) period = t - last;
-                    else if (t - last != period) regular = false;
-                }
-                last = t;
-            }
-        }
-        if (regular && period == 0) period = len; // a single sequence
-        if (regular && period > 0 && len % period == 0 && last == len - period) {
-            const int tail = len - 1;
-            if (fi[tail] - st[tail] + 1 >= period / 2) CausalPeriod = period;
-        }
-    }
     // pageable source: the copy has returned from the host's point of view when the call returns
     CheckHip(hipMemcpyAsync(SpanStart, st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
     CheckHip(hipMemcpyAsync(SpanFinish, fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
@@ -460,9 +433,8 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
                                             const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
                                             void *stream, bool deferStateUpdate)
 {
-    TAttentionVecHistory &kvCache = *pKVCache;
     const int headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
-    TS_VERIFY(kvCache.HeadCount == headCount && kvCache.HeadDim == headDim && kvCache.DType == TSATTN_I8,
+    TS_VERIFY(!pKVCache || (pKVCache->HeadCount == headCount && pKVCache->HeadDim == headDim && pKVCache->DType == TSATTN_I8),
               "the KV cache does not match the layer (%d heads of %d, int8)", headCount, headDim);
     Projections(len, pos, ropeBuf, ropeLen, att, true, state, stream);
     const uint8_t *qk = Q4, *qv = Q4 + qsum, *v = Q4 + 3 * (size_t)qsum;
@@ -481,7 +453,9 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
     pa.kv_k = Q4 + 2 * (size_t)qsum; pa.kv_k_pitch = pitch4; pa.kv_out = Kv; pa.kv_out_pitch = (int64_t)qsum * COMBINER_REP;
     pa.kv_rep = COMBINER_REP; pa.kv_mult = 1.0f;
     Check(tsattn_prefill(Handle, &pa, stream), "tsattn_prefill");
-    // kvCache.AddVectors for every token at once
+    // kvCache.AddVectors for every token at once (a forward pass over fragments that nobody continues has no cache)
+    if (pKVCache) {
+    TAttentionVecHistory &kvCache = *pKVCache;
     tsattn_fill_args fa = {};
     fa.n_seqs = kvCache.SeqCount; fa.n_heads = headCount; fa.head_dim = headDim; fa.n_tokens = len;
     fa.seq_offset = seqOffset; fa.k = qv; fa.v = v; fa.pitch = pitch4;
@@ -494,6 +468,7 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
     fa.s_seq_stride = (int64_t)headCount * kvCache.MaxLen; fa.s_head_stride = kvCache.MaxLen;
     fa.cache_len = kvCache.Length; fa.max_len = kvCache.MaxLen;
     Check(tsattn_cache_fill(Handle, &fa, stream), "tsattn_cache_fill");
+    }
     AfterAttention(len, att, true, deferStateUpdate, state, stream);
 }
 
@@ -524,6 +499,210 @@ void SampleFromDistr(tsattn_handle_t handle, int rows, int64_t vocabSize, const 
 {
     Check(tsattn_sample_rows(handle, rows, vocabSize, prediction, vocabSize, temperature, nullptr, 0, seed, offset, choice, stream),
           "tsattn_sample_rows");
+}
+
+// ---- TNodesBatch, TComputeContext ----------------------------------------------------------------------------------
+
+void TNodesBatch::Init(int attentionWidthCount)
+{
+    SampleIndex.resize(0);
+    LabelArr.resize(0);
+    LabelPtr.assign(1, 0u);
+    Target.resize(0);
+    AttArr.resize(attentionWidthCount);
+    for (TAttentionInfo &att : AttArr) att.Init();
+}
+
+void TNodesBatch::AddSample(int idx, const std::vector<int32_t> &labels, const std::vector<std::vector<TAttentionSpan>> &attSpansArr)
+{
+    SampleIndex.push_back(idx);
+    LabelArr.insert(LabelArr.end(), labels.begin(), labels.end());
+    LabelPtr.push_back((uint32_t)LabelArr.size());
+    TS_VERIFY(AttArr.size() == attSpansArr.size(), "%d span lists for %d attention widths", (int)attSpansArr.size(), (int)AttArr.size());
+    for (size_t k = 0; k < AttArr.size(); ++k) {
+        for (const TAttentionSpan &span : attSpansArr[k]) AttArr[k].AddSpan(span);
+        AttArr[k].AddSample();
+    }
+}
+
+// One inclusive span per row (rows without keys: an empty one) from the reference's span lists, and the launch-order
+// hint: rows without keys mark fragment starts; if they are equally spaced, cover the batch and the window is wide
+// (the last row of a fragment sees at least half of it), the batch has a causal period.
+static int FlattenSpans(const TAttentionInfo &attInfo, std::vector<int32_t> *pStart, std::vector<int32_t> *pFinish)
+{
+    const int len = (int)attInfo.GetSampleCount();
+    std::vector<int32_t> &st = *pStart, &fi = *pFinish;
+    st.resize(len);
+    fi.resize(len);
+    for (int t = 0; t < len; ++t) {
+        const int a = attInfo.SpanPtr[t], b = attInfo.SpanPtr[t + 1];
+        TS_VERIFY(b - a <= 1, "row %d has %d spans; one span per row is supported", t, b - a);
+        if (b > a) {
+            st[t] = attInfo.Spans[a].Start;
+            fi[t] = attInfo.Spans[a].Finish;
+        } else {
+            st[t] = t;
+            fi[t] = t - 1;
+        }
+    }
+    int period = 0, last = -1;
+    bool regular = len > 0 && fi[0] < st[0];
+    for (int t = 0; t < len && regular; ++t) {
+        if (fi[t] < st[t]) {
+            if (last >= 0) {
+                if (period == 0) period = t - last;
+                else if (t - last != period) regular = false;
+            }
+            last = t;
+        }
+    }
+    if (regular && period == 0) period = len; // a single fragment
+    if (regular && period > 0 && len % period == 0 && last == len - period) {
+        const int tail = len - 1;
+        if (fi[tail] - st[tail] + 1 >= period / 2) return period;
+    }
+    return 0;
+}
+
+TComputeContext::TComputeContext(tsattn_handle_t handle, const TModelDims &dims, const TInferModel &model, const std::vector<int> &layerWidthId,
+                                 int attentionWidthCount, int maxNodeCount, int maxLabelsPerNode)
+    : Handle(handle), Dims(dims), Model(model), LayerWidthId(layerWidthId), AttentionWidthCount(attentionWidthCount), MaxNodeCount(maxNodeCount),
+      MaxLabelsPerNode(maxLabelsPerNode), Layer(handle, dims, maxNodeCount, model.VocabSize)
+{
+    TS_VERIFY(layerWidthId.size() == model.LayerArr.size(), "%d width ids for %d layers", (int)layerWidthId.size(), (int)model.LayerArr.size());
+    for (int id : layerWidthId) TS_VERIFY(id >= 0 && id < attentionWidthCount, "attention width id %d of %d", id, attentionWidthCount);
+    TS_VERIFY(maxNodeCount > 0 && maxLabelsPerNode > 0, "empty context");
+    Nodes.Init(attentionWidthCount);
+    const size_t n = (size_t)maxNodeCount;
+    CheckHip(hipMalloc((void **)&Labels, n * maxLabelsPerNode * sizeof(int32_t)), "hipMalloc(labels)");
+    CheckHip(hipMalloc((void **)&Pos, n * sizeof(int32_t)), "hipMalloc(positions)");
+    CheckHip(hipMalloc((void **)&State, n * dims.Dim * sizeof(float)), "hipMalloc(state)");
+    CheckHip(hipMalloc((void **)&Prediction, n * (size_t)model.VocabSize * sizeof(float)), "hipMalloc(prediction)");
+    CheckHip(hipMalloc((void **)&RopeBuf, n * dims.QDim * sizeof(float)), "hipMalloc(rope table)");
+    SpanStart.assign(attentionWidthCount, nullptr);
+    SpanFinish.assign(attentionWidthCount, nullptr);
+    SpanTiles.assign(attentionWidthCount, nullptr);
+    CausalPeriod.assign(attentionWidthCount, 0);
+    for (int k = 0; k < attentionWidthCount; ++k) {
+        CheckHip(hipMalloc((void **)&SpanStart[k], n * sizeof(int32_t)), "hipMalloc(spans)");
+        CheckHip(hipMalloc((void **)&SpanFinish[k], n * sizeof(int32_t)), "hipMalloc(spans)");
+        CheckHip(hipMalloc((void **)&SpanTiles[k], ((n + 127) / 128) * 32 * sizeof(int32_t)), "hipMalloc(span summary)");
+    }
+    // FillRopeBuf for every node index of the largest batch, and the nodes' positions (their indices), once
+    std::vector<float> rope(n * dims.QDim);
+    tsattn_fill_rope_table(dims.QDim, maxNodeCount, rope.data());
+    std::vector<int32_t> pos(n);
+    for (size_t i = 0; i < n; ++i) pos[i] = (int32_t)i;
+    CheckHip(hipMemcpy(RopeBuf, rope.data(), rope.size() * sizeof(float), hipMemcpyHostToDevice), "rope table copy");
+    CheckHip(hipMemcpy(Pos, pos.data(), n * sizeof(int32_t), hipMemcpyHostToDevice), "position copy");
+}
+
+TComputeContext::~TComputeContext()
+{
+    for (void *p : {(void *)Labels, (void *)Pos, (void *)State, (void *)Prediction, (void *)RopeBuf}) (void)hipFree(p);
+    for (int k = 0; k < AttentionWidthCount; ++k) {
+        (void)hipFree(SpanStart[k]);
+        (void)hipFree(SpanFinish[k]);
+        (void)hipFree(SpanTiles[k]);
+    }
+}
+
+TNodesBatch &TComputeContext::GetNodes(int deviceId)
+{
+    TS_VERIFY(deviceId == 0, "device %d of 1", deviceId);
+    return Nodes;
+}
+
+// Per batch: the nodes' labels and every width's spans go to the device (gpt_cpu.cpp:862-883, gpt_cuda.cu:1350-1376).
+void TComputeContext::Init(int deviceId, EInitType initType)
+{
+    (void)initType; // (no dropout on this path: a training batch is computed like a test batch)
+    TS_VERIFY(deviceId == 0, "device %d of 1", deviceId);
+    const int len = Nodes.GetNodeCount();
+    TS_VERIFY(len <= MaxNodeCount, "%d nodes exceed the context's %d", len, MaxNodeCount);
+    TS_VERIFY((int)Nodes.LabelPtr.size() == len + 1 && (int)Nodes.AttArr.size() == AttentionWidthCount, "inconsistent batch");
+    Len = len;
+    KeepTarget = Nodes.Target;
+    // labels as rows of equal width; unused slots hold -1 (an empty slot for the embedding)
+    int perRow = 1;
+    for (int i = 0; i < len; ++i) perRow = std::max(perRow, (int)(Nodes.LabelPtr[i + 1] - Nodes.LabelPtr[i]));
+    TS_VERIFY(perRow <= MaxLabelsPerNode, "%d labels on a node exceed the context's %d", perRow, MaxLabelsPerNode);
+    LabelsPerRow = perRow;
+    std::vector<int32_t> labels((size_t)len * perRow, -1);
+    for (int i = 0; i < len; ++i)
+        for (uint32_t j = Nodes.LabelPtr[i]; j < Nodes.LabelPtr[i + 1]; ++j) labels[(size_t)i * perRow + (j - Nodes.LabelPtr[i])] = Nodes.LabelArr[j];
+    if (len > 0) CheckHip(hipMemcpy(Labels, labels.data(), labels.size() * sizeof(int32_t), hipMemcpyHostToDevice), "label copy");
+    std::vector<int32_t> st, fi;
+    for (int k = 0; k < AttentionWidthCount; ++k) {
+        TS_VERIFY((int)Nodes.AttArr[k].GetSampleCount() == len, "span list %d has %d samples for %d nodes", k, (int)Nodes.AttArr[k].GetSampleCount(), len);
+        CausalPeriod[k] = FlattenSpans(Nodes.AttArr[k], &st, &fi);
+        if (len == 0) continue;
+        CheckHip(hipMemcpy(SpanStart[k], st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice), "span copy");
+        CheckHip(hipMemcpy(SpanFinish[k], fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice), "span copy");
+        Check(tsattn_build_span_tiles(Handle, len, SpanStart[k], SpanFinish[k], SpanTiles[k], nullptr), "tsattn_build_span_tiles");
+    }
+    CheckHip(hipDeviceSynchronize(), "batch set-up");
+}
+
+// ComputeForward (gpt_cpu.cpp:886-938) up to the normalised final state
+const uint8_t *TComputeContext::ComputeForward(void *stream)
+{
+    TS_VERIFY(Len > 0, "Init() with a non-empty batch comes first");
+    const int dim = Dims.Dim;
+    Check(tsattn_embed_rows(Handle, Len, dim, Labels, LabelsPerRow, Model.LabelEmbed, dim, Model.LabelCount, Model.LabelEmbedScale, State, dim, stream),
+          "tsattn_embed_rows");
+    for (size_t d = 0; d < Model.LayerArr.size(); ++d) {
+        const int k = LayerWidthId[d];
+        Layer.AddLookupProductPrompt(Len, nullptr, Pos, RopeBuf, MaxNodeCount, Model.LayerArr[d], SpanStart[k], SpanFinish[k], SpanTiles[k],
+                                     CausalPeriod[k], nullptr, State, stream, true);
+    }
+    return Layer.FlushState(Len, State, stream);
+}
+
+void TComputeContext::ComputeFinalStateVectors(std::vector<std::vector<float>> *pStateVectors)
+{
+    ComputeForward(nullptr);
+    std::vector<float> flat((size_t)Len * Dims.Dim);
+    CheckHip(hipMemcpy(flat.data(), State, flat.size() * sizeof(float), hipMemcpyDeviceToHost), "state copy");
+    pStateVectors->resize(Len);
+    for (int i = 0; i < Len; ++i) (*pStateVectors)[i].assign(flat.begin() + (size_t)i * Dims.Dim, flat.begin() + (size_t)(i + 1) * Dims.Dim);
+}
+
+void TComputeContext::ComputeFragmentPredictions(std::vector<std::vector<float>> *pPrediction)
+{
+    const uint8_t *norm = ComputeForward(nullptr);
+    const int dim = Dims.Dim;
+    const int64_t vocab = Model.VocabSize;
+    const int planes = Layer.MulForwardPlanes(Len, norm, dim, Model.FinalLayer, (int)vocab, nullptr);
+    // finalScale = CalcDotScale(dim) * CalcFinalLayerMult() * params.FinalLayerScale * VEC_SCALE (cpu_infer.cpp:574-579)
+    const float finalScale = sqrtf(1.0f / (float)dim) * (1.0f / 0.693147f) * Model.FinalLayerScale * VEC_SCALE;
+    Check(tsattn_softmax_rows(Handle, Len, vocab, Layer.Planes, planes, (int64_t)Len * vocab, vocab, finalScale, Model.Bias, Prediction, vocab, nullptr,
+                              nullptr), "tsattn_softmax_rows");
+    std::vector<float> flat((size_t)Len * vocab);
+    CheckHip(hipMemcpy(flat.data(), Prediction, flat.size() * sizeof(float), hipMemcpyDeviceToHost), "prediction copy");
+    pPrediction->resize(Len);
+    for (int i = 0; i < Len; ++i) (*pPrediction)[i].assign(flat.begin() + (size_t)i * vocab, flat.begin() + (size_t)(i + 1) * vocab);
+}
+
+void TComputeContext::ComputeFragmentPredictions(std::vector<float> *pPrediction)
+{
+    std::vector<std::vector<float>> prediction;
+    ComputeFragmentPredictions(&prediction);
+    pPrediction->assign(prediction.size(), 0.0f);
+    for (const TNodeTarget &nt : KeepTarget) (*pPrediction)[nt.Node] = prediction[nt.Node][nt.TargetId];
+}
+
+float TComputeContext::ComputeScore()
+{
+    std::vector<std::vector<float>> prediction;
+    ComputeFragmentPredictions(&prediction);
+    double sum = 0;
+    int64_t count = 0;
+    for (const TNodeTarget &nt : KeepTarget) {
+        sum += log(prediction[nt.Node][nt.TargetId]);
+        count += 1;
+    }
+    return (float)(sum / (double)count);
 }
 
 } // namespace NTsAttn

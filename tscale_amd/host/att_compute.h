@@ -12,6 +12,8 @@
 //   AddLookupProduct                       gpt/train/cpu_infer.cpp:465-527            TLayerComputer::AddLookupProduct(Prompt)
 //   ComputePrediction                      gpt/train/cpu_infer.cpp:552-582            NTsAttn::ComputePrediction
 //   SampleFromDistr                        gpt/train/cpu_infer.cpp:585-599            NTsAttn::SampleFromDistr
+//   TNodeTarget / TNodesBatch              gpt/att/nodes_batch.h:10-36                NTsAttn::TNodeTarget / TNodesBatch
+//   IComputeContext (the forward half)     gpt/compute/model.h:55-155                 NTsAttn::TComputeContext
 //
 // All arithmetic runs in libtsattn.so through the C ABI of include/tsattn.h; this layer owns the
 // per-context device buffers (allocated once, like TAttentionComputeCtx::AllocateCuda,
@@ -181,6 +183,7 @@ class TLayerComputer
     void NormalizeState(int rows, float *state, void *stream);
     friend void ComputePrediction(TLayerComputer &, const TInferModel &, const std::vector<TAttentionVecHistory *> &, const int32_t *,
                                   const int32_t *, const float *, int64_t, float *, float *, int32_t *, void *);
+    friend class TComputeContext;
 
   public:
     // maxOutputs: the widest matrix product a caller will run through this object's buffers (the vocabulary size for
@@ -203,7 +206,8 @@ class TLayerComputer
     const uint8_t *FlushState(int rows, float *state, void *stream);
     // len tokens of the cache's sequences, concatenated (seqOffset: device int32 [seqCount + 1]); pos: device int32 [len],
     // each token's position in its sequence; spans (and optionally their summary and the launch-order hint) of
-    // att.AttentionWidth as for tsattn_prefill; state: device [len][Dim]; the tokens' rows are appended to the cache.
+    // att.AttentionWidth as for tsattn_prefill; state: device [len][Dim]; the tokens' rows are appended to the cache
+    // (pKVCache and seqOffset may be null: nothing is kept for later tokens).
     void AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
                                 const TAttentionMatrices &att, const int32_t *spanStart, const int32_t *spanFinish,
                                 const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
@@ -239,5 +243,75 @@ void ComputePrediction(TLayerComputer &layer, const TInferModel &model, const st
 // same choices; advance offset by rows * vocabSize per call), not from the reference's MT19937 stream.
 void SampleFromDistr(tsattn_handle_t handle, int rows, int64_t vocabSize, const float *prediction, float temperature, uint64_t seed,
                      uint64_t offset, int32_t *choice, void *stream);
+
+// The batch a context computes on, filled by the caller exactly as the reference's MakeTest / MakeTrain fill theirs
+// (gpt/att/nodes_batch.h:10-36, nodes_batch.cpp:5-31): a node is one token position of one fragment; LabelArr /
+// LabelPtr hold every node's embedding labels, AttArr one span list per attention width of the model, Target the
+// (node, label) pairs whose probability is asked for.
+struct TNodeTarget {
+    int64_t Node = 0;
+    int64_t TargetId = 0;
+    TNodeTarget() {}
+    TNodeTarget(int64_t nodeId, int64_t targetId) : Node(nodeId), TargetId(targetId) {}
+};
+
+struct TNodesBatch {
+    std::vector<int32_t> LabelArr;
+    std::vector<uint32_t> LabelPtr;
+    std::vector<int> SampleIndex;
+    std::vector<TNodeTarget> Target;
+    std::vector<TAttentionInfo> AttArr;
+
+    void Init(int attentionWidthCount);
+    void AddSample(int idx, const std::vector<int32_t> &labels, const std::vector<std::vector<TAttentionSpan>> &attSpansArr);
+    int GetNodeCount() const { return (int)SampleIndex.size(); }
+};
+
+// The forward half of the reference's IComputeContext (gpt/compute/model.h:55-155; its CPU form
+// gpt/compute/gpt_cpu.cpp:795-967) over the int8 model: fill GetNodes(0), Init(0, INIT_TEST), then
+// ComputeFragmentPredictions / ComputeFinalStateVectors / ComputeScore, which run the batch form of every layer
+// (AddLookupProductPrompt on the spans of the layer's attention width; a node's RoPE position is its index in the
+// batch, gpt/att/rope.cpp:53-62).  One device; nothing of the training half (Backprop, the gradient and parameter
+// accessors) exists here.
+class TComputeContext
+{
+  public:
+    enum EInitType { INIT_TRAIN, INIT_TEST };
+
+  private:
+    tsattn_handle_t Handle = nullptr;
+    TModelDims Dims;
+    TInferModel Model;
+    std::vector<int> LayerWidthId; // per layer: which of the batch's span lists it attends over (AttentionWidthId)
+    int AttentionWidthCount = 0, MaxNodeCount = 0, MaxLabelsPerNode = 0;
+    TLayerComputer Layer;
+    TNodesBatch Nodes;
+    std::vector<TNodeTarget> KeepTarget;
+    int Len = 0, LabelsPerRow = 1;
+    int32_t *Labels = nullptr, *Pos = nullptr;
+    std::vector<int32_t *> SpanStart, SpanFinish, SpanTiles; // per attention width, device
+    std::vector<int> CausalPeriod;
+    float *State = nullptr, *RopeBuf = nullptr, *Prediction = nullptr;
+
+    const uint8_t *ComputeForward(void *stream); // returns NormalizeState of the final state (device)
+
+  public:
+    // model: device copies of the int8 matrices, one TAttentionMatrices per layer; layerWidthId[d] in
+    // [0, attentionWidthCount).  maxLabelsPerNode bounds LabelPtr[i + 1] - LabelPtr[i].
+    TComputeContext(tsattn_handle_t handle, const TModelDims &dims, const TInferModel &model, const std::vector<int> &layerWidthId,
+                    int attentionWidthCount, int maxNodeCount, int maxLabelsPerNode = 1);
+    ~TComputeContext();
+    TComputeContext(const TComputeContext &) = delete;
+    TComputeContext &operator=(const TComputeContext &) = delete;
+
+    int GetDeviceCount() const { return 1; }
+    const TModelDims &GetModelDims() const { return Dims; }
+    TNodesBatch &GetNodes(int deviceId);
+    void Init(int deviceId, EInitType initType);
+    void ComputeFinalStateVectors(std::vector<std::vector<float>> *pStateVectors);
+    void ComputeFragmentPredictions(std::vector<std::vector<float>> *pPrediction);
+    void ComputeFragmentPredictions(std::vector<float> *pPrediction);
+    float ComputeScore();
+};
 
 } // namespace NTsAttn
