@@ -426,3 +426,36 @@ def test_prefill_fused_kv_product_argument_checks(ctx):
         ctx.compute_val_lookup(*args, kv_product=(kk, kv, 5, 1.0))
     with pytest.raises(capi.TsattnError):      # output rows too short
         ctx.compute_val_lookup(*args, kv_product=(kk, kv[:, :H * d * 2].contiguous(), 4, 1.0))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_prefill_arbitrary_spans(ctx, seed):
+    """Spans that no window mask makes: every row its own random [start, finish] anywhere in the batch (before it, after
+    it, across it), a fifth of the rows without keys, short and long ones mixed inside every 32-row group, so that the
+    tile classes a wave sees (not needed, cut at either end or both, fully inside) come in every order.  The reference
+    computes whatever TAttentionInfo lists (gpt/compute/gpt_cpu.cpp:391-441); so must the kernel, with and without the
+    span summary."""
+    rng = np.random.default_rng(7000 + seed)
+    dtype = [capi.I8, capi.E4M3][seed % 2]
+    d = [128, 64][(seed // 2) % 2]
+    H = int(rng.choice([1, 2, 4]))
+    n = int(rng.choice([97, 256, 300, 515, 777]))
+    slope = float(rng.choice([0.0, 0.25]))
+    st = rng.integers(0, n, n).astype(np.int32)
+    length = rng.choice([1, 2, 17, 40, 64, 65, 130, 300, n], n)
+    fi = np.minimum(st + length - 1, n - 1).astype(np.int32)
+    empty = rng.random(n) < 0.2
+    fi[empty] = st[empty] - 1
+    if seed >= 4:   # whole 32-row groups without keys, and one group that sees everything
+        fi[32:64] = st[32:64] - 1
+        st[64:96], fi[64:96] = 0, n - 1
+    q, qs, k, ks, v, vs = make_qkv(7100 + seed, n, H, d, dtype)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, slope)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    args = (dtype, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), t(st), t(fi), slope)
+    outs = [ctx.compute_val_lookup(*args).cpu().numpy(),
+            ctx.compute_val_lookup(*args, span_tiles=ctx.build_span_tiles(t(st), t(fi))).cpu().numpy()]
+    what = f"seed {seed}: dtype {dtype} d {d} H {H} n {n} slope {slope}"
+    assert np.array_equal(outs[0], outs[1]), what
+    assert_within_tolerance(outs[0], want, what)
+    assert not outs[0][fi < st].any(), what
