@@ -870,7 +870,42 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read before the next two blk overwrite it
         }
     }
-    if (row_ok && p.out) {
+    if constexpr (OUT_F16) {
+        if (p.out) {
+            // The result leaves through this wave's corner of LDS: a lane holds one query's row in pieces of four
+            // values, which stored directly would touch 32 rows per instruction, 16 bytes in each; staged, every store
+            // instruction writes four whole rows of the head (16 bytes per lane, consecutive), half as many of them.
+            constexpr int OUT_PITCH = D * 2 + 16;
+            static_assert(PF_WAVES * 32 * OUT_PITCH <= LDS_BYTES, "the waves' result rows fit into the tiles' LDS");
+            __syncthreads(); // every wave is done with the K and V tiles
+            // (computed from these copies, which the compiler cannot trace back: nothing of it is prepared before the
+            // tile loop and kept in registers through it)
+            int qi = lane & 31, g = lane >> 5, q0 = tile * PF_BM + wave * 32;
+#if defined(__HIP_DEVICE_COMPILE__)
+            asm volatile("" : "+v"(qi), "+v"(g), "+v"(q0));
+#endif
+            uint8_t *const stage = lds_raw + (q0 / 32 % PF_WAVES) * (32 * OUT_PITCH);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                for (int c4 = 0; c4 < 4; ++c4) {
+                    const int dcol = dt * 32 + 8 * c4 + 4 * g;
+                    const v4h hv = v4h{(_Float16)(o_acc[dt][c4 * 4 + 0] * inv), (_Float16)(o_acc[dt][c4 * 4 + 1] * inv),
+                                       (_Float16)(o_acc[dt][c4 * 4 + 2] * inv), (_Float16)(o_acc[dt][c4 * 4 + 3] * inv)};
+                    *(v4h *)(stage + qi * OUT_PITCH + dcol * 2) = hv;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's values are in LDS (nobody else reads them)
+            constexpr int ROW_CHUNKS = D * 2 / 16;
+#pragma unroll
+            for (int it = 0; it < 32 * ROW_CHUNKS / WAVE; ++it) {
+                const int id = it * WAVE + g * 32 + qi;
+                const int c = id % ROW_CHUNKS, r = id / ROW_CHUNKS;
+                const v4i w = *(const v4i *)(stage + r * OUT_PITCH + c * 16);
+                if (q0 + r < p.n_tokens) *(v4i *)((uint8_t *)p.out + (int64_t)(q0 + r) * p.out_pitch + hoff * 2 + c * 16) = w;
+            }
+        }
+    } else if (row_ok && p.out) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
