@@ -905,21 +905,37 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : TSATTN_PF_OCC) void prefi
                 if (q0 + r < p.n_tokens) *(v4i *)((uint8_t *)p.out + (int64_t)(q0 + r) * p.out_pitch + hoff * 2 + c * 16) = w;
             }
         }
-    } else if (row_ok && p.out) {
+    } else if (p.out) {
+        // the same for an f32 result, half of the head's columns at a time (a wave's corner of LDS holds 32 half rows)
+        constexpr int HALF = D / 2, OUT_PITCH = HALF * 4 + 16;
+        static_assert(PF_WAVES * 32 * OUT_PITCH <= LDS_BYTES, "the waves' result rows fit into the tiles' LDS");
+        __syncthreads(); // every wave is done with the K and V tiles (and with the rows a fused KVProduct staged)
+        int qi = lane & 31, g = lane >> 5, q0 = tile * PF_BM + wave * 32;
+#if defined(__HIP_DEVICE_COMPILE__)
+        asm volatile("" : "+v"(qi), "+v"(g), "+v"(q0));
+#endif
+        uint8_t *const stage = lds_raw + (q0 / 32 % PF_WAVES) * (32 * OUT_PITCH);
+        constexpr int ROW_CHUNKS = HALF * 4 / 16;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
+        for (int half = 0; half < 2; ++half) {
 #pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
-                const int dcol = dt * 32 + 8 * c4 + 4 * g;
-                float o0 = o_acc[dt][c4 * 4 + 0] * inv, o1 = o_acc[dt][c4 * 4 + 1] * inv;
-                float o2 = o_acc[dt][c4 * 4 + 2] * inv, o3 = o_acc[dt][c4 * 4 + 3] * inv;
-                if (OUT_F16) {
-                    v4h hv = v4h{(_Float16)o0, (_Float16)o1, (_Float16)o2, (_Float16)o3};
-                    *(v4h *)((uint8_t *)p.out + (int64_t)from * p.out_pitch + (hoff + dcol) * 2) = hv;
-                } else {
-                    *(v4f *)((uint8_t *)p.out + (int64_t)from * p.out_pitch + (hoff + dcol) * 4) = v4f{o0, o1, o2, o3};
+            for (int dt = half * (DT / 2); dt < (half + 1) * (DT / 2); ++dt) {
+#pragma unroll
+                for (int c4 = 0; c4 < 4; ++c4) {
+                    const int dcol = dt * 32 + 8 * c4 + 4 * g - half * HALF;
+                    *(v4f *)(stage + qi * OUT_PITCH + dcol * 4) =
+                        v4f{o_acc[dt][c4 * 4 + 0] * inv, o_acc[dt][c4 * 4 + 1] * inv, o_acc[dt][c4 * 4 + 2] * inv, o_acc[dt][c4 * 4 + 3] * inv};
                 }
             }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's values are in LDS (nobody else reads them)
+#pragma unroll
+            for (int it = 0; it < 32 * ROW_CHUNKS / WAVE; ++it) {
+                const int id = it * WAVE + g * 32 + qi;
+                const int c = id % ROW_CHUNKS, r = id / ROW_CHUNKS;
+                const v4i w = *(const v4i *)(stage + r * OUT_PITCH + c * 16);
+                if (q0 + r < p.n_tokens) *(v4i *)((uint8_t *)p.out + (int64_t)(q0 + r) * p.out_pitch + (hoff + half * HALF) * 4 + c * 16) = w;
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read before the second half overwrites it
         }
     }
     if (row_ok && p.sum_weight_log && g == 0) p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m_ref + __log2f(l_all);
