@@ -73,6 +73,7 @@ const char *tsattn_last_error(void);
  * Unlike Fp8Att, V is taken in the same [token][head*d] layout as Q and K: no transposed copy
  * (gpt_cuda.cu:501) is needed.
  */
+#define TSATTN_PREFILL_MAX_KV_PITCH ((int64_t)8 << 20)
 typedef struct tsattn_prefill_args {
     int dtype;                 /* tsattn_dtype of q, k, v */
     int out_dtype;             /* tsattn_out_dtype */
@@ -80,7 +81,8 @@ typedef struct tsattn_prefill_args {
     int n_heads;
     int head_dim;              /* 64 or 128 */
     const void *q, *k, *v;     /* [n_tokens][n_heads*head_dim] 8-bit */
-    int64_t q_pitch, k_pitch, v_pitch;   /* row pitch in bytes, multiple of 16 */
+    int64_t q_pitch, k_pitch, v_pitch;   /* row pitch in bytes, multiple of 16; k_pitch and v_pitch at most
+                                            TSATTN_PREFILL_MAX_KV_PITCH */
     const float *q_scale, *k_scale, *v_scale; /* [n_heads][n_tokens] or NULL = the constant below */
     int64_t scale_pitch;       /* floats between heads */
     float q_scale_const, k_scale_const, v_scale_const;

@@ -459,3 +459,44 @@ def test_prefill_arbitrary_spans(ctx, seed):
     assert np.array_equal(outs[0], outs[1]), what
     assert_within_tolerance(outs[0], want, what)
     assert not outs[0][fi < st].any(), what
+
+
+@pytest.mark.parametrize("dtype,d,H,n,window,slope", [
+    (capi.E4M3, 128, 1, 700, 10 ** 6, 0.0),   # common-tile path, 11 key tiles
+    (capi.I8, 64, 2, 600, 300, 0.25),         # windowed: the key range of the later workgroups starts far into the arrays
+    (capi.I8, 64, 2, 150, 10 ** 6, 0.0),      # d = 64, at most 192 keys: the path without a tile loop
+])
+def test_prefill_largest_key_row_pitch(ctx, dtype, d, H, n, window, slope):
+    """K and V rows TSATTN_PREFILL_MAX_KV_PITCH (8 MiB) apart: a 64-key tile spans 512 MiB, so the kernel's running
+    32-bit offsets pass 1 GiB every second tile and are folded back into the 64-bit base again and again; the arrays
+    end beyond 4 GiB, more than one buffer descriptor covers.  Results as for packed arrays; one byte more of pitch is
+    refused."""
+    import ctypes
+    pitch = 8 << 20
+    q, qs, k, ks, v, vs = make_qkv(7 * d + n, n, H, d, dtype)
+    st, fi = orc.make_spans([n], window)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, slope)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    def spread(a):   # only the rows' first H*d bytes are ever written or read
+        buf = torch.empty((n, pitch), dtype=torch.uint8, device="cuda")
+        buf[:, :H * d] = t(a)
+        return buf
+    kk, vv = spread(k), spread(v)
+    qq, sq, sk, sv, st_d, fi_d = t(q), t(qs), t(ks), t(vs), t(st), t(fi)
+    out = torch.empty((n, H * d), dtype=torch.float32, device="cuda")
+    a = capi.PrefillArgs()
+    a.dtype, a.out_dtype = dtype, capi.OUT_F32
+    a.n_tokens, a.n_heads, a.head_dim = n, H, d
+    a.q, a.k, a.v = qq.data_ptr(), kk.data_ptr(), vv.data_ptr()
+    a.q_pitch, a.k_pitch, a.v_pitch = H * d, pitch, pitch
+    a.q_scale, a.k_scale, a.v_scale, a.scale_pitch = sq.data_ptr(), sk.data_ptr(), sv.data_ptr(), n
+    a.span_start, a.span_finish = st_d.data_ptr(), fi_d.data_ptr()
+    a.alibi_slope = slope
+    a.out, a.out_pitch = out.data_ptr(), H * d * 4
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    capi.check(ctx.lib.tsattn_prefill(ctx.handle, ctypes.byref(a), stream))
+    torch.cuda.synchronize()
+    assert_within_tolerance(out.cpu().numpy(), want, "rows 8 MiB apart")
+    a.k_pitch = pitch + 16
+    with pytest.raises(capi.TsattnError):
+        capi.check(ctx.lib.tsattn_prefill(ctx.handle, ctypes.byref(a), stream))

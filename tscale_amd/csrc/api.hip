@@ -229,6 +229,9 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     const int64_t row = (int64_t)a->n_heads * a->head_dim;
     if (a->q_pitch < row || a->k_pitch < row || a->v_pitch < row || (a->q_pitch | a->k_pitch | a->v_pitch) % 16)
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: input pitch must be >= %lld and a multiple of 16", (long long)row);
+    // (the kernel addresses the rows of a key tile with 32-bit offsets from the tile's first row)
+    if (a->k_pitch > TSATTN_PREFILL_MAX_KV_PITCH || a->v_pitch > TSATTN_PREFILL_MAX_KV_PITCH)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: k_pitch and v_pitch may be at most %lld bytes", (long long)TSATTN_PREFILL_MAX_KV_PITCH);
     const int64_t out_row = row * (a->out_dtype == TSATTN_OUT_F16 ? 2 : 4);
     if (a->out && (a->out_pitch < out_row || a->out_pitch % 16)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: out_pitch must be >= %lld and a multiple of 16", (long long)out_row);
     if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out))
