@@ -324,10 +324,10 @@ enum tsattn_mm_mode {
 
 typedef struct tsattn_matmul_args {
     int64_t m, n, k;
-    const void *a;
-    int64_t a_pitch;
-    const void *w;
-    int64_t w_pitch;
+    const void *a;             /* int8 [m][k], 16-byte aligned */
+    int64_t a_pitch;           /* bytes, multiple of 16, at most 8 MiB */
+    const void *w;             /* int8 [n][k], 16-byte aligned */
+    int64_t w_pitch;           /* bytes, multiple of 16, at most 8 MiB */
     int mode;                  /* tsattn_mm_mode */
     float scale;
     void *out;

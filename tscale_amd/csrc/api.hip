@@ -489,7 +489,8 @@ int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *strea
     if (a->a_pitch < a->k || a->w_pitch < a->k || a->out_pitch < a->n || a->a_pitch % 16 || a->w_pitch % 16 || !aligned16(a->a) ||
         !aligned16(a->w) || (uintptr_t)a->out % 4)
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: pitches must cover a row; a, w and their pitches multiples of 16 bytes");
-    if (a->a_pitch > (1 << 24) || a->w_pitch > (1 << 24)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: row pitch above 16 MiB");
+    // (the kernels address up to 256 rows of a tile with signed 32-bit offsets)
+    if (a->a_pitch > (1 << 23) || a->w_pitch > (1 << 23)) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_matmul_i8: row pitch above 8 MiB");
     tsattn::GemmParams p = {};
     if (a->epilogue) {
         // the producer on the int32 result: its source is the product
