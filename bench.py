@@ -299,7 +299,7 @@ def bench_generation(ctx, steps):
                        "us_per_layer_step": round(gen_ms / gw.n_new / len(gw.sched) * 1e3, 2),
                        "GB/s": round(nbytes / gen_ms / 1e6, 1), "frac_of_hbm_peak": round(nbytes / gen_ms / 1e6 / PEAK_HBM_GBPS, 4),
                        "bytes": nbytes, "launch": "HIP graph of one step (24 x decode with fused append), replayed per token",
-                       "roofline": {"kernel": "decode_split_kernel<int8, d128> with fused append, 24 launches per token (+ 10 merges)",
+                       "roofline": {"kernel": "decode_split_kernel<int8, d128> with fused append, 24 launches per token (one split each: no merge)",
                                     "bound": "hbm", "achieved": round(nbytes / gen_ms / 1e6, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                                     "frac": round(nbytes / gen_ms / 1e6 / PEAK_HBM_GBPS, 4), "traffic": None,
                                     "bytes_per_token": nbytes // gw.n_new}}
