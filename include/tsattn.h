@@ -242,6 +242,33 @@ int64_t tsattn_span_tiles_count(int64_t n_tokens);
 int tsattn_build_span_tiles(tsattn_handle_t h, int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish,
                             int32_t *tiles, void *stream);
 
+/* Rows with more than one span.  TAttentionInfo holds any number of spans per row (gpt/att/att.h:24-47); the
+ * reference's CPU path loops over a row's spans inside one softmax (gpt/compute/gpt_cpu.cpp:405-436), its GPU kernels
+ * walk them as span groups (att.h:95-181).  Here: call tsattn_prefill once per span of the rows -- part i with every
+ * row's i-th span, an empty span (finish < start) for rows that have fewer -- each into its own f32 result and
+ * sum_weight_log, then combine the parts with this call.  Every part has the zero vector among its keys; the weights
+ * of the parts add up and the zero vector counts once: with W_i = 2^swl_i,
+ *   out = sum_i out_i W_i / (sum_i W_i - (n_parts - 1)),   sum_weight_log = log2 of that denominator,
+ * the result of one softmax over all the spans (keys that lie in two spans of a row count twice, as in the reference).
+ * part_out: n_parts results [n_tokens][n_heads*head_dim] f32, part_out_stride floats apart, rows part_out_pitch floats
+ * (a multiple of 4), 16-byte aligned; part_swl: n_parts planes [n_heads][scale_pitch], part_swl_stride floats apart.
+ * out must not overlap the parts. */
+typedef struct tsattn_merge_args {
+    int n_parts;               /* 1..64 */
+    int64_t n_tokens;
+    int n_heads, head_dim;     /* head_dim a multiple of 4 */
+    const float *part_out;
+    int64_t part_out_pitch, part_out_stride;
+    const float *part_swl;
+    int64_t scale_pitch, part_swl_stride;
+    int out_dtype;             /* tsattn_out_dtype */
+    void *out;                 /* [n_tokens][n_heads*head_dim], 16-byte aligned */
+    int64_t out_pitch;         /* bytes, multiple of 16 */
+    float *sum_weight_log;     /* optional [n_heads][scale_pitch] */
+} tsattn_merge_args;
+
+int tsattn_merge_lookups(tsattn_handle_t h, const tsattn_merge_args *a, void *stream);
+
 /* Producer of Q, K or V for the calls above from a projection result: optional RoPE at each row's position, then per
  * head sko = sqrt(mean x^2), scale = sko * vec_scale, values / scale converted to int8 (round to nearest even,
  * clamped to +-127) or e4m3, and scale * scale_mult written to scale[head * scale_pitch + row].  Replaces

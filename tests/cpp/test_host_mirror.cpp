@@ -718,9 +718,106 @@ static int RunContextCase(int firstLayer, int nLayers)
     return fails;
 }
 
+// Rows with several spans through TAttentionComputer (one launch per span of the rows, then the combining launch)
+// against the oracle's loop over a row's spans inside one softmax, on the dequantised operands.
+static int RunSeveralSpansCase(int dtype, float slope, bool outF16)
+{
+    const int H = 2, d = 128, len = 230;
+    TModelDims dims;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = H * d;
+    unsigned seed = 4242u + dtype;
+    std::vector<float> x((size_t)len * H * d), deq[3];
+    std::vector<uint8_t> q(x.size()), k(x.size()), v(x.size());
+    std::vector<float> qs((size_t)H * len), ks(qs.size()), vs(qs.size());
+    int which = 0;
+    for (auto *dst : {&q, &k, &v}) {
+        for (float &f : x) f = Gauss(seed);
+        float *sc = dst == &q ? qs.data() : dst == &k ? ks.data() : vs.data();
+        tso_quantize_rows(dtype, x.data(), H * d, len, H, d, dst->data(), H * d, sc, len);
+        deq[which].resize(x.size());
+        for (int t = 0; t < len; ++t)
+            for (int h = 0; h < H; ++h)
+                for (int i = 0; i < d; ++i) {
+                    const size_t at = ((size_t)t * H + h) * d + i;
+                    const float val = dtype == TSATTN_I8 ? (float)(int8_t)(*dst)[at] : tso_e4m3_to_float((*dst)[at]);
+                    deq[which][at] = val * sc[(size_t)h * len + t];
+                }
+        ++which;
+    }
+    // 0 to 3 spans per row, anywhere, overlapping now and then
+    TAttentionInfo att;
+    att.Init();
+    std::vector<int32_t> spanPtr(1, 0), spans;
+    for (int t = 0; t < len; ++t) {
+        const int n = (int)(Rand(seed) % 4);
+        for (int i = 0; i < n; ++i) {
+            const int a = (int)(Rand(seed) % len), b = std::min(len - 1, a + (int)(Rand(seed) % 50));
+            att.AddSpan(TAttentionSpan(a, b));
+            spans.push_back(a);
+            spans.push_back(b);
+        }
+        att.AddSample();
+        spanPtr.push_back((int32_t)spans.size() / 2);
+    }
+    std::vector<float> want((size_t)len * H * d);
+    tso_prefill_f32(len, H, d, d, deq[0].data(), deq[1].data(), deq[2].data(), spanPtr.data(), spans.data(), slope, want.data(), nullptr, nullptr);
+
+    TAttentionComputer attComp(dims, slope, 0, len + 26, 0); // (a context longer than the batch: pitches differ from len)
+    attComp.SetAttention(att, nullptr);
+    uint8_t *dq = ToDevice(q), *dk = ToDevice(k), *dv = ToDevice(v);
+    std::vector<float> qsP((size_t)H * (len + 26)), ksP(qsP.size()), vsP(qsP.size()); // scale planes of the context's pitch
+    for (int h = 0; h < H; ++h)
+        for (int t = 0; t < len; ++t) {
+            qsP[(size_t)h * (len + 26) + t] = qs[(size_t)h * len + t];
+            ksP[(size_t)h * (len + 26) + t] = ks[(size_t)h * len + t];
+            vsP[(size_t)h * (len + 26) + t] = vs[(size_t)h * len + t];
+        }
+    float *dqs = ToDevice(qsP), *dks = ToDevice(ksP), *dvs = ToDevice(vsP);
+    void *dout = nullptr;
+    const size_t esize = outF16 ? 2 : 4;
+    HIP_OK(hipMalloc(&dout, want.size() * esize));
+    TQuantRows rq, rk, rv;
+    rq.Data = dq; rq.PitchBytes = H * d; rq.Scale = dqs;
+    rk.Data = dk; rk.PitchBytes = H * d; rk.Scale = dks;
+    rv.Data = dv; rv.PitchBytes = H * d; rv.Scale = dvs;
+    attComp.ComputeValLookup(len, dtype, rq, rk, rv, nullptr, dout, (int64_t)H * d * esize, outF16, nullptr);
+    std::vector<float> got(want.size());
+    if (outF16) {
+        std::vector<_Float16> half(want.size());
+        HIP_OK(hipMemcpy(half.data(), dout, half.size() * 2, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < got.size(); ++i) got[i] = (float)half[i];
+    } else {
+        HIP_OK(hipMemcpy(got.data(), dout, got.size() * 4, hipMemcpyDeviceToHost));
+    }
+    double sum = 0, sum2 = 0;
+    for (float f : want) { sum += f; sum2 += (double)f * f; }
+    const double sd = sqrt(sum2 / want.size() - (sum / want.size()) * (sum / want.size()));
+    double maxErr = 0, meanErr = 0;
+    for (size_t i = 0; i < want.size(); ++i) {
+        const double e = fabs(got[i] - want[i]) / sd;
+        maxErr = e > maxErr ? e : maxErr;
+        meanErr += e;
+    }
+    meanErr /= want.size();
+    int fails = 0;
+    if (attComp.GetPartCount() != 3) {
+        printf("  several spans: %d parts, expected 3\n", attComp.GetPartCount());
+        ++fails;
+    }
+    if (!(maxErr <= 2e-2 && meanErr <= 2e-3)) {
+        printf("  several spans per row: max %.3e mean %.3e\n", maxErr, meanErr);
+        ++fails;
+    }
+    for (void *p : {(void *)dq, (void *)dk, (void *)dv, (void *)dqs, (void *)dks, (void *)dvs, dout}) HIP_OK(hipFree(p));
+    printf("several spans per row, dtype %d slope %g %s: max %.2e mean %.2e\n", dtype, slope, outF16 ? "f16" : "f32", maxErr, meanErr);
+    return fails;
+}
+
 int main()
 {
     int fails = 0;
+    fails += RunSeveralSpansCase(TSATTN_I8, 0.0f, false);
+    fails += RunSeveralSpansCase(TSATTN_E4M3, 0.25f, true);
     for (int l = 0; l < 3; ++l) fails += RunContextCase(l, 1);
     fails += RunContextCase(0, 3);
     fails += RunPromptLayerCase(1000, 0.0f, 128);

@@ -20,6 +20,7 @@ STRUCTS = {
     "tsattn_fill_args": capi.FillArgs,
     "tsattn_produce_args": capi.ProduceArgs,
     "tsattn_matmul_args": capi.MatmulArgs,
+    "tsattn_merge_args": capi.MergeArgs,
 }
 
 

@@ -500,3 +500,47 @@ def test_prefill_largest_key_row_pitch(ctx, dtype, d, H, n, window, slope):
     a.k_pitch = pitch + 16
     with pytest.raises(capi.TsattnError):
         capi.check(ctx.lib.tsattn_prefill(ctx.handle, ctypes.byref(a), stream))
+
+
+@pytest.mark.parametrize("dtype,d,H,n,max_spans,slope,out_f16", [
+    (capi.I8, 128, 2, 300, 3, 0.0, False),
+    (capi.E4M3, 64, 3, 257, 2, 0.25, True),
+    (capi.I8, 64, 1, 200, 5, 0.5, False),
+])
+def test_prefill_rows_with_several_spans(ctx, dtype, d, H, n, max_spans, slope, out_f16):
+    """Rows with any number of spans (TAttentionInfo, gpt/att/att.h:24-47): one tsattn_prefill per span of the rows and
+    tsattn_merge_lookups, against the oracle's loop over a row's spans inside one softmax (gpt_cpu.cpp:405-436) on the
+    dequantised operands.  Spans overlap (a key in two spans counts twice), some rows have none."""
+    from tests.test_oracle_attention import random_span_lists
+    rng = np.random.default_rng(100 * d + n)
+    q, qs, k, ks, v, vs = make_qkv(5 * d + n, n, H, d, dtype)
+    ptr, spans = random_span_lists(rng, n, max_spans)
+    tab = orc.e4m3_table()
+    def deq(x, s):
+        xf = x.view(np.int8).astype(np.float32) if dtype == capi.I8 else tab[x]
+        return (xf.reshape(n, H, d) * s.T[:, :, None]).reshape(n, H * d)
+    want, sw, mx = orc.prefill_f32(deq(q, qs), deq(k, ks), deq(v, vs), H, ptr, spans, slope)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    swl = torch.zeros((H, n), dtype=torch.float32, device="cuda")
+    out = ctx.compute_val_lookup_multi(dtype, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), ptr, spans, slope,
+                                       out_f16=out_f16, sum_weight_log=swl)
+    torch.cuda.synchronize()
+    assert out.dtype == (torch.float16 if out_f16 else torch.float32)
+    assert_within_tolerance(out.float().cpu().numpy(), want, "several spans per row")
+    none = ptr[1:] == ptr[:-1]
+    assert none.any() and not out[torch.from_numpy(none).cuda()].any()
+    # sum_weight_log = max logit + log2(sum of the shifted weights, zero vector included)
+    assert np.abs(swl.cpu().numpy() - (mx + np.log2(sw))).max() < 2e-3
+
+
+def test_merge_lookups_argument_checks(ctx):
+    import ctypes
+    parts = torch.zeros((2, 8, 64), dtype=torch.float32, device="cuda")
+    swl = torch.zeros((2, 1, 8), dtype=torch.float32, device="cuda")
+    assert not ctx.merge_lookups(parts, swl).any()        # two empty parts: an empty result
+    with pytest.raises(capi.TsattnError):                  # parts that overlap
+        ctx.merge_lookups(parts.as_strided((2, 8, 64), (64, 64, 1)), swl)
+    a = capi.MergeArgs()
+    a.n_parts, a.n_tokens, a.n_heads, a.head_dim = 0, 8, 1, 64
+    with pytest.raises(capi.TsattnError):                  # no parts
+        capi.check(ctx.lib.tsattn_merge_lookups(ctx.handle, ctypes.byref(a), None))

@@ -92,6 +92,40 @@ def test_prefill_f32_matches_textbook_softmax_with_zero_key():
     assert np.abs(out - want).max() < 2e-5
 
 
+def random_span_lists(rng, n, max_spans):
+    """Per row up to max_spans random spans anywhere in [0, n): some rows none, some spans overlapping."""
+    ptr, spans = [0], []
+    for _ in range(n):
+        for _ in range(int(rng.integers(0, max_spans + 1))):
+            a = int(rng.integers(0, n))
+            spans.append((a, min(n - 1, a + int(rng.integers(0, 40)))))
+        ptr.append(len(spans))
+    return np.array(ptr, dtype=np.int32), np.array(spans, dtype=np.int32).reshape(-1, 2)
+
+
+def test_prefill_f32_rows_with_several_spans_match_textbook_softmax():
+    # any number of spans per row (gpt_cpu.cpp:405-436 loops over them inside one softmax): a key that lies in c spans
+    # of a row counts c times, i.e. its logit gains ln c; everything else as in the test above
+    n, H, d = 90, 2, 64
+    rng = np.random.default_rng(5)
+    q, k, v = (rng.standard_normal((n, H * d)).astype(np.float32) for _ in range(3))
+    ptr, spans = random_span_lists(rng, n, 3)
+    out, _, _ = orc.prefill_f32(q, k, v, H, ptr, spans, 0.0)
+    count = np.zeros((n, n))
+    for row in range(n):
+        for a, b in spans[ptr[row]:ptr[row + 1]]:
+            count[row, a:b + 1] += 1
+    assert count.max() >= 2 and (count.sum(1) == 0).any()
+    tq, tk, tv = (torch.from_numpy(x).double().view(n, H, d).transpose(0, 1) for x in (q, k, v))
+    logits = tq @ tk.transpose(1, 2) * (0.5 / np.sqrt(d)) * (np.log(2.0) / float(LN2_REF))
+    with np.errstate(divide="ignore"):
+        logits = logits + torch.from_numpy(np.log(count))
+    logits = torch.cat([logits, torch.zeros(H, n, 1, dtype=torch.double)], dim=2)
+    p = torch.softmax(logits, dim=2)[:, :, :n]
+    want = (p @ tv).transpose(0, 1).reshape(n, H * d).numpy()
+    assert np.abs(out - want).max() < 2e-5
+
+
 def test_prefill_f32_shift_invariance_and_underflow():
     n, d = 20, 64
     rng = np.random.default_rng(4)

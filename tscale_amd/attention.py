@@ -319,6 +319,49 @@ class AttentionContext:
         capi.check(self.lib.tsattn_prefill(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
 
+    def merge_lookups(self, part_out, part_swl, out=None, out_f16=False, sum_weight_log=None):
+        """part_out: f32 [n_parts, n_tokens, H*d], part_swl: f32 [n_parts, H, n_tokens]: prefill results over each row's
+        i-th span; returns the attention result over all of a row's spans."""
+        n_parts, n_tokens, hd = part_out.shape
+        n_heads = part_swl.shape[1]
+        if out is None:
+            out = torch.empty((n_tokens, hd), dtype=torch.float16 if out_f16 else torch.float32, device=part_out.device)
+        a = capi.MergeArgs()
+        a.n_parts, a.n_tokens, a.n_heads, a.head_dim = n_parts, n_tokens, n_heads, hd // n_heads
+        a.part_out, a.part_out_pitch, a.part_out_stride = _ptr(part_out), part_out.stride(1), part_out.stride(0)
+        a.part_swl, a.scale_pitch, a.part_swl_stride = _ptr(part_swl), part_swl.stride(1), part_swl.stride(0)
+        a.out_dtype = capi.OUT_F16 if out.dtype == torch.float16 else capi.OUT_F32
+        a.out, a.out_pitch = _ptr(out), out.stride(0) * out.element_size()
+        if sum_weight_log is not None:
+            assert sum_weight_log.stride(0) == a.scale_pitch
+            a.sum_weight_log = _ptr(sum_weight_log)
+        capi.check(self.lib.tsattn_merge_lookups(self.handle, ctypes.byref(a), _stream_ptr()))
+        return out
+
+    def compute_val_lookup_multi(self, dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, span_ptr, spans, alibi_slope,
+                                 out_f16=False, sum_weight_log=None):
+        """Rows with any number of spans, as TAttentionInfo holds them (gpt/att/att.h:24-47): span_ptr int [n_tokens+1],
+        spans int [n_spans, 2] (inclusive start, finish), both on the host.  One prefill launch per span of the rows
+        (part i takes every row's i-th span) and one launch that combines them."""
+        n_tokens = q.shape[0]
+        span_ptr = np.asarray(span_ptr, dtype=np.int64)
+        spans = np.asarray(spans, dtype=np.int32).reshape(-1, 2)
+        counts = span_ptr[1:] - span_ptr[:-1]
+        n_parts = max(1, int(counts.max()) if n_tokens else 1)
+        st = np.tile(np.arange(n_tokens, dtype=np.int32), (n_parts, 1))
+        fi = st - 1                                   # rows that have no i-th span: an empty one
+        for i in range(n_parts):
+            rows = np.nonzero(counts > i)[0]
+            st[i, rows] = spans[span_ptr[rows] + i, 0]
+            fi[i, rows] = spans[span_ptr[rows] + i, 1]
+        st_d, fi_d = torch.from_numpy(st).to(q.device), torch.from_numpy(fi).to(q.device)
+        part_out = torch.empty((n_parts, n_tokens, q.shape[1]), dtype=torch.float32, device=q.device)
+        part_swl = torch.empty((n_parts, n_heads, n_tokens), dtype=torch.float32, device=q.device)
+        for i in range(n_parts):
+            self.compute_val_lookup(dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, st_d[i], fi_d[i], alibi_slope,
+                                    out=part_out[i], sum_weight_log=part_swl[i])
+        return self.merge_lookups(part_out, part_swl, out_f16=out_f16, sum_weight_log=sum_weight_log)
+
     # ---- decode ---------------------------------------------------------------------------------
     def compute_val_lookup_decode(self, cache, q, q_scale, window, alibi_slope, out=None, n_splits=0,
                                   debug_qk_acc=None, max_len=None, append=None, kv_product=None, static_scratch=False):

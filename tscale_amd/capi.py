@@ -108,8 +108,17 @@ class FillArgs(_c.Structure):
     ]
 
 
+class MergeArgs(_c.Structure):
+    _fields_ = [
+        ("n_parts", _c.c_int), ("n_tokens", _c.c_int64), ("n_heads", _c.c_int), ("head_dim", _c.c_int),
+        ("part_out", _c.c_void_p), ("part_out_pitch", _c.c_int64), ("part_out_stride", _c.c_int64),
+        ("part_swl", _c.c_void_p), ("scale_pitch", _c.c_int64), ("part_swl_stride", _c.c_int64),
+        ("out_dtype", _c.c_int), ("out", _c.c_void_p), ("out_pitch", _c.c_int64), ("sum_weight_log", _c.c_void_p),
+    ]
+
+
 EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
-           "tsattn_decode", "tsattn_decode_static", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_embed_rows", "tsattn_softmax_rows", "tsattn_sample_rows", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_debug_read_counters", "tsattn_version"]
+           "tsattn_decode", "tsattn_decode_static", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_merge_lookups", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_embed_rows", "tsattn_softmax_rows", "tsattn_sample_rows", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_debug_read_counters", "tsattn_version"]
 
 _lib = None
 
@@ -143,6 +152,8 @@ def load():
         L.tsattn_cache_append.argtypes = [_c.c_void_p, _c.POINTER(AppendArgs), _c.c_void_p]
         L.tsattn_cache_fill.restype = _c.c_int
         L.tsattn_cache_fill.argtypes = [_c.c_void_p, _c.POINTER(FillArgs), _c.c_void_p]
+        L.tsattn_merge_lookups.restype = _c.c_int
+        L.tsattn_merge_lookups.argtypes = [_c.c_void_p, _c.POINTER(MergeArgs), _c.c_void_p]
         L.tsattn_span_tiles_count.restype = _c.c_int64
         L.tsattn_span_tiles_count.argtypes = [_c.c_int64]
         L.tsattn_build_span_tiles.restype = _c.c_int

@@ -368,6 +368,34 @@ int tsattn_build_span_tiles(tsattn_handle_t h, int64_t n_tokens, const int32_t *
     return TSATTN_OK;
 }
 
+int tsattn_merge_lookups(tsattn_handle_t h, const tsattn_merge_args *a, void *stream)
+{
+    if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_merge_lookups: null argument");
+    if (a->n_parts < 1 || a->n_parts > 64) return fail(TSATTN_ERR_BAD_ARG, "tsattn_merge_lookups: n_parts %d (1..64)", a->n_parts);
+    if (a->n_tokens < 0 || a->n_heads <= 0 || a->head_dim <= 0 || a->head_dim % 4)
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_merge_lookups: n_tokens %lld, n_heads %d, head_dim %d (a multiple of 4)", (long long)a->n_tokens, a->n_heads, a->head_dim);
+    if (a->out_dtype != TSATTN_OUT_F32 && a->out_dtype != TSATTN_OUT_F16) return fail(TSATTN_ERR_UNSUPPORTED, "tsattn_merge_lookups: out_dtype %d", a->out_dtype);
+    if (a->n_tokens == 0) return TSATTN_OK;
+    if (!a->part_out || !a->part_swl || !a->out) return fail(TSATTN_ERR_BAD_ARG, "tsattn_merge_lookups: null data pointer");
+    const int64_t row = (int64_t)a->n_heads * a->head_dim;
+    if (a->part_out_pitch < row || a->part_out_pitch % 4 || a->part_out_stride % 4 || !aligned16(a->part_out) ||
+        (a->n_parts > 1 && a->part_out_stride < a->n_tokens * a->part_out_pitch))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_merge_lookups: parts must be 16-byte aligned, rows of part_out_pitch >= %lld floats (a multiple of 4), parts a whole result apart", (long long)row);
+    if (a->scale_pitch < a->n_tokens || (a->n_parts > 1 && a->part_swl_stride < (int64_t)a->n_heads * a->scale_pitch))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_merge_lookups: scale_pitch below n_tokens or sum_weight_log planes that overlap");
+    const int64_t out_row = row * (a->out_dtype == TSATTN_OUT_F16 ? 2 : 4);
+    if (a->out_pitch < out_row || a->out_pitch % 16 || !aligned16(a->out))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_merge_lookups: out must be 16-byte aligned with a pitch >= %lld bytes, a multiple of 16", (long long)out_row);
+    tsattn::MergeParams p;
+    p.n_parts = a->n_parts; p.n_tokens = a->n_tokens; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
+    p.part_out = a->part_out; p.part_out_pitch = a->part_out_pitch; p.part_out_stride = a->part_out_stride;
+    p.part_swl = a->part_swl; p.scale_pitch = a->scale_pitch; p.part_swl_stride = a->part_swl_stride;
+    p.out = a->out; p.out_pitch = a->out_pitch; p.swl = a->sum_weight_log;
+    const hipError_t e = tsattn::launch_merge_lookups(p, a->out_dtype == TSATTN_OUT_F16, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "merge launch");
+    return TSATTN_OK;
+}
+
 int tsattn_cache_fill(tsattn_handle_t h, const tsattn_fill_args *a, void *stream)
 {
     if (!h || !a) return fail(TSATTN_ERR_BAD_ARG, "tsattn_cache_fill: null argument");

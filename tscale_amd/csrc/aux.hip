@@ -1,5 +1,5 @@
 // Small kernels around the attention path: the absmax row quantiser, the span (window metadata)
-// builder and the KV-cache append.
+// builder, the KV-cache append and the combination of attention results over several spans per row.
 #include "common.hpp"
 #include "kernels.hpp"
 
@@ -288,6 +288,56 @@ hipError_t launch_cache_fill(const FillParams &p, hipStream_t st)
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(cache_len_add_kernel, dim3((unsigned)((p.n_seqs + 255) / 256)), dim3(256), 0, st, p.cache_len, p.seq_offset,
                        p.n_seqs, p.max_len);
+    return hipGetLastError();
+}
+
+// Rows whose keys come as several spans: tsattn_prefill has been run once per span of the rows, part i over every row's
+// i-th span, each part with the zero vector among its keys.  The weights of the parts add up and the zero vector counts
+// once: with W_i = 2^swl_i the total weight of part i (zero vector included, weight 1),
+//   out = sum_i out_i W_i / (sum_i W_i - (n - 1)),   swl = log2 of that denominator
+// -- what the reference's loop over a row's spans computes in one go (compute/gpt_cpu.cpp:405-436).  Evaluated against
+// the largest swl_i so that nothing overflows.  One thread per four consecutive values of a (row, head).
+template <bool OUT_F16>
+__global__ __launch_bounds__(256) void merge_lookups_kernel(MergeParams p)
+{
+    const int per_head = p.head_dim / 4;
+    const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (id >= p.n_tokens * p.n_heads * per_head) return;
+    const int c = (int)(id % per_head);
+    const int64_t pair = id / per_head;
+    const int head = (int)(pair % p.n_heads);
+    const int64_t row = pair / p.n_heads;
+    const int64_t s_at = (int64_t)head * p.scale_pitch + row;
+    const int64_t o_at = row * p.part_out_pitch + (int64_t)head * p.head_dim + 4 * c;
+    float top = 0.0f; // every swl_i is >= 0: the zero vector alone weighs 1
+    for (int i = 0; i < p.n_parts; ++i) top = fmaxf(top, p.part_swl[i * p.part_swl_stride + s_at]);
+    v4f acc = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    float total = 0.0f;
+    for (int i = 0; i < p.n_parts; ++i) {
+        const float w = exp2f(p.part_swl[i * p.part_swl_stride + s_at] - top);
+        const v4f x = *(const v4f *)(p.part_out + i * p.part_out_stride + o_at);
+        acc += x * w;
+        total += w;
+    }
+    total -= (float)(p.n_parts - 1) * exp2f(-top);
+    const v4f res = acc * (1.0f / total);
+    if (OUT_F16) {
+        uint8_t *dst = (uint8_t *)p.out + row * p.out_pitch + ((int64_t)head * p.head_dim + 4 * c) * 2;
+        *(v4h *)dst = v4h{(_Float16)res.x, (_Float16)res.y, (_Float16)res.z, (_Float16)res.w};
+    } else {
+        uint8_t *dst = (uint8_t *)p.out + row * p.out_pitch + ((int64_t)head * p.head_dim + 4 * c) * 4;
+        *(v4f *)dst = res;
+    }
+    if (p.swl && c == 0) p.swl[s_at] = top + log2f(total);
+}
+
+hipError_t launch_merge_lookups(const MergeParams &p, bool out_f16, hipStream_t st)
+{
+    const int64_t n = p.n_tokens * p.n_heads * (p.head_dim / 4);
+    if (n == 0) return hipSuccess;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (out_f16) hipLaunchKernelGGL((merge_lookups_kernel<true>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((merge_lookups_kernel<false>), grid, block, 0, st, p);
     return hipGetLastError();
 }
 

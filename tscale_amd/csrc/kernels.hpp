@@ -86,6 +86,21 @@ hipError_t launch_quantize_rows(int src_dtype, int dst_dtype, const void *src, i
 constexpr int SPAN_TILE_INTS = 32;
 constexpr int SPAN_TILE_MIN_A = 0, SPAN_TILE_MAX_B = 1; // over rows that have keys; MIN_A > MAX_B if none has
 constexpr int SPAN_TILE_WAVE0 = 4, SPAN_TILE_WAVE_INTS = 5; // per wave: min_a, max_a, min_b, max_b, all_have_keys
+// Combines attention results over disjoint (or repeated) key sets of the same rows, each with the zero vector in it
+struct MergeParams {
+    int n_parts;
+    int64_t n_tokens;
+    int n_heads, head_dim;
+    const float *part_out;   // part i: part_out + i * part_out_stride, rows of part_out_pitch floats
+    int64_t part_out_pitch, part_out_stride;
+    const float *part_swl;   // part i: part_swl + i * part_swl_stride, [head][scale_pitch]
+    int64_t scale_pitch, part_swl_stride;
+    void *out;               // f32 or f16 rows of out_pitch bytes
+    int64_t out_pitch;
+    float *swl;              // optional [head][scale_pitch]
+};
+hipError_t launch_merge_lookups(const MergeParams &p, bool out_f16, hipStream_t st);
+
 hipError_t launch_build_span_tiles(int64_t n_tokens, const int32_t *span_start, const int32_t *span_finish, int32_t *tiles, hipStream_t st);
 
 hipError_t launch_build_spans(int n_seqs, const int32_t *seq_offset, int64_t n_tokens, const uint8_t *doc_start_flag,

@@ -30,7 +30,8 @@ static void CheckHip(hipError_t e, const char *what)
     TS_VERIFY(e == hipSuccess, "%s failed: %s", what, hipGetErrorString(e));
 }
 
-static int FlattenSpans(const TAttentionInfo &attInfo, std::vector<int32_t> *pStart, std::vector<int32_t> *pFinish);
+static int FlattenSpans(const TAttentionInfo &attInfo, std::vector<int32_t> *pStart, std::vector<int32_t> *pFinish, int part = 0,
+                        bool oneSpanPerRow = true);
 
 void AddWindowSpans(int ptr, int len, int limitWindow, const uint8_t *docStartFlag, TAttentionInfo *pAtt)
 {
@@ -65,10 +66,27 @@ TAttentionComputer::TAttentionComputer(const TModelDims &dims, float alibiSlope,
     cfg.max_heads = dims.HeadCount;
     cfg.max_head_dim = dims.QDim;
     Check(tsattn_create(&cfg, &Handle), "tsattn_create");
-    CheckHip(hipMalloc((void **)&SpanStart, sizeof(int32_t) * (size_t)maxLen), "hipMalloc(spans)");
-    CheckHip(hipMalloc((void **)&SpanFinish, sizeof(int32_t) * (size_t)maxLen), "hipMalloc(spans)");
-    CheckHip(hipMalloc((void **)&SpanTiles, sizeof(int32_t) * TSATTN_SPAN_TILE_INTS * (size_t)tsattn_span_tiles_count(maxLen)), "hipMalloc(span tiles)");
     CheckHip(hipMalloc((void **)&SumWeightLog, sizeof(float) * (size_t)maxLen * dims.HeadCount), "hipMalloc(sumWeightLog)");
+    Reserve(1);
+}
+
+// room for the spans of `parts` parts; with more than one also for the parts' results
+void TAttentionComputer::Reserve(int parts)
+{
+    if (parts <= PartCapacity) return;
+    void *old[] = {SpanStart, SpanFinish, SpanTiles, PartOut, PartSwl};
+    for (void *p : old) (void)hipFree(p);
+    SpanStart = SpanFinish = SpanTiles = nullptr;
+    PartOut = PartSwl = nullptr;
+    const size_t n = (size_t)parts * MaxLen;
+    CheckHip(hipMalloc((void **)&SpanStart, sizeof(int32_t) * n), "hipMalloc(spans)");
+    CheckHip(hipMalloc((void **)&SpanFinish, sizeof(int32_t) * n), "hipMalloc(spans)");
+    CheckHip(hipMalloc((void **)&SpanTiles, sizeof(int32_t) * TSATTN_SPAN_TILE_INTS * (size_t)tsattn_span_tiles_count(MaxLen) * parts), "hipMalloc(span tiles)");
+    if (parts > 1) {
+        CheckHip(hipMalloc((void **)&PartOut, sizeof(float) * n * Dims.HeadCount * Dims.TTDim), "hipMalloc(parts)");
+        CheckHip(hipMalloc((void **)&PartSwl, sizeof(float) * n * Dims.HeadCount), "hipMalloc(parts)");
+    }
+    PartCapacity = parts;
 }
 
 TAttentionComputer::~TAttentionComputer()
@@ -77,6 +95,8 @@ TAttentionComputer::~TAttentionComputer()
     (void)hipFree(SpanFinish);
     (void)hipFree(SpanTiles);
     (void)hipFree(SumWeightLog);
+    (void)hipFree(PartOut);
+    (void)hipFree(PartSwl);
     tsattn_destroy(Handle);
 }
 
@@ -84,13 +104,24 @@ void TAttentionComputer::SetAttention(const TAttentionInfo &attInfo, void *strea
 {
     int len = (int)attInfo.GetSampleCount();
     TS_VERIFY(len <= MaxLen, "%d samples exceed the context's %d", len, MaxLen);
-    std::vector<int32_t> st, fi;
-    CausalPeriod = FlattenSpans(attInfo, &st, &fi); // (and the launch-order hint)
+    int parts = 1;
+    for (int t = 0; t < len; ++t) parts = std::max(parts, attInfo.SpanPtr[t + 1] - attInfo.SpanPtr[t]);
+    TS_VERIFY(parts <= 64, "a row with %d spans; up to 64 are supported", parts);
+    CheckHip(hipStreamSynchronize((hipStream_t)stream), "stream"); // nothing may still use what Reserve frees
+    Reserve(parts);
+    Parts = parts;
     Len = len;
-    // pageable source: the copy has returned from the host's point of view when the call returns
-    CheckHip(hipMemcpyAsync(SpanStart, st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
-    CheckHip(hipMemcpyAsync(SpanFinish, fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
-    Check(tsattn_build_span_tiles(Handle, len, SpanStart, SpanFinish, SpanTiles, stream), "tsattn_build_span_tiles");
+    const int64_t tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(MaxLen);
+    std::vector<int32_t> st, fi;
+    for (int i = 0; i < parts; ++i) {
+        const int period = FlattenSpans(attInfo, &st, &fi, i, false); // (and the launch-order hint)
+        CausalPeriod = parts == 1 ? period : 0;
+        // pageable source: the copy has returned from the host's point of view when the call returns
+        CheckHip(hipMemcpyAsync(SpanStart + (size_t)i * MaxLen, st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
+        CheckHip(hipMemcpyAsync(SpanFinish + (size_t)i * MaxLen, fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
+        Check(tsattn_build_span_tiles(Handle, len, SpanStart + (size_t)i * MaxLen, SpanFinish + (size_t)i * MaxLen, SpanTiles + i * tileInts, stream),
+              "tsattn_build_span_tiles");
+    }
     CheckHip(hipStreamSynchronize((hipStream_t)stream), "span copy");
 }
 
@@ -111,13 +142,35 @@ void TAttentionComputer::ComputeValLookup(int len, int dtype, const TQuantRows &
     a.scale_pitch = MaxLen;
     a.q_scale_const = qk.ConstScale; a.k_scale_const = qv.ConstScale; a.v_scale_const = v.ConstScale;
     a.k_global_scale = qvGlobalScale;
-    a.span_start = SpanStart; a.span_finish = SpanFinish;
-    a.span_tiles = SpanTiles;
     a.alibi_slope = AlibiSlope;
-    a.out = valLookup; a.out_pitch = valLookupPitchBytes;
-    a.sum_weight_log = SumWeightLog;
-    a.causal_period = CausalPeriod;
-    Check(tsattn_prefill(Handle, &a, stream), "tsattn_prefill");
+    if (Parts == 1) {
+        a.span_start = SpanStart; a.span_finish = SpanFinish;
+        a.span_tiles = SpanTiles;
+        a.out = valLookup; a.out_pitch = valLookupPitchBytes;
+        a.sum_weight_log = SumWeightLog;
+        a.causal_period = CausalPeriod;
+        Check(tsattn_prefill(Handle, &a, stream), "tsattn_prefill");
+        return;
+    }
+    // one softmax over all the spans of a row (gpt_cpu.cpp:405-436) = the parts' results combined by their weights
+    const int64_t row = (int64_t)Dims.HeadCount * Dims.TTDim, tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(MaxLen);
+    a.out_dtype = TSATTN_OUT_F32;
+    a.out_pitch = row * 4;
+    for (int i = 0; i < Parts; ++i) {
+        a.span_start = SpanStart + (size_t)i * MaxLen; a.span_finish = SpanFinish + (size_t)i * MaxLen;
+        a.span_tiles = SpanTiles + i * tileInts;
+        a.out = PartOut + (size_t)i * MaxLen * row;
+        a.sum_weight_log = PartSwl + (size_t)i * Dims.HeadCount * MaxLen;
+        Check(tsattn_prefill(Handle, &a, stream), "tsattn_prefill");
+    }
+    tsattn_merge_args m = {};
+    m.n_parts = Parts; m.n_tokens = len; m.n_heads = Dims.HeadCount; m.head_dim = Dims.TTDim;
+    m.part_out = PartOut; m.part_out_pitch = row; m.part_out_stride = (int64_t)MaxLen * row;
+    m.part_swl = PartSwl; m.scale_pitch = MaxLen; m.part_swl_stride = (int64_t)Dims.HeadCount * MaxLen;
+    m.out_dtype = outF16 ? TSATTN_OUT_F16 : TSATTN_OUT_F32;
+    m.out = valLookup; m.out_pitch = valLookupPitchBytes;
+    m.sum_weight_log = SumWeightLog;
+    Check(tsattn_merge_lookups(Handle, &m, stream), "tsattn_merge_lookups");
 }
 
 TAttentionVecHistory::TAttentionVecHistory(tsattn_handle_t handle, int dtype, int seqCount, int headCount, int maxLen, int headDim)
@@ -528,15 +581,15 @@ void TNodesBatch::AddSample(int idx, const std::vector<int32_t> &labels, const s
 // One inclusive span per row (rows without keys: an empty one) from the reference's span lists, and the launch-order
 // hint: rows without keys mark fragment starts; if they are equally spaced, cover the batch and the window is wide
 // (the last row of a fragment sees at least half of it), the batch has a causal period.
-static int FlattenSpans(const TAttentionInfo &attInfo, std::vector<int32_t> *pStart, std::vector<int32_t> *pFinish)
+static int FlattenSpans(const TAttentionInfo &attInfo, std::vector<int32_t> *pStart, std::vector<int32_t> *pFinish, int part, bool oneSpanPerRow)
 {
     const int len = (int)attInfo.GetSampleCount();
     std::vector<int32_t> &st = *pStart, &fi = *pFinish;
     st.resize(len);
     fi.resize(len);
     for (int t = 0; t < len; ++t) {
-        const int a = attInfo.SpanPtr[t], b = attInfo.SpanPtr[t + 1];
-        TS_VERIFY(b - a <= 1, "row %d has %d spans; one span per row is supported", t, b - a);
+        const int a = attInfo.SpanPtr[t] + part, b = attInfo.SpanPtr[t + 1];
+        if (oneSpanPerRow) TS_VERIFY(b - a <= 1, "row %d has %d spans; one span per row is supported here", t, b - a);
         if (b > a) {
             st[t] = attInfo.Spans[a].Start;
             fi[t] = attInfo.Spans[a].Finish;

@@ -84,10 +84,15 @@ class TAttentionComputer
     int MaxLen = 0;
     int Len = 0;
     int CausalPeriod = 0; // launch-order hint derived from the spans by SetAttention
-    int32_t *SpanStart = nullptr; // device
+    // Rows may hold several spans: part i of the batch is every row's i-th span (an empty one for rows with fewer)
+    int Parts = 1, PartCapacity = 0;
+    int32_t *SpanStart = nullptr; // device [PartCapacity][MaxLen]
     int32_t *SpanFinish = nullptr;
-    int32_t *SpanTiles = nullptr; // per-128-row summary of the spans (tsattn_build_span_tiles)
+    int32_t *SpanTiles = nullptr; // per part: per-128-row summary of the spans (tsattn_build_span_tiles)
     float *SumWeightLog = nullptr; // device [headCount][MaxLen]
+    float *PartOut = nullptr;      // device [PartCapacity][MaxLen][headCount*TTDim], only with more than one part
+    float *PartSwl = nullptr;      // device [PartCapacity][headCount][MaxLen]
+    void Reserve(int parts);
 
   public:
     // maxSeqs > 0 also provisions the handle for KV-cache decode of that many sequences
@@ -97,8 +102,10 @@ class TAttentionComputer
     TAttentionComputer &operator=(const TAttentionComputer &) = delete;
 
     // Per batch, like TComputeContext::Init copying the spans to the device (gpt_cuda.cu:1362-1376).
-    // Rows with more than one span are not supported by the kernels and abort.
+    // Rows with several spans (TAttentionInfo allows any number) cost one attention launch per span of the rows and
+    // one launch that combines them (tsattn_merge_lookups).
     void SetAttention(const TAttentionInfo &attInfo, void *stream);
+    int GetPartCount() const { return Parts; }
 
     // valLookup: device [len][headCount*TTDim] fp32 (outF16 = false) or fp16.
     void ComputeValLookup(int len, int dtype, const TQuantRows &qk, const TQuantRows &qv, const TQuantRows &v,
