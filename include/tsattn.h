@@ -281,7 +281,8 @@ typedef struct tsattn_produce_args {
     int src_dtype;             /* TSATTN_SRC_F32 or TSATTN_SRC_I32 */
     int dst_dtype;             /* tsattn_dtype */
     int64_t n_rows;
-    int n_heads, head_dim;
+    int n_heads, head_dim;     /* head_dim 64 or 128; also 256, 384, 512 (the feed-forward groups of 128 * ReluMult,
+                                  gpt/model_params/model_dim.h:66) with an int8 result and no rotation */
     const void *src;           /* [n_rows][n_heads*head_dim], 16-byte aligned */
     int64_t src_pitch;         /* elements per row, multiple of 4 */
     const int32_t *pos;        /* device [n_rows]: position of each row in its sequence; NULL = no rotation */

@@ -181,12 +181,12 @@ static int RunCase(int dtype, int window, float slope)
 // holds, so each step is checked on identical inputs: the rows appended to the two KV caches must then be identical
 // bytes (normalisation and integer products are exact on both sides), the attention output and the new state agree
 // within the attention tolerance.
-static int RunLayerCase(int width, float slope, int headDim, bool oneProjectionMatrix)
+static int RunLayerCase(int width, float slope, int headDim, bool oneProjectionMatrix, int reluMult = 1)
 {
     const int B = 5, H = 4, d = headDim, dim = 512, steps = 7, maxLen = 16;
-    const int qsum = H * d, kvDim = qsum * 4, reluDim = H * 128; // GetReluDim(): 128 per head whatever the head width
+    const int qsum = H * d, kvDim = qsum * 4, reluDim = H * 128 * reluMult; // GetReluDim(): 128 * ReluMult per head whatever the head width
     TModelDims dims;
-    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim; dims.ReluMult = reluMult;
     unsigned seed = 99u + width * 3 + headDim;
     auto randMatrix = [&](size_t n) {
         std::vector<int8_t> m(n);
@@ -349,13 +349,13 @@ struct TCpuCache {
 // The prompt form of the layer: all tokens of two fragments in one call against the oracle's token-by-token run of
 // the same layer.  Every token's projections depend on its own input state only, so the rows both sides append to the
 // cache must be identical bytes; attention output and new state within the attention tolerance.
-static int RunPromptLayerCase(int width, float slope, int headDim)
+static int RunPromptLayerCase(int width, float slope, int headDim, int reluMult = 1)
 {
     const int B = 2, H = 4, d = headDim, dim = 512, maxLen = 256;
     const int fragLen[B] = {150, 70};
     const int len = fragLen[0] + fragLen[1], qsum = H * d;
     TModelDims dims;
-    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim; dims.ReluMult = reluMult;
     unsigned seed = 4242u + width * 5 + headDim;
     tsattn_config cfg = {};
     cfg.device = 0; cfg.max_seqs = B; cfg.max_heads = H; cfg.max_head_dim = d;
@@ -824,12 +824,15 @@ int main()
     fails += RunPromptLayerCase(64, 0.5f, 128);
     fails += RunPromptLayerCase(1, 0.0f, 64);
     fails += RunPromptLayerCase(0, 0.0f, 128);
+    fails += RunPromptLayerCase(1000, 0.0f, 128, 2); // feed-forward groups of 256
     fails += RunPredictionCase();
     fails += RunLayerCase(1000, 0.0f, 128, true);
     fails += RunLayerCase(1000, 0.0f, 128, false);
     fails += RunLayerCase(4, 0.5f, 128, true);
     fails += RunLayerCase(1, 0.0f, 64, false);
     fails += RunLayerCase(0, 0.0f, 128, true);
+    fails += RunLayerCase(1000, 0.0f, 128, true, 3); // ... of 384
+    fails += RunLayerCase(4, 0.5f, 64, false, 4);    // ... of 512
     for (int dtype : {TSATTN_I8, TSATTN_E4M3}) {
         fails += RunCase(dtype, 64, 0.5f);
         fails += RunCase(dtype, 1000, 0.0f);

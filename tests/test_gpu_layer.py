@@ -21,14 +21,17 @@ def ctx():
     c.close()
 
 
-@pytest.mark.parametrize("H,d,dim,width,slope", [(2, 128, 256, 1000, 0.0), (4, 64, 512, 3, 0.5), (2, 128, 384, 0, 0.0)])
-def test_layer_steps_match_the_oracle(ctx, H, d, dim, width, slope):
+@pytest.mark.parametrize("H,d,dim,width,slope,relu_dim", [
+    (2, 128, 256, 1000, 0.0, 256), (4, 64, 512, 3, 0.5, 256), (2, 128, 384, 0, 0.0, 256),
+    # feed-forward groups of 128 * ReluMult (model_dim.h:66): ReluMult 2, 3 and 4
+    (2, 128, 256, 1000, 0.0, 512), (3, 128, 384, 5, 0.5, 3 * 384), (2, 64, 256, 2, 0.0, 2 * 512)])
+def test_layer_steps_match_the_oracle(ctx, H, d, dim, width, slope, relu_dim):
     B, max_len, steps = 4, 12, 6
     qsum = H * d
     rng = np.random.default_rng(H * d + width)
     mat = lambda n, k: np.clip(np.rint(rng.standard_normal((n, k)) * 32), -127, 127).astype(np.int8)
     mats = {"qk": mat(qsum, dim), "qv": mat(qsum, dim), "k": mat(qsum, dim), "v": mat(qsum, dim),
-            "combiner": mat(dim, qsum * 4), "expand": mat(qsum, dim), "contract": mat(dim, qsum)}
+            "combiner": mat(dim, qsum * 4), "expand": mat(relu_dim, dim), "contract": mat(dim, relu_dim)}
     scales = (0.031, 0.027, 0.035)
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
     layer = {"proj": dev(np.concatenate([mats[n] for n in ("qk", "qv", "k", "v")]).view(np.uint8)),

@@ -43,6 +43,30 @@ def test_producer_bit_exact(ctx, dtype, d, H, with_rope):
     assert not q.cpu().numpy()[7].any() and s.cpu().numpy()[1, 9] == 0
 
 
+@pytest.mark.parametrize("group", [256, 384, 512])
+@pytest.mark.parametrize("n", [5, 700])
+def test_producer_wide_groups_bit_exact(ctx, group, n):
+    """The feed-forward groups of 128 * ReluMult (NormalizeState(relu, headCount), cpu_infer.cpp:519-524): int32 sums in
+    two planes, ReLU on the int8 result; rotation and e4m3 are refused for such groups."""
+    H = 3
+    rng = np.random.default_rng(group + n)
+    a = rng.integers(-20000, 20000, (n, H * group)).astype(np.int32)
+    b = rng.integers(-20000, 20000, (n, H * group)).astype(np.int32)
+    a[2, group:2 * group] = -b[2, group:2 * group]           # a group of zeros
+    want_q, want_s = orc.rope_normalize_rows(orc.I8, a + b, H)
+    want_q = np.where(want_q.view(np.int8) < 0, 0, want_q.view(np.int8)).astype(np.int8).view(np.uint8)
+    planes = torch.from_numpy(np.stack([a, b])).cuda()
+    q, s = ctx.rope_normalize_rows(planes, H, capi.I8, relu=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy(), want_q) and np.array_equal(s.cpu().numpy(), want_s)
+    assert not q.cpu().numpy()[2, group:2 * group].any()
+    x = torch.from_numpy((a + b).astype(np.float32)).cuda()
+    with pytest.raises(capi.TsattnError):
+        ctx.rope_normalize_rows(x, H, capi.E4M3)
+    with pytest.raises(capi.TsattnError):
+        ctx.rope_normalize_rows(x, H, capi.I8, pos=torch.zeros(n, dtype=torch.int32, device="cuda"), rope=ctx.fill_rope_table(128, 4))
+
+
 def test_producer_int32_source_reverse_direction_and_clamped_positions(ctx):
     H, d, n = 4, 128, 70
     rng = np.random.default_rng(1)

@@ -431,7 +431,7 @@ def add_lookup_product(ctx, layer, cache, t, rope, state, workspace=None, scratc
     f32 = np.float32
     sc = scratch if scratch is not None else {}
     if "planes" not in sc:
-        sc["planes"] = torch.empty((16, B, max(4 * qsum, dim)), dtype=torch.int32, device=state.device)
+        sc["planes"] = torch.empty((16, B, max(4 * qsum, dim, layer["expand"].shape[0])), dtype=torch.int32, device=state.device)
         sc["v_scale"] = torch.full((B, H), VEC_SCALE, dtype=torch.float32, device=state.device)
     planes_buf, v_scale = sc["planes"], sc["v_scale"]
     if pending is not None:   # the previous layer's contract product, still in parts: state += sum * scale, then normalise
@@ -498,7 +498,7 @@ def add_lookup_product_prompt(ctx, layer, cache, seq_offset, pos, rope, state, s
     # every product with its normalisation as epilogue (large products never write their int32 sums); one scratch
     # buffer for whichever falls back to two launches
     key_mult = float(f32(layer["qv_scale"]) * f32(VEC_SCALE) * f32(np.sqrt(f32(1.0) / f32(dim))))
-    room = torch.empty((16 if n <= 128 else 1) * n * max(4 * qsum, dim), dtype=torch.int32, device=state.device)
+    room = torch.empty((16 if n <= 128 else 1) * n * max(4 * qsum, dim, layer["expand"].shape[0]), dtype=torch.int32, device=state.device)
     q4, qv_scale = ctx.matmul_normalize(norm, layer["proj"], 4 * H, capi.I8, room, pos=pos, rope=rope, scale_mult=key_mult,
                                         rope_heads=2 * H, scale_heads=(H, H))      # scales as [head][token] planes
     qk, qv, k, v = q4[:, :qsum], q4[:, qsum:2 * qsum], q4[:, 2 * qsum:3 * qsum], q4[:, 3 * qsum:]

@@ -431,7 +431,12 @@ static int fill_produce(const tsattn_produce_args *a, const char *who, tsattn::P
     *empty = false;
     if (!dtype_ok(a->dst_dtype) || (a->src_dtype != TSATTN_SRC_F32 && a->src_dtype != TSATTN_SRC_I32))
         return fail(TSATTN_ERR_UNSUPPORTED, "%s: dtypes %d -> %d", who, a->src_dtype, a->dst_dtype);
-    if (!head_dim_ok(a->head_dim)) return fail(TSATTN_ERR_UNSUPPORTED, "%s: head_dim %d (64 or 128 supported)", who, a->head_dim);
+    // groups wider than a head (the feed-forward groups of 128 * ReluMult): int8 results, no rotation
+    const bool wide_group = a->head_dim == 256 || a->head_dim == 384 || a->head_dim == 512;
+    if (!head_dim_ok(a->head_dim) && !wide_group)
+        return fail(TSATTN_ERR_UNSUPPORTED, "%s: head_dim %d (64, 128; 256, 384, 512 without rotation)", who, a->head_dim);
+    if (wide_group && (a->pos || a->dst_dtype != TSATTN_I8))
+        return fail(TSATTN_ERR_UNSUPPORTED, "%s: groups of %d values are normalised to int8 and not rotated", who, a->head_dim);
     if (a->n_rows < 0 || a->n_heads <= 0) return fail(TSATTN_ERR_BAD_ARG, "%s: negative size", who);
     if (a->n_rows == 0) { *empty = true; return TSATTN_OK; }
     if (!a->src || !a->dst) return fail(TSATTN_ERR_BAD_ARG, "%s: null data pointer", who);
@@ -524,7 +529,7 @@ int tsattn_matmul_i8(tsattn_handle_t h, const tsattn_matmul_args *a, void *strea
         // the producer on the int32 result: its source is the product
         if (a->mode != TSATTN_MM_I32_PLANES) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: an epilogue goes with the planes mode");
         tsattn_produce_args e = *a->epilogue;
-        if (!head_dim_ok(e.head_dim) || a->n % e.head_dim) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: n %lld is not a whole number of the epilogue's heads", (long long)a->n);
+        if (e.head_dim <= 0 || a->n % e.head_dim) return fail(TSATTN_ERR_BAD_ARG, "tsattn_matmul_i8: n %lld is not a whole number of the epilogue's heads", (long long)a->n);
         e.src_dtype = TSATTN_SRC_I32; e.src = a->out; e.src_pitch = a->n; e.n_rows = a->m; e.n_heads = (int)(a->n / e.head_dim);
         e.src_planes = 1; e.src_plane_stride = 0;
         bool empty;

@@ -683,7 +683,8 @@ hipError_t launch_matmul_i8(const GemmParams &p, hipStream_t st, int *planes_out
             const bool offsets_fit = q.ep.dst_pitch < (1 << 23) && (!q.ep.resid || q.ep.resid_pitch < (1 << 21)) &&
                                      (!q.ep.pos || q.ep.rope_len * p.ep_head_dim * 4 < ((int64_t)1 << 31));
             const bool one_operand = !(q.ep.resid && q.ep.pos); // (registers for the old state or for cos and sin)
-            if (p.m > 32 * GS_MB && wide >= 512 && p.ep_dst_dtype == TSATTN_I8 && offsets_fit && one_operand) {
+            const bool head_group = p.ep_head_dim == 64 || p.ep_head_dim == 128; // (wider groups: the producer's own launch)
+            if (p.m > 32 * GS_MB && wide >= 512 && p.ep_dst_dtype == TSATTN_I8 && offsets_fit && one_operand && head_group) {
                 if (p.ep_head_dim == 128) hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 128>), dim3((unsigned)wide), dim3(GW_THREADS), gw_lds_bytes(128), st, q);
                 else hipLaunchKernelGGL((gemm_wide_kernel<TSATTN_MM_I32, 64>), dim3((unsigned)wide), dim3(GW_THREADS), gw_lds_bytes(64), st, q);
                 return hipGetLastError();

@@ -175,7 +175,8 @@ hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head
     if (n_pairs == 0) return hipSuccess;
     // a small launch (one token per sequence) is a chain of waits -- positions, rows, the ordered sums -- that more,
     // smaller workgroups get through sooner; a large one is bound by memory and takes 32 pairs per workgroup
-    const bool few = n_pairs <= 4096;
+    // (groups wider than a head -- the feed-forward groups of 128 * ReluMult -- always: 32 of them would not fit in LDS)
+    const bool few = n_pairs <= 4096 || head_dim > 128;
     const int per_wg = few ? PR_PAIRS_FEW : PR_PAIRS;
     dim3 grid((unsigned)((n_pairs + per_wg - 1) / per_wg)), block(256);
 #define TSATTN_PR(D_, DST_, I32_)                                                                                   \
@@ -191,6 +192,15 @@ hipError_t launch_rope_normalize(const ProduceParams &p, int dst_dtype, int head
     else if (head_dim == 64 && dst_dtype == TSATTN_I8 && src_i32) TSATTN_PR(64, TSATTN_I8, true);
     else if (head_dim == 64 && dst_dtype == TSATTN_E4M3 && !src_i32) TSATTN_PR(64, TSATTN_E4M3, false);
     else if (head_dim == 64 && dst_dtype == TSATTN_E4M3 && src_i32) TSATTN_PR(64, TSATTN_E4M3, true);
+#define TSATTN_PR_WIDE(D_)                                                                                          \
+    else if (head_dim == D_ && dst_dtype == TSATTN_I8 && !src_i32)                                                  \
+        hipLaunchKernelGGL((rope_normalize_kernel<D_, TSATTN_I8, false, PR_PAIRS_FEW>), grid, block, 0, st, p);     \
+    else if (head_dim == D_ && dst_dtype == TSATTN_I8 && src_i32)                                                   \
+        hipLaunchKernelGGL((rope_normalize_kernel<D_, TSATTN_I8, true, PR_PAIRS_FEW>), grid, block, 0, st, p);
+    TSATTN_PR_WIDE(256)
+    TSATTN_PR_WIDE(384)
+    TSATTN_PR_WIDE(512)
+#undef TSATTN_PR_WIDE
     else return hipErrorInvalidValue;
 #undef TSATTN_PR
     return hipGetLastError();

@@ -246,8 +246,8 @@ TLayerComputer::TLayerComputer(tsattn_handle_t handle, const TModelDims &dims, i
     TS_VERIFY(dims.QDim == dims.TTDim && (dims.QDim == 64 || dims.QDim == 128), "QDim %d TTDim %d: equal, 64 or 128", dims.QDim, dims.TTDim);
     TS_VERIFY(dims.Dim % STATE_NORM_TILE == 0, "Dim %d is not a multiple of %d", dims.Dim, STATE_NORM_TILE);
     // NormalizeState(relu, headCount) takes groups of 128 * ReluMult whatever the head width (gpt/train/cpu_infer.cpp:519-524,
-    // model_dim.h:66); the producer kernels normalise groups of 64 or 128
-    TS_VERIFY(dims.ReluMult == 1, "ReluMult %d: feed-forward groups of %d are not supported (128 is)", dims.ReluMult, 128 * dims.ReluMult);
+    // model_dim.h:66); the producer kernels normalise groups of up to 512
+    TS_VERIFY(dims.ReluMult >= 1 && dims.ReluMult <= 4, "ReluMult %d: feed-forward groups of 128 to 512 values are supported", dims.ReluMult);
     ReluDim = dims.GetReluDim();
     const size_t n = (size_t)maxRows, qsum = (size_t)dims.GetQSum();
     auto alloc = [](void **p, size_t bytes) { CheckHip(hipMalloc(p, bytes), "hipMalloc(layer buffers)"); };

@@ -164,7 +164,7 @@ constexpr int COMBINER_REP = 4;        // gpt/model_params/model_dim.h:12
 // per token call: the four projections are one product when QK, QV, K and V lie one after the other in memory, the
 // normalisations that follow them are one call, K-split products leave their parts for the consumer to add up, and the
 // combiner's AddScaled is done by the normalisation after it.  QDim == TTDim == 64 or 128; the feed-forward width is
-// reluDim = HeadCount * 128 * ReluMult with ReluMult 1.
+// reluDim = HeadCount * 128 * ReluMult with ReluMult 1 to 4.
 struct TInferModel; // below
 
 class TLayerComputer
