@@ -78,6 +78,35 @@ def test_prefill_replays(ctx, dtype, window, slope):
         assert torch.equal(out, want)
 
 
+def test_several_spans_per_row_replay(ctx):
+    """Two prefill launches over the rows' first and second spans and the launch that combines them, as one graph."""
+    dtype, H, d, n = capi.I8, 2, 128, 400
+    g0 = torch.Generator(device="cuda").manual_seed(9)
+    q, qs = ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g0), H, dtype)
+    k, ks = ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g0), H, dtype)
+    v, vs = ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g0), H, dtype)
+    t = torch.arange(n, dtype=torch.int32, device="cuda")
+    spans = [(torch.clamp(t - 40, min=0), t - 1), (torch.zeros_like(t), torch.clamp(t - 300, min=-1))]   # a window and a far prefix
+    parts = torch.zeros((2, n, H * d), dtype=torch.float32, device="cuda")
+    swl = torch.zeros((2, H, n), dtype=torch.float32, device="cuda")
+    out = torch.zeros((n, H * d), dtype=torch.float32, device="cuda")
+    def run():
+        for i, (st, fi) in enumerate(spans):
+            ctx.compute_val_lookup(dtype, H, q, k, v, qs, ks, vs, st.contiguous(), fi.contiguous(), 0.25, out=parts[i], sum_weight_log=swl[i])
+        ctx.merge_lookups(parts, swl, out=out)
+    run()
+    torch.cuda.synchronize()
+    want = out.clone()
+    assert want.abs().max() > 0
+    graph = capture(run)
+    for _ in range(3):
+        out.zero_(); parts.zero_(); swl.zero_()
+        eager_noise()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+
+
 @pytest.mark.parametrize("window,splits", [(64, 1), (10 ** 6, 0), (10 ** 6, 5)])
 def test_fused_append_and_decode_replays(ctx, window, splits):
     """Every replay appends one more row per sequence and attends over the longer cache; the arrival counters of the
