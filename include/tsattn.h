@@ -117,9 +117,23 @@ typedef struct tsattn_prefill_args {
     int64_t kv_out_pitch;
     int kv_rep;                /* 1..4 */
     float kv_mult;
+    /* Optional scratch for rows with long spans (NULL = none).  With at least tsattn_prefill_workspace_bytes(n_tokens,
+     * n_heads, head_dim) bytes here (16-byte aligned) and span_len_hint >= 512, head_dim 128 and no ALiBi slope, the
+     * call first writes V once as f16 with the value scales folded in, transposed, into the workspace, and the attention
+     * kernel streams K and that copy through LDS without touching them in registers (the reference keeps such a
+     * transposed copy of V too: Transpose, gpt_cuda.cu:501, VT of TAttentionComputeCtx).  Same result within the
+     * output tolerance; the workspace holds nothing between calls.  span_len_hint: the typical number of keys of a
+     * row -- the layer's attention width clipped to the sequence length (gpt/model_params/model_dim.h:83-91); 0 =
+     * unknown.  Only the choice of kernel depends on it. */
+    void *workspace;
+    int64_t workspace_bytes;
+    int64_t span_len_hint;
 } tsattn_prefill_args;
 
 int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream);
+/* Bytes of tsattn_prefill_args.workspace that let a call of this size take the long-span kernel (0: that kernel does
+ * not serve this head_dim). */
+size_t tsattn_prefill_workspace_bytes(int64_t n_tokens, int n_heads, int head_dim);
 
 /* ---------------------------------------------------------------------------------------------
  * Decode of one new token per sequence over a KV cache.  Replaces

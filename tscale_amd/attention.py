@@ -59,6 +59,7 @@ class AttentionContext:
         capi.check(self.lib.tsattn_create(ctypes.byref(cfg), ctypes.byref(h)))
         self.handle = h
         self.device = torch.device("cuda", device)
+        self._workspace = None  # scratch of the long-span prefill kernel, grown on demand
 
     def close(self):
         if self.handle:
@@ -276,13 +277,17 @@ class AttentionContext:
     # ---- prefill --------------------------------------------------------------------------------
     def compute_val_lookup(self, dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, span_start, span_finish,
                            alibi_slope, out=None, out_f16=False, sum_weight_log=None, k_global_scale=None,
-                           debug_qk_acc=None, causal_period=0, span_tiles=None, kv_product=None, want_out=True):
+                           debug_qk_acc=None, causal_period=0, span_tiles=None, kv_product=None, want_out=True,
+                           span_len_hint=0, workspace=None):
         """q,k,v: uint8 [n_tokens, n_heads*d] (row pitch = stride(0)); scales f32 [n_heads, n_tokens] or numbers.
         causal_period: launch-order hint for batches of equal-length sequences under a wide causal window (the
         common sequence length); never changes the result.  span_tiles: what build_span_tiles made of these spans.
         kv_product = (k, kv_out, rep, mult): KVProduct of the f32 result with the tokens' K vectors, written by the same
         launch (k uint8 [n_tokens, H*d], kv_out uint8 [n_tokens, H*rep*d]); with want_out=False the result itself is
-        not written and None is returned."""
+        not written and None is returned.
+        span_len_hint: typical number of keys per row (the layer's attention width clipped to the sequence length); from
+        512 on, with head width 128 and no slope, the call goes through the long-span kernel, which needs a workspace
+        (uint8 tensor; by default one that this context keeps and grows on demand)."""
         n_tokens, hd = q.shape
         d = hd // n_heads
         assert want_out or kv_product is not None
@@ -316,6 +321,15 @@ class AttentionContext:
             a.kv_rep, a.kv_mult = int(kv_rep), float(kv_mult)
         a.causal_period = int(causal_period)
         a.span_tiles = _ptr(span_tiles)
+        a.span_len_hint = int(span_len_hint)
+        if span_len_hint >= 512:
+            need = int(self.lib.tsattn_prefill_workspace_bytes(n_tokens, n_heads, d))
+            if workspace is None and need > 0:
+                if self._workspace is None or self._workspace.numel() < need or self._workspace.device != q.device:
+                    self._workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+                workspace = self._workspace
+            if workspace is not None:
+                a.workspace, a.workspace_bytes = _ptr(workspace), workspace.numel() * workspace.element_size()
         capi.check(self.lib.tsattn_prefill(self.handle, ctypes.byref(a), _stream_ptr()))
         return out
 

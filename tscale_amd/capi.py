@@ -44,6 +44,7 @@ class PrefillArgs(_c.Structure):
         ("debug_pitch", _c.c_int64), ("span_tiles", _c.c_void_p), ("causal_period", _c.c_int64),
         ("kv_k", _c.c_void_p), ("kv_k_pitch", _c.c_int64), ("kv_out", _c.c_void_p), ("kv_out_pitch", _c.c_int64),
         ("kv_rep", _c.c_int), ("kv_mult", _c.c_float),
+        ("workspace", _c.c_void_p), ("workspace_bytes", _c.c_int64), ("span_len_hint", _c.c_int64),
     ]
 
 
@@ -117,7 +118,7 @@ class MergeArgs(_c.Structure):
     ]
 
 
-EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill",
+EXPORTS = ["tsattn_scratch_bytes", "tsattn_create", "tsattn_destroy", "tsattn_last_error", "tsattn_prefill", "tsattn_prefill_workspace_bytes",
            "tsattn_decode", "tsattn_decode_static", "tsattn_cache_append", "tsattn_cache_fill", "tsattn_merge_lookups", "tsattn_span_tiles_count", "tsattn_build_span_tiles", "tsattn_rope_normalize_rows", "tsattn_fill_rope_table", "tsattn_kv_product", "tsattn_matmul_i8", "tsattn_embed_rows", "tsattn_softmax_rows", "tsattn_sample_rows", "tsattn_quantize_rows", "tsattn_build_spans", "tsattn_debug_read_counters", "tsattn_version"]
 
 _lib = None
@@ -142,6 +143,8 @@ def load():
         L.tsattn_version.restype = _c.c_char_p
         L.tsattn_prefill.restype = _c.c_int
         L.tsattn_prefill.argtypes = [_c.c_void_p, _c.POINTER(PrefillArgs), _c.c_void_p]
+        L.tsattn_prefill_workspace_bytes.restype = _c.c_size_t
+        L.tsattn_prefill_workspace_bytes.argtypes = [_c.c_int64, _c.c_int, _c.c_int]
         L.tsattn_decode.restype = _c.c_int
         L.tsattn_decode.argtypes = [_c.c_void_p, _c.POINTER(DecodeArgs), _c.c_void_p]
         L.tsattn_debug_read_counters.restype = _c.c_int

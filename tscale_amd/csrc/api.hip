@@ -270,9 +270,26 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     p.dbg = a->debug_qk_acc; p.dbg_pitch = a->debug_pitch;
     p.n_tokens = (int)a->n_tokens; p.n_heads = a->n_heads;
     p.period_tiles = (a->causal_period > 0 && a->causal_period % 128 == 0 && a->n_tokens % a->causal_period == 0) ? (int)(a->causal_period / 128) : 0;
+    // Long spans with room for the f16 copy of V: the kernel that streams K and that copy through LDS.  (It addresses
+    // K and the copy with 31-bit byte offsets.)
+    if (a->workspace && a->span_len_hint >= 512 && a->head_dim == 128 && a->alibi_slope == 0.0f && !a->debug_qk_acc && !a->kv_out) {
+        const size_t need = tsattn::prefill_long_workspace_bytes(a->n_tokens, a->n_heads, a->head_dim);
+        const int64_t vt_pitch = tsattn::prefill_long_vt_pitch(a->n_tokens);
+        if (!aligned16(a->workspace)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: workspace must be 16-byte aligned");
+        if (need != 0 && a->workspace_bytes >= (int64_t)need && a->n_tokens * a->k_pitch < ((int64_t)1 << 31) && 128 * vt_pitch * 2 < ((int64_t)1 << 31)) {
+            p.vt = a->workspace;
+            p.vt_pitch = vt_pitch;
+        }
+    }
     hipError_t e = tsattn::launch_prefill(p, a->dtype, a->head_dim, a->out_dtype, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "prefill launch");
     return TSATTN_OK;
+}
+
+size_t tsattn_prefill_workspace_bytes(int64_t n_tokens, int n_heads, int head_dim)
+{
+    if (n_tokens <= 0 || n_heads <= 0) return 0;
+    return tsattn::prefill_long_workspace_bytes(n_tokens, n_heads, head_dim);
 }
 
 int tsattn_decode(tsattn_handle_t h, const tsattn_decode_args *a, void *stream)

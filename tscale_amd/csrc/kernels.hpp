@@ -72,10 +72,20 @@ struct PrefillParams {
     int64_t kv_out_pitch;
     int kv_rep;
     float kv_mult;
+    // optional scratch of the long-range kernel (vt != nullptr selects it): room for V as f16, transposed
+    void *vt;
+    int64_t vt_pitch; // halves per (head, x) row
     WgMap map;        // set by the launcher: how workgroup ids map to (head, query tile)
 };
 
 hipError_t launch_prefill(const PrefillParams &p, int dtype, int head_dim, int out_dtype, hipStream_t st);
+
+// The long-range kernel (head width 128, no ALiBi slope) and its scratch: V as f16 [head][x][vt_pitch], the column of
+// token t at VT_PAD + t (tokens of every 16 reordered), every other column zero.
+constexpr int VT_PAD = 32;
+inline int64_t prefill_long_vt_pitch(int64_t n_tokens) { return (n_tokens + 63) / 64 * 64 + 256; }
+size_t prefill_long_workspace_bytes(int64_t n_tokens, int n_heads, int head_dim);
+hipError_t launch_prefill_long(const PrefillParams &p, int dtype, int out_dtype, hipStream_t st);
 
 hipError_t launch_quantize_rows(int src_dtype, int dst_dtype, const void *src, int64_t src_pitch, int64_t n_rows,
                                 int n_heads, int head_dim, void *dst, int64_t dst_pitch, float *scale,

@@ -48,9 +48,9 @@ struct WgMap {
 
 // Plans the mapping of a launch of n_qtiles * n_heads workgroups.  The period-aware order is usable only if every
 // XCD's share of the grid is a whole number of (head group, sequence) units; units are then walked in groups whose
-// K and V rows (2 * period * d bytes per head) stay within about the size of the XCD's 4 MB L2 (the rows are
+// K and V rows (kv_bytes_per_value * period * d bytes per head: 2 for 8-bit K and V) stay within about the size of the XCD's 4 MB L2 (the rows are
 // streamed, so slightly more than it still pays).
-inline WgMap wg_plan(int n_qtiles, int n_heads, int head_dim, int rows_per_tile, int period_tiles)
+inline WgMap wg_plan(int n_qtiles, int n_heads, int head_dim, int rows_per_tile, int period_tiles, int kv_bytes_per_value = 2)
 {
     WgMap m;
     m.period_tiles = period_tiles;
@@ -64,7 +64,7 @@ inline WgMap wg_plan(int n_qtiles, int n_heads, int head_dim, int rows_per_tile,
     const int64_t n_wg = (int64_t)n_qtiles * n_heads, per_xcd = n_wg / 8;
     if (T > 1 && n_wg % 8 == 0 && per_xcd % (T * hg) == 0 && n_qtiles % T == 0) {
         const int R = (int)(per_xcd / (T * hg));
-        const int64_t unit_bytes = (int64_t)2 * T * rows_per_tile * head_dim * hg;
+        const int64_t unit_bytes = (int64_t)kv_bytes_per_value * T * rows_per_tile * head_dim * hg;
         int G = 1;
         for (int c = 1; c <= R; ++c)
             if (R % c == 0 && c * unit_bytes <= (5 << 20)) G = c;
