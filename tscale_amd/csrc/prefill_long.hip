@@ -190,13 +190,22 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
                 fb = ((w_min_b + 1 - kb_first) >> 5) - 1;
             }
         }
-        // iterations whose two steps are complete and unmasked: K.Q^T of sub-tiles 2 it and 2 it + 1, softmax of
-        // 2 it - 1 and 2 it, V^T.P^T of 2 it - 2 and 2 it - 1
+        // Iterations [it_f0, it_f1): both steps complete and no span cuts through them -- K.Q^T of sub-tiles 2 it and
+        // 2 it + 1, softmax of 2 it - 1 and 2 it (inside every span), V^T.P^T of 2 it - 2 and 2 it - 1.  Before and after
+        // them, up to it_last (the iteration of the wave's last V^T.P^T), the steps look at the spans; a key outside a
+        // row's span -- a sub-tile the wave does not need at all included -- gets the weight zero.
         int it_f0 = max((ua + 3) >> 1, (fa + 2) >> 1);
         int it_f1 = min(fb >> 1, (ub - 1) >> 1) + 1; // one past the last
-        if (fb < fa || it_f1 < it_f0) it_f1 = it_f0 = 0;
+        int it_last = (ub + 2) >> 1;
+        if (ub < ua) it_last = -1, it_f0 = it_f1 = 0;
+        else if (fb < fa || it_f1 <= it_f0) it_f0 = it_f1 = 0;
+        it_last = min(it_last, n_tiles);
         it_f0 = __builtin_amdgcn_readfirstlane(it_f0);
         it_f1 = __builtin_amdgcn_readfirstlane(it_f1);
+        it_last = __builtin_amdgcn_readfirstlane(it_last);
+        // in span <=> (unsigned)(key - sp_a) <= sp_b - sp_a; per lane the keys are first key + 4 g + {0..3, 8..11, ...}
+        const int mask_lo = sp_b >= sp_a ? sp_a - 4 * g : 0x40000000;
+        const unsigned mask_w = sp_b >= sp_a ? (unsigned)(sp_b - sp_a) : 0u;
 
         // ---- requests: memory -> LDS ------------------------------------------------------------------------
         auto rsrc = [](const void *base, int64_t bytes) {
@@ -226,8 +235,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
         }
         const int64_t k_step = (int64_t)PL_BN * p.k_pitch;
         uint32_t k_soff = 0, v_soff = 0, s_soff = 0;
-        int dma_stage = 0;
-        auto request_tile = [&]() __attribute__((always_inline)) { // the next tile in sequence -> the next stage
+        auto request_tile = [&](int dma_stage) __attribute__((always_inline)) { // the next tile in sequence -> that stage
             uint8_t *const kd = pl_lds + PL_K_OFF + dma_stage * PL_K_BYTES + wave * 2048;
             uint8_t *const vd = pl_lds + PL_V_OFF + dma_stage * PL_V_BYTES + wave * 4096;
 #pragma unroll
@@ -241,7 +249,6 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
             k_soff += (uint32_t)k_step;
             v_soff += PL_BN * 2;
             s_soff += PL_BN * 4;
-            dma_stage = dma_stage == PL_STAGES - 1 ? 0 : dma_stage + 1;
         };
 #define PL_WAIT_TILE asm volatile("s_waitcnt vmcnt(7)" ::: "memory") // all but the newest tile's seven requests have landed
 #define PL_WAIT_ALL asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
@@ -303,57 +310,64 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
             va[m] = *(const v8h *)(vt_tile + dt * 4096 + vx[sv][grp]);
         };
 
-        // Weights of two keys (accumulator registers 2 pr, 2 pr + 1) on the common path: no mask, no maximum.
-        auto weights_pair = [&](const typename Qk::acc_t &a, int pr, v2h &out) __attribute__((always_inline)) {
+        // Weights of two keys (accumulator registers 2 pr, 2 pr + 1) against the zero vector's logit: no maximum.
+        // MASKED: a weight whose key lies outside the row's span becomes zero (rel_lo: the span's start relative to this
+        // lane's first key of the sub-tile; span_w: its length - 1, or a bound no key meets for a row without keys).
+        auto weights_pair = [&](auto masked_tag, const typename Qk::acc_t &a, int pr, int rel_lo, unsigned span_w, v2h &out) __attribute__((always_inline)) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
             const int r = 2 * pr;
             const v4f kq = ksv[pr >> 1];
             const float k0 = kq[2 * (pr & 1)], k1 = kq[2 * (pr & 1) + 1];
-            const float p0 = fast_exp2((Qk::to_float(a, r) * k0) * qs);
-            const float p1 = fast_exp2((Qk::to_float(a, r + 1) * k1) * qs);
+            float p0 = fast_exp2((Qk::to_float(a, r) * k0) * qs);
+            float p1 = fast_exp2((Qk::to_float(a, r + 1) * k1) * qs);
+            if (MASKED) {
+                const int off = 8 * (r >> 2) + (r & 3); // key of register r relative to the lane's first key
+                p0 = ((unsigned)(off - rel_lo) <= span_w) ? p0 : 0.0f;
+                p1 = ((unsigned)(off + 1 - rel_lo) <= span_w) ? p1 : 0.0f;
+            }
             out = v2h{(_Float16)p0, (_Float16)p1};
         };
 
-        // ---- one step on the common path -----------------------------------------------------------------------
-        // s = T & 1.  kt: K sub-tile T; ks_next: key scales of sub-tile T (for the next step); v_next: the V tile and
-        // half that hold sub-tile T - 1 (for the next step).
-        auto fast_step = [&](auto s_tag, const uint8_t *kt, const float *ks_next, const uint8_t *v_next) __attribute__((always_inline)) {
+        // ---- one step ------------------------------------------------------------------------------------------------
+        // s = T & 1.  kt: K sub-tile T; ks_next: key scales of sub-tile T (for the next step); v_next: the V tile that holds
+        // sub-tile T - 1 in half s (for the next step).  MASKED: the softmax of sub-tile T - 1 (first key key0) looks at the
+        // spans.  Order: four V^T.P^T, K.Q^T, four V^T.P^T, with the weight sums and eight pairs of weights between them.
+        auto fast_step = [&](auto s_tag, auto masked_tag, int key0, const uint8_t *kt, const float *ks_next, const uint8_t *v_next) __attribute__((always_inline)) {
             constexpr int s = decltype(s_tag)::value;
             typename Qk::acc_t &accC = acc[s ^ 1];
             const v2h(&pc)[8] = pw[s];
             v2h(&pn)[8] = pw[s ^ 1];
+            const int rel_lo = mask_lo - key0;
             kop_t kop[QS];
             read_k(kt, kop);
+            // what the previous step asked for (this step's V^T operands and key scales) has arrived once only the four
+            // reads above are outstanding: one wait here instead of one in front of every first use
+            __builtin_amdgcn_s_waitcnt(0xc07f | (4 << 8)); // lgkmcnt(4), the other counters untouched
             PL_FENCE;
-            // order: four V^T.P^T, K.Q^T, four V^T.P^T, the four sums; eight pairs of weights between them
             int pr = 0;
             typename Qk::acc_t accN = {0};
+            auto pair = [&]() __attribute__((always_inline)) {
+                weights_pair(masked_tag, accC, pr, rel_lo, mask_w, pn[pr]);
+                ++pr;
+                if ((pr & 1) == 0) ksv[(pr >> 1) - 1] = *(const v4f *)(ks_next + 8 * ((pr >> 1) - 1));
+                PL_FENCE;
+            };
 #pragma unroll
             for (int m = 0; m < 2 * DT; ++m) {
                 pv_mfma(m, pc);
                 read_v(m, v_next, s);
+                if (m & 1) sum_mfma(m >> 1, pc);
                 PL_FENCE;
-                if (m == 0 || m == 2 || m == 3 || m == 4 || m == 6 || m == 7) {
-                    weights_pair(accC, pr, pn[pr]);
-                    ++pr;
-                    if ((pr & 1) == 0) ksv[(pr >> 1) - 1] = *(const v4f *)(ks_next + 8 * ((pr >> 1) - 1));
-                    PL_FENCE;
-                }
+                if (m == 0 || m == 2 || m == 3 || m == 4 || m == 6 || m == 7) pair();
                 if (m == DT - 1) {
 #pragma unroll
                     for (int st = 0; st < QS; ++st) {
                         accN = qk.step(kop[st], st, accN);
                         PL_FENCE;
-                        if (st == QS / 2 - 1 || st == QS - 1) {
-                            weights_pair(accC, pr, pn[pr]);
-                            ++pr;
-                            if ((pr & 1) == 0) ksv[(pr >> 1) - 1] = *(const v4f *)(ks_next + 8 * ((pr >> 1) - 1));
-                            PL_FENCE;
-                        }
+                        if (st == QS / 2 - 1 || st == QS - 1) pair();
                     }
                 }
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) sum_mfma(i, pc);
             acc[s] = accN;
             PL_FENCE;
         };
@@ -433,41 +447,63 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
             for (int m = 0; m < 2 * DT; ++m) va[m] = v8h{0};
 #pragma unroll
             for (int c4 = 0; c4 < 4; ++c4) ksv[c4] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-            k_soff = 0, v_soff = 0, s_soff = 0, dma_stage = 0;
-            request_tile();
-            request_tile();
+            k_soff = 0, v_soff = 0, s_soff = 0;
+            request_tile(0);
+            request_tile(1);
             PL_WAIT_TILE;
             PL_BARRIER;
             int stage = 0, it = 0;
-            // (three loops rather than one with a branch: each keeps only what it needs in registers)
-            auto general_iters = [&](int end) __attribute__((always_inline)) {
-                for (; it < end; ++it) {
-                    const uint8_t *const kt = pl_lds + PL_K_OFF + stage * PL_K_BYTES;
-                    const uint8_t *const vt_tile = pl_lds + PL_V_OFF + stage * PL_V_BYTES;
-                    const float *const ksp = (const float *)(pl_lds + PL_KS_OFF + stage * PL_KS_BYTES) + 4 * g;
-                    request_tile(); // (past the last tile: rows that are never computed with, or zeros past the end)
-                    general_step(std::integral_constant<int, 0>{}, safe_tag, 2 * it, kt, ksp, vt_tile);
-                    general_step(std::integral_constant<int, 1>{}, safe_tag, 2 * it + 1, kt + 32 * 128, ksp + 32, vt_tile);
+            // Separate loops rather than one with branches: each keeps only what it needs in registers, and a loop body
+            // without branches keeps the order it was written in.  Each loop is unrolled over the three stages, entered at
+            // the current one, so that every LDS address is a lane constant plus an immediate.
+            auto one = [&](auto mode_tag, int st_k, int st_dma) __attribute__((always_inline)) { // st_k: a constant in the unrolled loop
+                constexpr int MODE = decltype(mode_tag)::value; // 0: slow path, 1: spans looked at, 2: common, 3: nothing to compute
+                const uint8_t *const kt = pl_lds + PL_K_OFF + st_k * PL_K_BYTES;
+                const uint8_t *const vt_tile = pl_lds + PL_V_OFF + st_k * PL_V_BYTES;
+                const float *const ksp = (const float *)(pl_lds + PL_KS_OFF + st_k * PL_KS_BYTES) + 4 * g;
+                request_tile(st_dma); // (past the last tile: rows that are never computed with, or zeros past the end)
+                if (MODE == 0) {
+                    general_step(std::integral_constant<int, 0>{}, std::true_type{}, 2 * it, kt, ksp, vt_tile);
+                    general_step(std::integral_constant<int, 1>{}, std::true_type{}, 2 * it + 1, kt + 32 * 128, ksp + 32, vt_tile);
+                } else if (MODE == 1) {
+                    const int key0 = kb_first + 64 * it - 32; // first key of sub-tile 2 it - 1
+                    fast_step(std::integral_constant<int, 0>{}, std::true_type{}, key0, kt, ksp, vt_tile);
+                    fast_step(std::integral_constant<int, 1>{}, std::true_type{}, key0 + 32, kt + 32 * 128, ksp + 32, vt_tile);
+                } else if (MODE == 2) {
+                    fast_step(std::integral_constant<int, 0>{}, std::false_type{}, 0, kt, ksp, vt_tile);
+                    fast_step(std::integral_constant<int, 1>{}, std::false_type{}, 0, kt + 32 * 128, ksp + 32, vt_tile);
+                }
+                PL_WAIT_TILE;
+                PL_BARRIER;
+            };
+            auto iterations = [&](auto mode_tag, int end) __attribute__((always_inline)) {
+                constexpr int MODE = decltype(mode_tag)::value;
+                // the common path runs three iterations at a time from stage 0 on, every LDS address then being a lane constant
+                // plus an immediate; single iterations in front of and behind that
+                for (; it < end && (MODE != 2 || stage != 0 || it + PL_STAGES > end); ++it) {
+                    one(mode_tag, stage, stage == 0 ? 2 : stage - 1);
                     stage = stage == PL_STAGES - 1 ? 0 : stage + 1;
-                    PL_WAIT_TILE;
-                    PL_BARRIER;
+                }
+                if (MODE == 2) {
+                    for (; it + PL_STAGES <= end; it += PL_STAGES) {
+                        one(mode_tag, 0, 2);
+                        one(mode_tag, 1, 0);
+                        one(mode_tag, 2, 1);
+                    }
+                    for (; it < end; ++it) {
+                        one(mode_tag, stage, stage == 0 ? 2 : stage - 1);
+                        stage = stage == PL_STAGES - 1 ? 0 : stage + 1;
+                    }
                 }
             };
-            if (!SAFE) {
-                general_iters(it_f0);
-                for (; it < it_f1; ++it) {
-                    const uint8_t *const kt = pl_lds + PL_K_OFF + stage * PL_K_BYTES;
-                    const uint8_t *const vt_tile = pl_lds + PL_V_OFF + stage * PL_V_BYTES;
-                    const float *const ksp = (const float *)(pl_lds + PL_KS_OFF + stage * PL_KS_BYTES) + 4 * g;
-                    request_tile();
-                    fast_step(std::integral_constant<int, 0>{}, kt, ksp, vt_tile);
-                    fast_step(std::integral_constant<int, 1>{}, kt + 32 * 128, ksp + 32, vt_tile);
-                    stage = stage == PL_STAGES - 1 ? 0 : stage + 1;
-                    PL_WAIT_TILE;
-                    PL_BARRIER;
-                }
+            if (SAFE) {
+                iterations(std::integral_constant<int, 0>{}, n_tiles + 1);
+            } else {
+                iterations(std::integral_constant<int, 1>{}, it_f0);
+                iterations(std::integral_constant<int, 2>{}, it_f1);
+                iterations(std::integral_constant<int, 1>{}, it_last + 1);
+                iterations(std::integral_constant<int, 3>{}, n_tiles + 1);
             }
-            general_iters(n_tiles + 1);
             PL_WAIT_ALL; // nothing may still be on its way into LDS
         };
         run(std::false_type{});
