@@ -75,6 +75,7 @@ struct PrefillParams {
     // optional scratch of the long-range kernel (vt != nullptr selects it): room for V as f16, transposed
     void *vt;
     int64_t vt_pitch; // halves per (head, x) row
+    int64_t ks_pitch; // long-range kernel only: floats between the heads of ks (set by its launcher)
     WgMap map;        // set by the launcher: how workgroup ids map to (head, query tile)
 };
 

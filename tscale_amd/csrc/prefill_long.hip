@@ -43,14 +43,22 @@ constexpr int PL_LDS_BYTES = PL_SPARE_OFF + PL_KS_BYTES;
 // feed into one V^T.P^T instruction).  Columns that stand for no token are zero.  The column of a token is shifted by
 // VT_PAD = 32 so that the tile of V a loop iteration needs (the second sub-tile of one K tile and the first of the next)
 // starts at a multiple of 64 columns.
+//
+// With a constant query scale the same kernel also writes the key scales times that constant, the logit scale and the
+// optional global key scale (ksq[head][t], pitch ksq_pitch): the attention kernel then has one multiply per logit.
 template <int DTYPE>
 __global__ __launch_bounds__(256) void widen_v_kernel(const uint8_t *v, int64_t v_pitch, const float *vs, int64_t scale_pitch, float vs_const,
-                                                      int n_tokens, _Float16 *vt, int64_t vt_pitch)
+                                                      int n_tokens, _Float16 *vt, int64_t vt_pitch, const float *ks, float ks_mult,
+                                                      const float *k_global_scale, float *ksq, int64_t ksq_pitch)
 {
     constexpr int D = PL_D, PITCH = 64 + 8; // halves per LDS row: 16-byte aligned, rows 36 banks apart
     __shared__ __attribute__((aligned(16))) _Float16 tile[D * PITCH];
     const int tid = threadIdx.x, head = blockIdx.y;
     const int col0 = blockIdx.x * 64; // first column of this block; column c holds position c - VT_PAD
+    if (ksq && tid < 64 && col0 + tid < n_tokens) {
+        const float m = k_global_scale ? ks_mult * *k_global_scale : ks_mult;
+        ksq[(int64_t)head * ksq_pitch + col0 + tid] = ks[(int64_t)head * scale_pitch + col0 + tid] * m;
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int ch = tid + i * 256;   // 64 columns x 8 chunks of 16 bytes
@@ -90,7 +98,9 @@ __global__ __launch_bounds__(256) void widen_v_kernel(const uint8_t *v, int64_t 
 
 typedef __attribute__((address_space(3))) void *pl_lds_ptr;
 
-template <int DTYPE, int D, bool OUT_F16>
+// QS_CONST: the query scale is one number for all rows and has been multiplied into the key scales the kernel reads
+// (p.ks then points at the plane the first kernel wrote, or p.ks_const holds the product).
+template <int DTYPE, int D, bool OUT_F16, bool QS_CONST>
 __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillParams p, int n_qtiles)
 {
     static_assert(D == PL_D, "written for a head width of 128");
@@ -161,10 +171,12 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
         __syncthreads(); // red is used again at the end
     }
     // the logit scale goes into the query's scale: the key scales arrive in LDS as they are in memory
-    {
+    if (!QS_CONST) {
         float ads = att_dot_scale(D);
         if (p.k_global_scale) ads *= *p.k_global_scale;
         qs *= ads;
+    } else {
+        qs = 1.0f; // (rows past the end have zero operands)
     }
     w_min_a = __builtin_amdgcn_readfirstlane(w_min_a);
     w_max_a = __builtin_amdgcn_readfirstlane(w_max_a);
@@ -217,7 +229,7 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
         const int64_t vt_row_bytes = p.vt_pitch * 2;
         const __amdgpu_buffer_rsrc_t vr = rsrc((const uint8_t *)p.vt + (int64_t)head * D * vt_row_bytes + (int64_t)kb_first * 2, D * vt_row_bytes - (int64_t)kb_first * 2);
         const bool ks_plane = p.ks != nullptr;
-        const float *ks_ptr = ks_plane ? p.ks + (int64_t)head * p.scale_pitch + kb_first : nullptr;
+        const float *ks_ptr = ks_plane ? p.ks + (int64_t)head * p.ks_pitch + kb_first : nullptr;
         const __amdgpu_buffer_rsrc_t ksr = rsrc(ks_ptr, ks_plane ? (int64_t)(p.n_tokens - kb_first) * 4 : 0);
         if (!ks_plane && tid < PL_STAGES * PL_BN) ((float *)(pl_lds + PL_KS_OFF))[tid] = p.ks_const; // (the first barrier of the loop follows)
         // A request of one wave fills 1 KiB of LDS = 8 rows of 128 bytes: lane L writes position L % 8 of row L / 8,
@@ -318,8 +330,8 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
             const int r = 2 * pr;
             const v4f kq = ksv[pr >> 1];
             const float k0 = kq[2 * (pr & 1)], k1 = kq[2 * (pr & 1) + 1];
-            float p0 = fast_exp2((Qk::to_float(a, r) * k0) * qs);
-            float p1 = fast_exp2((Qk::to_float(a, r + 1) * k1) * qs);
+            float p0 = fast_exp2(QS_CONST ? Qk::to_float(a, r) * k0 : (Qk::to_float(a, r) * k0) * qs);
+            float p1 = fast_exp2(QS_CONST ? Qk::to_float(a, r + 1) * k1 : (Qk::to_float(a, r + 1) * k1) * qs);
             if (MASKED) {
                 const int off = 8 * (r >> 2) + (r & 3); // key of register r relative to the lane's first key
                 p0 = ((unsigned)(off - rel_lo) <= span_w) ? p0 : 0.0f;
@@ -584,19 +596,22 @@ __global__ __launch_bounds__(PF_THREADS, 2) void prefill_long_kernel(PrefillPara
     if (row_ok && p.sum_weight_log && g == 0) p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m_ref + __log2f(l_all);
 }
 
+// Bytes of scratch: the f16 copy of V, then (used with a constant query scale only) a plane of scaled key scales.
+static int64_t ksq_pitch_of(int64_t n_tokens) { return (n_tokens + 63) / 64 * 64; }
 size_t prefill_long_workspace_bytes(int64_t n_tokens, int n_heads, int head_dim)
 {
     if (head_dim != PL_D || n_tokens <= 0) return 0;
-    return (size_t)n_heads * PL_D * (size_t)prefill_long_vt_pitch(n_tokens) * 2;
+    return (size_t)n_heads * PL_D * (size_t)prefill_long_vt_pitch(n_tokens) * 2 + (size_t)n_heads * (size_t)ksq_pitch_of(n_tokens) * 4;
 }
 
-template <int DTYPE, bool OUT_F16>
+template <int DTYPE, bool OUT_F16, bool QS_CONST>
 static hipError_t launch_long_do(const PrefillParams &p_in, hipStream_t st)
 {
     PrefillParams p = p_in;
     const int n_qtiles = (int)((p.n_tokens + PF_BM - 1) / PF_BM);
+    p.ks_pitch = p.scale_pitch;
     p.map = wg_plan(n_qtiles, p.n_heads, PL_D, PF_BM, p.period_tiles, 3); // K as it is, V as f16
-    auto kernel = prefill_long_kernel<DTYPE, PL_D, OUT_F16>;
+    auto kernel = prefill_long_kernel<DTYPE, PL_D, OUT_F16, QS_CONST>;
     static bool attr_set = false; // (per instantiation; setting it again is harmless)
     if (!attr_set) {
         const hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, PL_LDS_BYTES);
@@ -604,7 +619,21 @@ static hipError_t launch_long_do(const PrefillParams &p_in, hipStream_t st)
         attr_set = true;
     }
     const dim3 wgrid((unsigned)(p.vt_pitch / 64), (unsigned)p.n_heads);
-    hipLaunchKernelGGL((widen_v_kernel<DTYPE>), wgrid, dim3(256), 0, st, p.v, p.v_pitch, p.vs, p.scale_pitch, p.vs_const, p.n_tokens, (_Float16 *)p.vt, p.vt_pitch);
+    float *ksq = nullptr;
+    const int64_t ksq_pitch = ksq_pitch_of(p.n_tokens);
+    const float ks_mult = p.qs_const * att_dot_scale(PL_D);
+    if (QS_CONST && p.ks) ksq = (float *)((uint8_t *)p.vt + (size_t)p.n_heads * PL_D * (size_t)p.vt_pitch * 2);
+    hipLaunchKernelGGL((widen_v_kernel<DTYPE>), wgrid, dim3(256), 0, st, p.v, p.v_pitch, p.vs, p.scale_pitch, p.vs_const, p.n_tokens, (_Float16 *)p.vt, p.vt_pitch,
+                       p.ks, ks_mult, p.k_global_scale, ksq, ksq_pitch);
+    if (QS_CONST) {
+        if (p.ks) {
+            p.ks = ksq;
+            p.ks_pitch = ksq_pitch;
+        } else {
+            if (p.k_global_scale) return hipErrorInvalidValue; // filtered out by launch_prefill_long: the product would need the device value
+            p.ks_const = p.ks_const * ks_mult;
+        }
+    }
     hipLaunchKernelGGL(kernel, dim3((unsigned)(n_qtiles * p.n_heads)), dim3(PF_THREADS), PL_LDS_BYTES, st, p, n_qtiles);
     return hipGetLastError();
 }
@@ -612,8 +641,15 @@ static hipError_t launch_long_do(const PrefillParams &p_in, hipStream_t st)
 hipError_t launch_prefill_long(const PrefillParams &p, int dtype, int out_dtype, hipStream_t st)
 {
     const bool f16 = out_dtype == TSATTN_OUT_F16;
-    if (dtype == TSATTN_E4M3) return f16 ? launch_long_do<TSATTN_E4M3, true>(p, st) : launch_long_do<TSATTN_E4M3, false>(p, st);
-    return f16 ? launch_long_do<TSATTN_I8, true>(p, st) : launch_long_do<TSATTN_I8, false>(p, st);
+    // one multiply per logit where the query scale is a constant (and, with a constant key scale too, no device value
+    // would be needed on the host to form the product)
+    const bool qs_const = p.qs == nullptr && !(p.ks == nullptr && p.k_global_scale != nullptr);
+    if (dtype == TSATTN_E4M3) {
+        if (qs_const) return f16 ? launch_long_do<TSATTN_E4M3, true, true>(p, st) : launch_long_do<TSATTN_E4M3, false, true>(p, st);
+        return f16 ? launch_long_do<TSATTN_E4M3, true, false>(p, st) : launch_long_do<TSATTN_E4M3, false, false>(p, st);
+    }
+    if (qs_const) return f16 ? launch_long_do<TSATTN_I8, true, true>(p, st) : launch_long_do<TSATTN_I8, false, true>(p, st);
+    return f16 ? launch_long_do<TSATTN_I8, true, false>(p, st) : launch_long_do<TSATTN_I8, false, false>(p, st);
 }
 
 } // namespace tsattn
