@@ -147,8 +147,10 @@ class PrefillWorkload:
         W, slope = self.layers[i]
         st, fi = self.spans[W]
         # equal-length sequences: tell the library the causal period of the wide layers (a launch-order hint)
+        # (and the layer's attention width: with long spans the library takes its workspace kernel)
         self.ctx.compute_val_lookup(self.dtype, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
-                                    causal_period=self.S if W >= self.S else 0, span_tiles=self.span_tiles[W])
+                                    causal_period=self.S if W >= self.S else 0, span_tiles=self.span_tiles[W],
+                                    span_len_hint=min(W, self.S))
 
     def step(self):
         for i in range(len(self.layers)):
@@ -220,7 +222,8 @@ class GenerationWorkload:
         W, slope = self.sched[i]
         st, fi = self.spans[W]
         self.ctx.compute_val_lookup(self.i8, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
-                                    causal_period=self.prompt if W >= self.prompt else 0, span_tiles=self.span_tiles[W])
+                                    causal_period=self.prompt if W >= self.prompt else 0, span_tiles=self.span_tiles[W],
+                                    span_len_hint=min(W, self.prompt))
 
     def fill_caches(self):
         (_, _), (k, ks), (v, vs) = self.qkv

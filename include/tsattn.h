@@ -74,6 +74,7 @@ const char *tsattn_last_error(void);
  * (gpt_cuda.cu:501) is needed.
  */
 #define TSATTN_PREFILL_MAX_KV_PITCH ((int64_t)8 << 20)
+#define TSATTN_PREFILL_LONG_SPAN 6144   /* span_len_hint from which a workspace is used: measured equal to the standard kernel at 4096 keys per row, 7-10 % faster from 8192 on */
 typedef struct tsattn_prefill_args {
     int dtype;                 /* tsattn_dtype of q, k, v */
     int out_dtype;             /* tsattn_out_dtype */
@@ -118,7 +119,8 @@ typedef struct tsattn_prefill_args {
     int kv_rep;                /* 1..4 */
     float kv_mult;
     /* Optional scratch for rows with long spans (NULL = none).  With at least tsattn_prefill_workspace_bytes(n_tokens,
-     * n_heads, head_dim) bytes here (16-byte aligned) and span_len_hint >= 512, head_dim 128 and no ALiBi slope, the
+     * n_heads, head_dim) bytes here (16-byte aligned) and span_len_hint >= TSATTN_PREFILL_LONG_SPAN, head_dim 128 and no
+     * ALiBi slope (nor debug_qk_acc, nor the fused KVProduct), the
      * call first writes V once as f16 with the value scales folded in, transposed, into the workspace, and the attention
      * kernel streams K and that copy through LDS without touching them in registers (the reference keeps such a
      * transposed copy of V too: Transpose, gpt_cuda.cu:501, VT of TAttentionComputeCtx).  Same result within the

@@ -25,7 +25,7 @@ def t(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def run_long(ctx, dtype, H, q, qs, k, ks, v, vs, st, fi, out_f16=False, want_swl=False, hint=4096, **kw):
+def run_long(ctx, dtype, H, q, qs, k, ks, v, vs, st, fi, out_f16=False, want_swl=False, hint=8192, **kw):
     sc = lambda s: t(s) if isinstance(s, np.ndarray) else s
     n = q.shape[0]
     swl = torch.zeros((H, n), dtype=torch.float32, device="cuda") if want_swl else None
@@ -48,7 +48,7 @@ def test_workspace_size_and_selection(ctx):
     assert ctx._workspace is None
     b = run_long(ctx, capi.E4M3, 2, q, qs, k, ks, v, vs, st, fi, hint=300)   # below the threshold: the standard kernel
     assert np.array_equal(a, b)
-    c = run_long(ctx, capi.E4M3, 2, q, qs, k, ks, v, vs, st, fi, hint=4096)
+    c = run_long(ctx, capi.E4M3, 2, q, qs, k, ks, v, vs, st, fi, hint=8192)
     assert ctx._workspace is not None and np.abs(c - a).max() < 5e-3
 
 
@@ -135,7 +135,7 @@ def test_long_full_size_properties(ctx):
     st = (torch.arange(n, device="cuda", dtype=torch.int32) // S) * S
     fi = torch.arange(n, device="cuda", dtype=torch.int32) - 1
     swl = torch.zeros((H, n), dtype=torch.float32, device="cuda")
-    out = ctx.compute_val_lookup(capi.E4M3, H, q, k, v, qs, ks, 1.0, st, fi, 0.0, sum_weight_log=swl, causal_period=S, span_len_hint=S)
+    out = ctx.compute_val_lookup(capi.E4M3, H, q, k, v, qs, ks, 1.0, st, fi, 0.0, sum_weight_log=swl, causal_period=S, span_len_hint=2 * S)
     base = ctx.compute_val_lookup(capi.E4M3, H, q, k, v, qs, ks, 1.0, st, fi, 0.0, causal_period=S)
     torch.cuda.synchronize()
     want = (1.0 - torch.exp2(-swl)).t()                     # [n, H]

@@ -286,7 +286,7 @@ class AttentionContext:
         launch (k uint8 [n_tokens, H*d], kv_out uint8 [n_tokens, H*rep*d]); with want_out=False the result itself is
         not written and None is returned.
         span_len_hint: typical number of keys per row (the layer's attention width clipped to the sequence length); from
-        512 on, with head width 128 and no slope, the call goes through the long-span kernel, which needs a workspace
+        capi.PREFILL_LONG_SPAN on, with head width 128 and no slope, the call goes through the long-span kernel, which needs a workspace
         (uint8 tensor; by default one that this context keeps and grows on demand)."""
         n_tokens, hd = q.shape
         d = hd // n_heads
@@ -322,7 +322,7 @@ class AttentionContext:
         a.causal_period = int(causal_period)
         a.span_tiles = _ptr(span_tiles)
         a.span_len_hint = int(span_len_hint)
-        if span_len_hint >= 512:
+        if span_len_hint >= capi.PREFILL_LONG_SPAN:
             need = int(self.lib.tsattn_prefill_workspace_bytes(n_tokens, n_heads, d))
             if workspace is None and need > 0:
                 if self._workspace is None or self._workspace.numel() < need or self._workspace.device != q.device:

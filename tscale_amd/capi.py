@@ -16,6 +16,7 @@ SRC_F32, SRC_BF16, SRC_I32 = 0, 1, 2
 MM_I32, MM_F32, MM_ADD_SCALED, MM_I32_PLANES = 0, 1, 2, 3
 Q_8BIT, Q_BF16 = 0, 1
 SPAN_TILE_INTS = 32
+PREFILL_LONG_SPAN = 6144   # TSATTN_PREFILL_LONG_SPAN: span_len_hint from which tsattn_prefill uses a workspace
 
 STATUS_NAMES = {0: "OK", 1: "BAD_ARG", 2: "UNSUPPORTED", 3: "HIP", 4: "SCRATCH"}
 

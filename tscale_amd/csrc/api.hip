@@ -272,7 +272,7 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     p.period_tiles = (a->causal_period > 0 && a->causal_period % 128 == 0 && a->n_tokens % a->causal_period == 0) ? (int)(a->causal_period / 128) : 0;
     // Long spans with room for the f16 copy of V: the kernel that streams K and that copy through LDS.  (It addresses
     // K and the copy with 31-bit byte offsets.)
-    if (a->workspace && a->span_len_hint >= 512 && a->head_dim == 128 && a->alibi_slope == 0.0f && !a->debug_qk_acc && !a->kv_out) {
+    if (a->workspace && a->span_len_hint >= TSATTN_PREFILL_LONG_SPAN && a->head_dim == 128 && a->alibi_slope == 0.0f && !a->debug_qk_acc && !a->kv_out) {
         const size_t need = tsattn::prefill_long_workspace_bytes(a->n_tokens, a->n_heads, a->head_dim);
         const int64_t vt_pitch = tsattn::prefill_long_vt_pitch(a->n_tokens);
         if (!aligned16(a->workspace)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: workspace must be 16-byte aligned");
