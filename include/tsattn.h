@@ -130,6 +130,14 @@ typedef struct tsattn_prefill_args {
     void *workspace;
     int64_t workspace_bytes;
     int64_t span_len_hint;
+    /* Rows with several spans (TAttentionInfo allows any number per row, gpt/att/att.h:24-47; the reference's kernels walk
+     * a list of key ranges per query block, att.h:95-181): n_span_parts > 1 says that span_start and span_finish hold that
+     * many arrays of n_tokens entries, span_part_stride entries apart -- part i is every row's i-th span, finish < start
+     * where a row has fewer -- and span_tiles (if given) one summary after the other, tsattn_span_tiles_count(n_tokens)
+     * entries each.  One launch, one softmax over all keys of all of a row's spans, a key that lies in c of them counted c
+     * times, as the CPU loop over the spans counts it (gpt_cpu.cpp:405-436).  0 or 1: one span per row.  At most 64. */
+    int n_span_parts;
+    int64_t span_part_stride;
 } tsattn_prefill_args;
 
 int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream);
@@ -444,10 +452,6 @@ int tsattn_quantize_rows(tsattn_handle_t h, int src_dtype, int dst_dtype, const 
 int tsattn_build_spans(tsattn_handle_t h, int n_seqs, const int32_t *seq_offset, int64_t n_tokens,
                        const uint8_t *doc_start_flag, int64_t window, int32_t *span_start,
                        int32_t *span_finish, void *stream);
-
-/* Diagnostic: copies the handle's per-sequence arrival counters (used by the single-split fused append of tsattn_decode;
- * every launch leaves them at zero) into dst, a device array of n int32, on the stream.  For tests of graph replays. */
-int tsattn_debug_read_counters(tsattn_handle_t h, int32_t *dst, int n, void *stream);
 
 /* Library build identification (kernel set and target), for logs. */
 const char *tsattn_version(void);

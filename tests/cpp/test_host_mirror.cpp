@@ -14,6 +14,7 @@
 
 #include "../../oracle/tsattn_oracle.h"
 #include "../../tscale_amd/host/att_compute.h"
+#include "../../tscale_amd/host/model_init.h"
 
 using namespace NTsAttn;
 
@@ -324,6 +325,22 @@ struct TLayerData {
         Att.QVScale = L.qv_scale; Att.CombinerScale = L.combiner_scale; Att.ContractScale = L.contract_scale;
         Att.AttentionWidth = width; Att.AlibiSlope = slope;
     }
+    // the same from a layer NTsAttn::InitModel made (its matrix sizes are what is under test), with the test's own mask
+    TLayerData(const TModelDims &dims, int width, float slope, const NTsAttn::THostAttention &h)
+    {
+        QK = h.QK; QV = h.QV; K = h.K; V = h.V; Comb = h.Combiner; Expand = h.Expand; Contract = h.Contract;
+        L.dim = dims.Dim; L.head_count = dims.HeadCount; L.head_dim = dims.QDim; L.relu_dim = dims.GetReluDim();
+        L.qk = QK.data(); L.qv = QV.data(); L.k = K.data(); L.v = V.data(); L.combiner = Comb.data(); L.expand = Expand.data(); L.contract = Contract.data();
+        L.qv_scale = h.QVScale; L.combiner_scale = h.CombinerScale; L.contract_scale = h.ContractScale;
+        L.attention_width = width; L.alibi_slope = slope;
+        std::vector<int8_t> all;
+        for (const auto *m : {&QK, &QV, &K, &V}) all.insert(all.end(), m->begin(), m->end());
+        Proj = ToDevice(all);
+        Att.QK = Proj; Att.QV = Proj + QK.size(); Att.K = Proj + 2 * QK.size(); Att.V = Proj + 3 * QK.size();
+        Att.Combiner = ToDevice(Comb); Att.Expand = ToDevice(Expand); Att.Contract = ToDevice(Contract);
+        Att.QVScale = L.qv_scale; Att.CombinerScale = L.combiner_scale; Att.ContractScale = L.contract_scale;
+        Att.AttentionWidth = width; Att.AlibiSlope = slope;
+    }
     ~TLayerData()
     {
         (void)hipFree(Proj);
@@ -583,14 +600,21 @@ static int RunPredictionCase()
 // TNodesBatch::AddSample (one span list per attention width, some nodes with two embedding labels), Init, then
 // ComputeFragmentPredictions / ComputeScore / ComputeFinalStateVectors against the oracle's token-by-token pass of the
 // same three layers (each fragment on its own cache rows; a node's position is its index in the batch).
-static int RunContextCase(int firstLayer, int nLayers)
+// fromInitModel: the layers' matrices come from NTsAttn::InitModel (head width and feed-forward multiplier as given:
+// its matrices must have the sizes the layer reads).
+static int RunContextCase(int firstLayer, int nLayers, int headDim = 128, int reluMult = 1, bool fromInitModel = false)
 {
-    const int B = 2, H = 2, d = 128, dim = 256, vocab = 512, maxLen = 64;
+    const int B = 2, H = 2, d = headDim, dim = 256, vocab = 512, maxLen = 64;
     const int fragLen[B] = {24, 40};
     const int len = fragLen[0] + fragLen[1];
     TModelDims dims;
-    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim;
+    dims.HeadCount = H; dims.QDim = d; dims.TTDim = d; dims.Dim = dim; dims.ReluMult = reluMult;
     unsigned seed = 20252u;
+    NTsAttn::THostModel hostModel;
+    if (fromInitModel) {
+        NTsAttn::InitModel(&hostModel, 777, dim, H, d, reluMult, 4, 1000, vocab, vocab, NTsAttn::COMBINER_INIT_RANDOM);
+        if (hostModel.ReluDim != dims.GetReluDim() || (int)hostModel.LayerArr.size() < 3) { printf("InitModel: ReluDim %d, layers %d\n", hostModel.ReluDim, (int)hostModel.LayerArr.size()); return 1; }
+    }
     tsattn_config cfg = {};
     cfg.device = 0; cfg.max_seqs = B; cfg.max_heads = H; cfg.max_head_dim = d;
     tsattn_handle_t handle = nullptr;
@@ -604,7 +628,8 @@ static int RunContextCase(int firstLayer, int nLayers)
         TInferModel model;
         std::vector<int> widthId;
         for (int l = firstLayer; l < firstLayer + nLayers; ++l) {
-            layers.emplace_back(new TLayerData(dims, widths[l], slopes[l], seed));
+            if (fromInitModel) layers.emplace_back(new TLayerData(dims, widths[l], slopes[l], hostModel.LayerArr[l]));
+            else layers.emplace_back(new TLayerData(dims, widths[l], slopes[l], seed));
             cpuCaches.emplace_back(B, H, maxLen, d);
             model.LayerArr.push_back(layers.back()->Att);
             widthId.push_back(l);
@@ -820,6 +845,7 @@ int main()
     fails += RunSeveralSpansCase(TSATTN_E4M3, 0.25f, true);
     for (int l = 0; l < 3; ++l) fails += RunContextCase(l, 1);
     fails += RunContextCase(0, 3);
+    fails += RunContextCase(0, 3, 64, 2, true);   // a model from InitModel: head width 64, feed-forward groups of 256
     fails += RunPromptLayerCase(1000, 0.0f, 128);
     fails += RunPromptLayerCase(64, 0.5f, 128);
     fails += RunPromptLayerCase(1, 0.0f, 64);

@@ -11,6 +11,7 @@ from tscale_amd import capi
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "tsattn.h")
+TEST_HOOKS = os.path.join(ROOT, "include", "tsattn_test_hooks.h")   # entry points for the library's own tests
 
 STRUCTS = {
     "tsattn_config": capi.Config,
@@ -25,7 +26,7 @@ STRUCTS = {
 
 
 def declared_functions():
-    text = open(HEADER).read()
+    text = open(HEADER).read() + open(TEST_HOOKS).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tsattn_[a-z_0-9]+)\s*\(", text)))
 

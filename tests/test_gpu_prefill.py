@@ -508,9 +508,10 @@ def test_prefill_largest_key_row_pitch(ctx, dtype, d, H, n, window, slope):
     (capi.I8, 64, 1, 200, 5, 0.5, False),
 ])
 def test_prefill_rows_with_several_spans(ctx, dtype, d, H, n, max_spans, slope, out_f16):
-    """Rows with any number of spans (TAttentionInfo, gpt/att/att.h:24-47): one tsattn_prefill per span of the rows and
-    tsattn_merge_lookups, against the oracle's loop over a row's spans inside one softmax (gpt_cpu.cpp:405-436) on the
-    dequantised operands.  Spans overlap (a key in two spans counts twice), some rows have none."""
+    """Rows with any number of spans (TAttentionInfo, gpt/att/att.h:24-47): one tsattn_prefill launch that walks the parts
+    (n_span_parts), and the fallback of one launch per span of the rows plus tsattn_merge_lookups, both against the
+    oracle's loop over a row's spans inside one softmax (gpt_cpu.cpp:405-436) on the dequantised operands, and against
+    each other within 1e-6 of the output's scale.  Spans overlap (a key in two spans counts twice), some rows have none."""
     from tests.test_oracle_attention import random_span_lists
     rng = np.random.default_rng(100 * d + n)
     q, qs, k, ks, v, vs = make_qkv(5 * d + n, n, H, d, dtype)
@@ -531,6 +532,21 @@ def test_prefill_rows_with_several_spans(ctx, dtype, d, H, n, max_spans, slope, 
     assert none.any() and not out[torch.from_numpy(none).cuda()].any()
     # sum_weight_log = max logit + log2(sum of the shifted weights, zero vector included)
     assert np.abs(swl.cpu().numpy() - (mx + np.log2(sw))).max() < 2e-3
+    # the fallback: a launch per part and the merge
+    swl2 = torch.zeros((H, n), dtype=torch.float32, device="cuda")
+    out2 = ctx.compute_val_lookup_multi(dtype, H, t(q), t(k), t(v), t(qs), t(ks), t(vs), ptr, spans, slope,
+                                        out_f16=out_f16, sum_weight_log=swl2, merge=True)
+    torch.cuda.synchronize()
+    assert_within_tolerance(out2.float().cpu().numpy(), want, "several spans per row, merged launches")
+    if not out_f16:
+        # The same sums in another order (the merge adds the parts' f32 results; the single launch keeps one accumulator):
+        # equal to f32 rounding while no logit is far above the zero vector's.  Where one is (a span of keys behind the
+        # row under a slope), the two raise the reference maximum at different moments and round their f16 weights against
+        # different references.
+        diff = (out - out2).abs().max().item()
+        print(f"single launch vs merged launches: max abs difference {diff:.2e} (largest logit {mx.max():.1f})")
+        assert diff <= (2e-6 if mx.max() <= 8.0 else 1e-3) * max(1.0, float(np.abs(want).max()))
+    assert (swl - swl2).abs().max().item() < 2e-3
 
 
 def test_merge_lookups_argument_checks(ctx):

@@ -76,3 +76,23 @@ def test_init_matrix_normal():
     assert q.shape == (3, 64, 128) and not np.array_equal(q[0], q[1]) and np.all(np.abs(s - 0.5 / 32) < 2e-3)
     qz, sz = mi.random_int8_matrices(9, 2, 8, 16, sko=0.0)              # COMBINER_INIT_ZERO
     assert not qz.any() and not sz.any()
+
+
+@pytest.mark.parametrize("dim,heads,head_dim,relu_mult", [(2048, 16, 128, 1), (768, 12, 64, 1), (512, 4, 128, 2), (256, 2, 64, 3)])
+def test_init_model_matrix_sizes(dim, heads, head_dim, relu_mult):
+    """The matrices NTsAttn::InitModel makes have the sizes the layer (TLayerComputer, and the reference's AddLookupProduct)
+    reads: the feed-forward block is HeadCount * 128 * ReluMult wide whatever the head width (model_dim.h:66)."""
+    s = mi.init_model_shapes(dim, heads, head_dim, relu_mult)
+    q_sum, relu = heads * head_dim, heads * 128 * relu_mult
+    assert s["QK"] == s["QV"] == s["K"] == s["V"] == (q_sum, dim)
+    assert s["Combiner"] == (dim, q_sum * 4)
+    assert s["Expand"] == (relu, dim) and s["Contract"] == (dim, relu)
+
+
+def test_init_alibi_respects_the_capacity():
+    lib = mi.load()
+    assert lib.tshost_init_alibi(mi.ALIBI_V3, 5, 100, None, None, 0) == 6      # an odd depth gains a layer
+    w = np.full(8, -7, dtype=np.int32)
+    s = np.full(8, -7.0, dtype=np.float32)
+    assert lib.tshost_init_alibi(mi.ALIBI_V3, 5, 100, w.ctypes.data, s.ctypes.data, 4) == 6
+    assert (w[4:] == -7).all() and (s[4:] == -7.0).all() and (w[:4] != -7).all()

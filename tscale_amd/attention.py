@@ -307,6 +307,10 @@ class AttentionContext:
         a.scale_pitch = pitches[0] if pitches else n_tokens
         a.k_global_scale = _ptr(k_global_scale)
         a.span_start, a.span_finish = _ptr(span_start), _ptr(span_finish)
+        if span_start.dim() == 2:      # rows with several spans: [n_parts, n_tokens], part i = every row's i-th span
+            assert span_finish.shape == span_start.shape and span_start.stride(1) == 1 and span_finish.stride() == span_start.stride()
+            a.n_span_parts, a.span_part_stride = span_start.shape[0], span_start.stride(0)
+            assert span_tiles is None or (span_tiles.is_contiguous() and span_tiles.shape[0] == span_start.shape[0])
         a.alibi_slope = float(alibi_slope)
         if out is not None:
             a.out, a.out_pitch = _ptr(out), out.stride(0) * out.element_size()
@@ -353,10 +357,11 @@ class AttentionContext:
         return out
 
     def compute_val_lookup_multi(self, dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, span_ptr, spans, alibi_slope,
-                                 out_f16=False, sum_weight_log=None):
+                                 out_f16=False, sum_weight_log=None, merge=False):
         """Rows with any number of spans, as TAttentionInfo holds them (gpt/att/att.h:24-47): span_ptr int [n_tokens+1],
-        spans int [n_spans, 2] (inclusive start, finish), both on the host.  One prefill launch per span of the rows
-        (part i takes every row's i-th span) and one launch that combines them."""
+        spans int [n_spans, 2] (inclusive start, finish), both on the host.  Part i takes every row's i-th span; one
+        launch walks all parts (n_span_parts of tsattn_prefill_args), or with merge=True one launch per part and one that
+        combines them (tsattn_merge_lookups)."""
         n_tokens = q.shape[0]
         span_ptr = np.asarray(span_ptr, dtype=np.int64)
         spans = np.asarray(spans, dtype=np.int32).reshape(-1, 2)
@@ -369,6 +374,9 @@ class AttentionContext:
             st[i, rows] = spans[span_ptr[rows] + i, 0]
             fi[i, rows] = spans[span_ptr[rows] + i, 1]
         st_d, fi_d = torch.from_numpy(st).to(q.device), torch.from_numpy(fi).to(q.device)
+        if not merge:
+            return self.compute_val_lookup(dtype, n_heads, q, k, v, q_scale, k_scale, v_scale, st_d, fi_d, alibi_slope,
+                                           out_f16=out_f16, sum_weight_log=sum_weight_log)
         part_out = torch.empty((n_parts, n_tokens, q.shape[1]), dtype=torch.float32, device=q.device)
         part_swl = torch.empty((n_parts, n_heads, n_tokens), dtype=torch.float32, device=q.device)
         for i in range(n_parts):

@@ -46,6 +46,7 @@ class PrefillArgs(_c.Structure):
         ("kv_k", _c.c_void_p), ("kv_k_pitch", _c.c_int64), ("kv_out", _c.c_void_p), ("kv_out_pitch", _c.c_int64),
         ("kv_rep", _c.c_int), ("kv_mult", _c.c_float),
         ("workspace", _c.c_void_p), ("workspace_bytes", _c.c_int64), ("span_len_hint", _c.c_int64),
+        ("n_span_parts", _c.c_int), ("span_part_stride", _c.c_int64),
     ]
 
 

@@ -9,6 +9,7 @@
 #include <mutex>
 
 #include "../../include/tsattn.h"
+#include "../../include/tsattn_test_hooks.h"
 #include "kernels.hpp"
 
 struct tsattn_ctx {
@@ -240,6 +241,8 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
         return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: scale_pitch %lld < n_tokens", (long long)a->scale_pitch);
     if (a->debug_qk_acc && a->debug_pitch < a->n_tokens) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: debug_pitch < n_tokens");
 
+    if (a->n_span_parts > 1 && (a->n_span_parts > 64 || a->span_part_stride < a->n_tokens))
+        return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: n_span_parts %d (at most 64) with span_part_stride %lld (at least n_tokens)", a->n_span_parts, (long long)a->span_part_stride);
     if (a->kv_out) {
         if (!a->kv_k) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: the fused KVProduct needs kv_k");
         if (a->out_dtype != TSATTN_OUT_F32 || a->dtype != TSATTN_I8)
@@ -264,6 +267,8 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     p.k_global_scale = a->k_global_scale;
     p.span_start = a->span_start; p.span_finish = a->span_finish;
     p.span_tiles = a->span_tiles;
+    p.n_parts = a->n_span_parts > 1 ? a->n_span_parts : 1;
+    p.span_part_stride = p.n_parts > 1 ? a->span_part_stride : 0;
     p.slope = a->alibi_slope;
     p.out = a->out; p.out_pitch = a->out_pitch;
     p.sum_weight_log = a->sum_weight_log;
@@ -272,7 +277,7 @@ int tsattn_prefill(tsattn_handle_t h, const tsattn_prefill_args *a, void *stream
     p.period_tiles = (a->causal_period > 0 && a->causal_period % 128 == 0 && a->n_tokens % a->causal_period == 0) ? (int)(a->causal_period / 128) : 0;
     // Long spans with room for the f16 copy of V: the kernel that streams K and that copy through LDS.  (It addresses
     // K and the copy with 31-bit byte offsets.)
-    if (a->workspace && a->span_len_hint >= TSATTN_PREFILL_LONG_SPAN && a->head_dim == 128 && a->alibi_slope == 0.0f && !a->debug_qk_acc && !a->kv_out) {
+    if (a->workspace && a->span_len_hint >= TSATTN_PREFILL_LONG_SPAN && a->head_dim == 128 && a->alibi_slope == 0.0f && !a->debug_qk_acc && !a->kv_out && a->n_span_parts <= 1) {
         const size_t need = tsattn::prefill_long_workspace_bytes(a->n_tokens, a->n_heads, a->head_dim);
         const int64_t vt_pitch = tsattn::prefill_long_vt_pitch(a->n_tokens);
         if (!aligned16(a->workspace)) return fail(TSATTN_ERR_BAD_ARG, "tsattn_prefill: workspace must be 16-byte aligned");

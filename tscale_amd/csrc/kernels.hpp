@@ -54,8 +54,10 @@ struct PrefillParams {
     int64_t scale_pitch;
     float qs_const, ks_const, vs_const;
     const float *k_global_scale;
-    const int32_t *span_start, *span_finish;
-    const int32_t *span_tiles; // optional per-128-row summary (SPAN_TILE_* layout below)
+    const int32_t *span_start, *span_finish; // n_parts arrays, span_part_stride entries apart (part i: every row's i-th span)
+    const int32_t *span_tiles; // optional per-128-row summary (SPAN_TILE_* layout below), one after the other for the parts
+    int n_parts;
+    int64_t span_part_stride;
     float slope;
     void *out;
     int64_t out_pitch;

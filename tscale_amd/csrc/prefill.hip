@@ -80,8 +80,9 @@ __device__ inline void widen_v_word(int w, v2h vs2, v2h &h0, v2h &h1)
 
 typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
 
-template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP>
-__global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : 2) void prefill_kernel(PrefillParams p, int n_qtiles)
+// MULTI: rows may have several spans (p.n_parts arrays of them); otherwise the one-span kernel, which needs fewer registers.
+template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP, bool MULTI>
+__global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefill_kernel(PrefillParams p, int n_qtiles)
 {
     typedef PfLayout<D> L;
     typedef QkMma<DTYPE, D> Qk;
@@ -132,17 +133,40 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : 2) void prefill_kernel(Pr
     const bool row_ok = from < p.n_tokens;
     const int64_t hoff = (int64_t)head * D;
 
+    // ---- query operand and per-row constants -----------------------------------------------------------------
+    Qk qk;
+    if (row_ok) qk.load_q(p.q + (int64_t)from * p.q_pitch + hoff, g);
+    else qk.clear_q();
+    const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
+
+    float ads = att_dot_scale(D);
+    if (p.k_global_scale) ads *= *p.k_global_scale;
+
+    v16f o_acc[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o_acc[i] = v16f{0};
+    float m_ref = 0.0f; // reference maximum: starts at the zero vector's logit
+    float l = 0.0f, l2 = 0.0f; // this lane's share of the weight sum (its 32 of every 64 keys), in two chains
+
+    // Rows with several spans (TAttentionInfo allows them, gpt/att/att.h:24-47; the reference's kernel walks a list of
+    // key ranges per query block, att.h:95-181, gpt_att_fp8.cuh:103-112): part i of the span arrays holds every row's
+    // i-th span (an empty one where a row has fewer), and the parts are walked one after the other into the same
+    // accumulators -- one softmax over all keys of all spans, a key in c spans counted c times, as the CPU loop over
+    // the spans does (gpt_cpu.cpp:405-436).
+    const int n_parts = MULTI ? p.n_parts : 1;
+    for (int part = 0; part < n_parts; ++part) {
+    const int32_t *const part_start = p.span_start + (int64_t)part * p.span_part_stride;
+    const int32_t *const part_finish = p.span_finish + (int64_t)part * p.span_part_stride;
     // ---- spans --------------------------------------------------------------------------------
     // What the loop needs to know about the spans: the workgroup's key range and the extremes of this wave's 32
-    // spans.  Either read from the caller's summary (scalar loads issued first of all, so K and V can be requested
-    // as soon as they return, without waiting for the per-row spans) or reduced below from the rows' spans
-    // (shuffles, LDS, a barrier).
+    // spans.  Either read from the caller's summary (scalar loads, so K and V can be requested as soon as they
+    // return, without waiting for the per-row spans) or reduced below from the rows' spans (shuffles, LDS, a barrier).
     bool w_all_have_keys = false;
     int w_min_a = 0, w_max_a = 0, w_min_b = 0, w_max_b = 0, b_min_a = 0, b_max_b = 0;
     const bool have_summary = p.span_tiles != nullptr;
     if (have_summary) {
         typedef __attribute__((address_space(4))) const int32_t *const_i32_ptr;
-        const const_i32_ptr t = (const_i32_ptr)(p.span_tiles + (int64_t)tile * SPAN_TILE_INTS);
+        const const_i32_ptr t = (const_i32_ptr)(p.span_tiles + ((int64_t)part * n_qtiles + tile) * SPAN_TILE_INTS);
         const const_i32_ptr w = t + SPAN_TILE_WAVE0 + __builtin_amdgcn_readfirstlane(wave) * SPAN_TILE_WAVE_INTS;
         b_min_a = t[SPAN_TILE_MIN_A];
         b_max_b = t[SPAN_TILE_MAX_B];
@@ -154,14 +178,9 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : 2) void prefill_kernel(Pr
     }
     int sp_a = 1, sp_b = 0;
     if (row_ok) {
-        sp_a = p.span_start[from];
-        sp_b = p.span_finish[from];
+        sp_a = part_start[from];
+        sp_b = part_finish[from];
     }
-    // ---- query operand and per-row constants (issued before anything waits for the spans) -------------------
-    Qk qk;
-    if (row_ok) qk.load_q(p.q + (int64_t)from * p.q_pitch + hoff, g);
-    else qk.clear_q();
-    const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
     if (!have_summary) {
         const bool hk = sp_b >= sp_a;
         w_all_have_keys = __all(hk);
@@ -184,15 +203,6 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : 2) void prefill_kernel(Pr
             b_max_b = max(b_max_b, red_lds[PF_WAVES + w]);
         }
     }
-
-    float ads = att_dot_scale(D);
-    if (p.k_global_scale) ads *= *p.k_global_scale;
-
-    v16f o_acc[DT];
-#pragma unroll
-    for (int i = 0; i < DT; ++i) o_acc[i] = v16f{0};
-    float m_ref = 0.0f; // reference maximum: starts at the zero vector's logit
-    float l = 0.0f, l2 = 0.0f; // this lane's share of the weight sum (its 32 of every 64 keys), in two chains
 
     if (b_max_b >= b_min_a) {
         // the same in every lane; said explicitly so that everything derived from them stays in scalar registers
@@ -698,6 +708,8 @@ __global__ __launch_bounds__(PF_THREADS, D == 64 ? 3 : 2) void prefill_kernel(Pr
         }
         } // tile loop
     }
+    if (MULTI && part + 1 < n_parts) __syncthreads(); // the next part stages its tiles into the same LDS (and reduces into red_lds)
+    } // parts
 
     // ---- epilogue: add the zero vector's weight, normalise, store -----------------------------------
     l += l2;
@@ -849,13 +861,17 @@ static void launch_prefill_do(const PrefillParams &p_in, dim3 grid2, hipStream_t
     const bool dump = p.dbg != nullptr;
     const bool slope = p.slope != 0.0f;
     dim3 block(PF_THREADS);
+    const bool multi = p.n_parts > 1;
     if (dump) {
         // the debug variant always takes the general (slope) path
-        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, true>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, false>), grid, block, 0, st, p, n_qtiles);
     } else if (slope) {
-        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, true>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false>), grid, block, 0, st, p, n_qtiles);
     } else {
-        hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, true>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false>), grid, block, 0, st, p, n_qtiles);
     }
 }
 

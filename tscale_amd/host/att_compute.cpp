@@ -67,6 +67,9 @@ TAttentionComputer::TAttentionComputer(const TModelDims &dims, float alibiSlope,
     cfg.max_head_dim = dims.QDim;
     Check(tsattn_create(&cfg, &Handle), "tsattn_create");
     CheckHip(hipMalloc((void **)&SumWeightLog, sizeof(float) * (size_t)maxLen * dims.HeadCount), "hipMalloc(sumWeightLog)");
+    // room for the long-span kernel's copy of V where a batch can have such spans at all
+    WorkspaceBytes = maxLen >= TSATTN_PREFILL_LONG_SPAN ? tsattn_prefill_workspace_bytes(maxLen, dims.HeadCount, dims.QDim) : 0;
+    if (WorkspaceBytes) CheckHip(hipMalloc(&Workspace, WorkspaceBytes), "hipMalloc(prefill workspace)");
     Reserve(1);
 }
 
@@ -97,6 +100,7 @@ TAttentionComputer::~TAttentionComputer()
     (void)hipFree(SumWeightLog);
     (void)hipFree(PartOut);
     (void)hipFree(PartSwl);
+    (void)hipFree(Workspace);
     tsattn_destroy(Handle);
 }
 
@@ -112,16 +116,20 @@ void TAttentionComputer::SetAttention(const TAttentionInfo &attInfo, void *strea
     Parts = parts;
     Len = len;
     const int64_t tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(MaxLen);
-    std::vector<int32_t> st, fi;
+    // every part's host arrays live until the copies have been waited for below
+    std::vector<std::vector<int32_t>> st(parts), fi(parts);
+    int64_t keys = 0;
     for (int i = 0; i < parts; ++i) {
-        const int period = FlattenSpans(attInfo, &st, &fi, i, false); // (and the launch-order hint)
+        const int period = FlattenSpans(attInfo, &st[i], &fi[i], i, false); // (and the launch-order hint)
         CausalPeriod = parts == 1 ? period : 0;
-        // pageable source: the copy has returned from the host's point of view when the call returns
-        CheckHip(hipMemcpyAsync(SpanStart + (size_t)i * MaxLen, st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
-        CheckHip(hipMemcpyAsync(SpanFinish + (size_t)i * MaxLen, fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
+        for (int t = 0; t < len; ++t) keys += std::max(0, fi[i][t] - st[i][t] + 1);
+        CheckHip(hipMemcpyAsync(SpanStart + (size_t)i * MaxLen, st[i].data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
+        CheckHip(hipMemcpyAsync(SpanFinish + (size_t)i * MaxLen, fi[i].data(), sizeof(int32_t) * len, hipMemcpyHostToDevice, (hipStream_t)stream), "span copy");
         Check(tsattn_build_span_tiles(Handle, len, SpanStart + (size_t)i * MaxLen, SpanFinish + (size_t)i * MaxLen, SpanTiles + i * tileInts, stream),
               "tsattn_build_span_tiles");
     }
+    // keys per row of the longer rows (a causal window over sequences of S tokens averages S / 2): the library's hint
+    SpanLenHint = len > 0 ? 2 * keys / ((int64_t)len * parts) : 0;
     CheckHip(hipStreamSynchronize((hipStream_t)stream), "span copy");
 }
 
@@ -143,6 +151,7 @@ void TAttentionComputer::ComputeValLookup(int len, int dtype, const TQuantRows &
     a.q_scale_const = qk.ConstScale; a.k_scale_const = qv.ConstScale; a.v_scale_const = v.ConstScale;
     a.k_global_scale = qvGlobalScale;
     a.alibi_slope = AlibiSlope;
+    a.workspace = Workspace; a.workspace_bytes = (int64_t)WorkspaceBytes; a.span_len_hint = SpanLenHint;
     if (Parts == 1) {
         a.span_start = SpanStart; a.span_finish = SpanFinish;
         a.span_tiles = SpanTiles;

@@ -84,6 +84,9 @@ class TAttentionComputer
     int MaxLen = 0;
     int Len = 0;
     int CausalPeriod = 0; // launch-order hint derived from the spans by SetAttention
+    int64_t SpanLenHint = 0; // typical keys per row of the spans set (tsattn_prefill_args.span_len_hint)
+    void *Workspace = nullptr; // device scratch of the long-span kernel (tsattn_prefill_args.workspace), if maxLen can need it
+    size_t WorkspaceBytes = 0;
     // Rows may hold several spans: part i of the batch is every row's i-th span (an empty one for rows with fewer)
     int Parts = 1, PartCapacity = 0;
     int32_t *SpanStart = nullptr; // device [PartCapacity][MaxLen]

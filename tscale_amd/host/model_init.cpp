@@ -98,12 +98,13 @@ static float RandomInt8(std::vector<int8_t> *dst, std::vector<float> &tmp, int64
 }
 
 // gpt/model_params/model_params.cpp:47-151 (InitEmbedMatrix, InitAttention, InitModel) + gpt/train/cpu_infer.cpp:128-161
-void InitModel(THostModel *p, uint64_t seed, int dim, int headCount, int headDim, int depth, int wideLimitWindow, int64_t labelCount,
-               int64_t vocabSize, ECombinerInit combinerInit)
+void InitModel(THostModel *p, uint64_t seed, int dim, int headCount, int headDim, int reluMult, int depth, int wideLimitWindow,
+               int64_t labelCount, int64_t vocabSize, ECombinerInit combinerInit)
 {
     TFastNormalRng rng(seed);
     std::vector<float> tmp;
-    p->Dim = dim, p->QDim = headDim, p->TTDim = headDim, p->HeadCount = headCount, p->ReluDim = headCount * headDim;
+    p->Dim = dim, p->QDim = headDim, p->TTDim = headDim, p->HeadCount = headCount, p->ReluMult = reluMult;
+    p->ReluDim = headCount * 128 * reluMult; // TModelDims::GetReluDim, gpt/model_params/model_dim.h:66
     p->LabelCount = labelCount, p->VocabSize = vocabSize;
     // embedding: plain table values (not halved), the noise labels' rows zero
     tmp.assign((size_t)labelCount * dim, 0.0f);
@@ -136,15 +137,30 @@ void InitModel(THostModel *p, uint64_t seed, int dim, int headCount, int headDim
 
 extern "C" {
 
-int tshost_init_alibi(int alibi, int depth, int wide_limit_window, int *widths, float *slopes)
+int tshost_init_alibi(int alibi, int depth, int wide_limit_window, int *widths, float *slopes, int capacity)
 {
     NTsAttn::TLayerSchedule s;
     NTsAttn::InitAlibi(&s, (NTsAttn::EAlibi)alibi, depth, wide_limit_window);
-    for (size_t d = 0; d < s.Layers.size(); ++d) {
+    for (size_t d = 0; d < s.Layers.size() && (int)d < capacity; ++d) {
         widths[d] = s.GetAttentionWidth((int)d);
         slopes[d] = s.GetAlibiSlope((int)d);
     }
     return (int)s.Layers.size();
+}
+
+void tshost_init_model_shapes(int dim, int head_count, int head_dim, int relu_mult, int64_t shapes[7][2])
+{
+    // a model of one layer and the smallest tables: only the layer's matrix sizes are looked at
+    NTsAttn::THostModel m;
+    NTsAttn::InitModel(&m, 1, dim, head_count, head_dim, relu_mult, 1, 64, NTsAttn::NOISE_LABELS_COUNT + 1, 1, NTsAttn::COMBINER_INIT_RANDOM);
+    const NTsAttn::THostAttention &a = m.LayerArr[0];
+    const int64_t q_sum = (int64_t)head_count * head_dim;
+    const std::vector<int8_t> *mats[7] = {&a.QK, &a.QV, &a.K, &a.V, &a.Combiner, &a.Expand, &a.Contract};
+    const int64_t cols[7] = {dim, dim, dim, dim, q_sum * 4, dim, m.ReluDim};
+    for (int i = 0; i < 7; ++i) {
+        shapes[i][1] = cols[i];
+        shapes[i][0] = (int64_t)mats[i]->size() / cols[i];
+    }
 }
 
 float tshost_convert_matrix(const float *data, int64_t x_size, int64_t y_size, int8_t *dst) { return NTsAttn::ConvertMatrix(data, x_size, y_size, dst); }

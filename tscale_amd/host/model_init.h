@@ -68,7 +68,8 @@ struct THostAttention {                       // one layer, int8, one row per ou
 };
 
 struct THostModel {                            // TCPUModelParams of the reference, on the host
-    int Dim = 0, QDim = 0, TTDim = 0, HeadCount = 0, ReluDim = 0;
+    int Dim = 0, QDim = 0, TTDim = 0, HeadCount = 0, ReluMult = 1;
+    int ReluDim = 0;                           // HeadCount * 128 * ReluMult whatever the head width (gpt/model_params/model_dim.h:66)
     int64_t LabelCount = 0, VocabSize = 0;
     std::vector<int8_t> LabelEmbed, FinalLayer; // [LabelCount][Dim], [VocabSize][Dim]
     float LabelEmbedScale = 0, FinalLayerScale = 0;
@@ -81,15 +82,20 @@ struct THostModel {                            // TCPUModelParams of the referen
 // combinerInit: the reference's create_model() starts combiner and contract at zero, which cuts the attention output off
 // from the result; a random-init model that is to exercise attention uses COMBINER_INIT_RANDOM, as the reference's own
 // CPU/GPU comparison does (gpt/train/main_gpt.cpp:274).
-void InitModel(THostModel *p, uint64_t seed, int dim, int headCount, int headDim, int depth, int wideLimitWindow, int64_t labelCount,
-               int64_t vocabSize, ECombinerInit combinerInit);
+// reluMult: the feed-forward block's width in units of 128 per head (TModelDims::ReluMult).
+void InitModel(THostModel *p, uint64_t seed, int dim, int headCount, int headDim, int reluMult, int depth, int wideLimitWindow,
+               int64_t labelCount, int64_t vocabSize, ECombinerInit combinerInit);
 
 } // namespace NTsAttn
 
 // The same through a C ABI (libtshost.so), for callers that are not C++.
 extern "C" {
-// widths[depth], slopes[depth]: every layer's attention width and ALiBi slope
-int tshost_init_alibi(int alibi, int depth, int wide_limit_window, int *widths, float *slopes);
+// Every layer's attention width and ALiBi slope.  Returns the number of layers the schedule has -- depth rounded up to
+// an even number for ALIBI_V3, whose layers come in pairs (gpt/model_params/model_dim.cpp:63-79) -- and writes the first
+// min(that, capacity) of them; call with capacity 0 to ask for the count.
+int tshost_init_alibi(int alibi, int depth, int wide_limit_window, int *widths, float *slopes, int capacity);
+// the sizes InitModel gives the matrices of one layer: {QK, QV, K, V} rows x cols, Combiner, Expand, Contract (rows, cols each)
+void tshost_init_model_shapes(int dim, int head_count, int head_dim, int relu_mult, int64_t shapes[7][2]);
 float tshost_convert_matrix(const float *data, int64_t x_size, int64_t y_size, int8_t *dst);
 // data[y_size][x_size] floats as InitMatrixNormal makes them from a generator seeded with `seed`
 void tshost_init_matrix_normal(uint64_t seed, float sko, int64_t x_size, int64_t y_size, float *data);

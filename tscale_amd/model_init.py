@@ -19,7 +19,9 @@ def load():
             raise FileNotFoundError(f"{LIB_PATH} is missing: build it with `make -C tscale_amd/host`")
         L = _c.CDLL(LIB_PATH)
         L.tshost_init_alibi.restype = _c.c_int
-        L.tshost_init_alibi.argtypes = [_c.c_int, _c.c_int, _c.c_int, _c.c_void_p, _c.c_void_p]
+        L.tshost_init_alibi.argtypes = [_c.c_int, _c.c_int, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int]
+        L.tshost_init_model_shapes.restype = None
+        L.tshost_init_model_shapes.argtypes = [_c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p]
         L.tshost_convert_matrix.restype = _c.c_float
         L.tshost_convert_matrix.argtypes = [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p]
         L.tshost_init_matrix_normal.argtypes = [_c.c_uint64, _c.c_float, _c.c_int64, _c.c_int64, _c.c_void_p]
@@ -30,11 +32,19 @@ def load():
 
 def init_alibi(depth, wide_limit_window, alibi=ALIBI_V3):
     """[(attention width, ALiBi slope)] per layer."""
-    n = max(depth, 1) + 1
+    n = load().tshost_init_alibi(alibi, depth, wide_limit_window, None, None, 0)   # the schedule's own count (an odd depth gains a layer)
     w = np.zeros(n, dtype=np.int32)
     s = np.zeros(n, dtype=np.float32)
-    got = load().tshost_init_alibi(alibi, depth, wide_limit_window, w.ctypes.data, s.ctypes.data)
+    got = load().tshost_init_alibi(alibi, depth, wide_limit_window, w.ctypes.data, s.ctypes.data, n)
+    assert got == n
     return [(int(w[i]), float(s[i])) for i in range(got)]
+
+
+def init_model_shapes(dim, head_count, head_dim, relu_mult=1):
+    """(rows, cols) of the matrices NTsAttn::InitModel gives a layer: QK, QV, K, V, Combiner, Expand, Contract."""
+    out = np.zeros((7, 2), dtype=np.int64)
+    load().tshost_init_model_shapes(dim, head_count, head_dim, relu_mult, out.ctypes.data)
+    return dict(zip(("QK", "QV", "K", "V", "Combiner", "Expand", "Contract"), (tuple(int(x) for x in r) for r in out)))
 
 
 def convert_matrix(data):
