@@ -743,9 +743,10 @@ static int RunContextCase(int firstLayer, int nLayers, int headDim = 128, int re
     return fails;
 }
 
-// Rows with several spans through TAttentionComputer (one launch per span of the rows, then the combining launch)
-// against the oracle's loop over a row's spans inside one softmax, on the dequantised operands.
-static int RunSeveralSpansCase(int dtype, float slope, bool outF16)
+// Rows with several spans through TAttentionComputer -- one launch that walks the parts, or (mergeParts) one launch per
+// span of the rows and the combining launch -- against the oracle's loop over a row's spans inside one softmax, on the
+// dequantised operands.
+static int RunSeveralSpansCase(int dtype, float slope, bool outF16, bool mergeParts)
 {
     const int H = 2, d = 128, len = 230;
     TModelDims dims;
@@ -788,6 +789,7 @@ static int RunSeveralSpansCase(int dtype, float slope, bool outF16)
     tso_prefill_f32(len, H, d, d, deq[0].data(), deq[1].data(), deq[2].data(), spanPtr.data(), spans.data(), slope, want.data(), nullptr, nullptr);
 
     TAttentionComputer attComp(dims, slope, 0, len + 26, 0); // (a context longer than the batch: pitches differ from len)
+    attComp.MergeParts = mergeParts;
     attComp.SetAttention(att, nullptr);
     uint8_t *dq = ToDevice(q), *dk = ToDevice(k), *dv = ToDevice(v);
     std::vector<float> qsP((size_t)H * (len + 26)), ksP(qsP.size()), vsP(qsP.size()); // scale planes of the context's pitch
@@ -834,15 +836,18 @@ static int RunSeveralSpansCase(int dtype, float slope, bool outF16)
         ++fails;
     }
     for (void *p : {(void *)dq, (void *)dk, (void *)dv, (void *)dqs, (void *)dks, (void *)dvs, dout}) HIP_OK(hipFree(p));
-    printf("several spans per row, dtype %d slope %g %s: max %.2e mean %.2e\n", dtype, slope, outF16 ? "f16" : "f32", maxErr, meanErr);
+    printf("several spans per row, dtype %d slope %g %s, %s: max %.2e mean %.2e\n", dtype, slope, outF16 ? "f16" : "f32",
+           mergeParts ? "a launch per part + merge" : "one launch", maxErr, meanErr);
     return fails;
 }
 
 int main()
 {
     int fails = 0;
-    fails += RunSeveralSpansCase(TSATTN_I8, 0.0f, false);
-    fails += RunSeveralSpansCase(TSATTN_E4M3, 0.25f, true);
+    for (int merge = 0; merge < 2; ++merge) {
+        fails += RunSeveralSpansCase(TSATTN_I8, 0.0f, false, merge != 0);
+        fails += RunSeveralSpansCase(TSATTN_E4M3, 0.25f, true, merge != 0);
+    }
     for (int l = 0; l < 3; ++l) fails += RunContextCase(l, 1);
     fails += RunContextCase(0, 3);
     fails += RunContextCase(0, 3, 64, 2, true);   // a model from InitModel: head width 64, feed-forward groups of 256

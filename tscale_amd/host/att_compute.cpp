@@ -115,7 +115,7 @@ void TAttentionComputer::SetAttention(const TAttentionInfo &attInfo, void *strea
     Reserve(parts);
     Parts = parts;
     Len = len;
-    const int64_t tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(MaxLen);
+    const int64_t tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(len); // the parts' summaries follow one another
     // every part's host arrays live until the copies have been waited for below
     std::vector<std::vector<int32_t>> st(parts), fi(parts);
     int64_t keys = 0;
@@ -161,8 +161,17 @@ void TAttentionComputer::ComputeValLookup(int len, int dtype, const TQuantRows &
         Check(tsattn_prefill(Handle, &a, stream), "tsattn_prefill");
         return;
     }
-    // one softmax over all the spans of a row (gpt_cpu.cpp:405-436) = the parts' results combined by their weights
-    const int64_t row = (int64_t)Dims.HeadCount * Dims.TTDim, tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(MaxLen);
+    if (!MergeParts) {
+        // one launch walks every row's spans part by part: one softmax over all of them (gpt_cpu.cpp:405-436)
+        a.span_start = SpanStart; a.span_finish = SpanFinish; a.span_tiles = SpanTiles;
+        a.n_span_parts = Parts; a.span_part_stride = MaxLen;
+        a.out = valLookup; a.out_pitch = valLookupPitchBytes;
+        a.sum_weight_log = SumWeightLog;
+        Check(tsattn_prefill(Handle, &a, stream), "tsattn_prefill");
+        return;
+    }
+    // the same as one launch per part and their results combined by their weights
+    const int64_t row = (int64_t)Dims.HeadCount * Dims.TTDim, tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(len);
     a.out_dtype = TSATTN_OUT_F32;
     a.out_pitch = row * 4;
     for (int i = 0; i < Parts; ++i) {
@@ -493,7 +502,7 @@ void TLayerComputer::AddLookupProduct(const int32_t *t, const float *ropeBuf, in
 void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
                                             const TAttentionMatrices &att, const int32_t *spanStart, const int32_t *spanFinish,
                                             const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
-                                            void *stream, bool deferStateUpdate)
+                                            void *stream, bool deferStateUpdate, int nSpanParts, int64_t spanPartStride)
 {
     const int headCount = Dims.HeadCount, headDim = Dims.QDim, qsum = Dims.GetQSum();
     TS_VERIFY(!pKVCache || (pKVCache->HeadCount == headCount && pKVCache->HeadDim == headDim && pKVCache->DType == TSATTN_I8),
@@ -509,6 +518,7 @@ void TLayerComputer::AddLookupProductPrompt(int len, const int32_t *seqOffset, c
     pa.q_scale = nullptr; pa.q_scale_const = VEC_SCALE; pa.k_scale = QvHeadScale; pa.v_scale = nullptr; pa.v_scale_const = VEC_SCALE;
     pa.scale_pitch = len;
     pa.span_start = spanStart; pa.span_finish = spanFinish; pa.span_tiles = spanTiles; pa.causal_period = causalPeriod;
+    pa.n_span_parts = nSpanParts; pa.span_part_stride = spanPartStride;
     pa.alibi_slope = att.AlibiSlope;
     pa.out = WriteValLookup ? ValLookup : nullptr; pa.out_pitch = (int64_t)qsum * 4;
     // KVProduct (cpu_infer.cpp:511) as the attention kernel's last step
@@ -645,11 +655,9 @@ TComputeContext::TComputeContext(tsattn_handle_t handle, const TModelDims &dims,
     SpanFinish.assign(attentionWidthCount, nullptr);
     SpanTiles.assign(attentionWidthCount, nullptr);
     CausalPeriod.assign(attentionWidthCount, 0);
-    for (int k = 0; k < attentionWidthCount; ++k) {
-        CheckHip(hipMalloc((void **)&SpanStart[k], n * sizeof(int32_t)), "hipMalloc(spans)");
-        CheckHip(hipMalloc((void **)&SpanFinish[k], n * sizeof(int32_t)), "hipMalloc(spans)");
-        CheckHip(hipMalloc((void **)&SpanTiles[k], ((n + 127) / 128) * 32 * sizeof(int32_t)), "hipMalloc(span summary)");
-    }
+    SpanParts.assign(attentionWidthCount, 1);
+    SpanPartCapacity.assign(attentionWidthCount, 0);
+    for (int k = 0; k < attentionWidthCount; ++k) ReserveSpans(k, 1);
     // FillRopeBuf for every node index of the largest batch, and the nodes' positions (their indices), once
     std::vector<float> rope(n * dims.QDim);
     tsattn_fill_rope_table(dims.QDim, maxNodeCount, rope.data());
@@ -667,6 +675,20 @@ TComputeContext::~TComputeContext()
         (void)hipFree(SpanFinish[k]);
         (void)hipFree(SpanTiles[k]);
     }
+}
+
+// room for `parts` spans per row of width k's span list (more than one only where a batch has such rows)
+void TComputeContext::ReserveSpans(int k, int parts)
+{
+    if (parts <= SpanPartCapacity[k]) return;
+    (void)hipFree(SpanStart[k]);
+    (void)hipFree(SpanFinish[k]);
+    (void)hipFree(SpanTiles[k]);
+    const size_t n = (size_t)MaxNodeCount * parts;
+    CheckHip(hipMalloc((void **)&SpanStart[k], n * sizeof(int32_t)), "hipMalloc(spans)");
+    CheckHip(hipMalloc((void **)&SpanFinish[k], n * sizeof(int32_t)), "hipMalloc(spans)");
+    CheckHip(hipMalloc((void **)&SpanTiles[k], (size_t)((MaxNodeCount + 127) / 128) * parts * TSATTN_SPAN_TILE_INTS * sizeof(int32_t)), "hipMalloc(span summary)");
+    SpanPartCapacity[k] = parts;
 }
 
 TNodesBatch &TComputeContext::GetNodes(int deviceId)
@@ -695,13 +717,27 @@ void TComputeContext::Init(int deviceId, EInitType initType)
         for (uint32_t j = Nodes.LabelPtr[i]; j < Nodes.LabelPtr[i + 1]; ++j) labels[(size_t)i * perRow + (j - Nodes.LabelPtr[i])] = Nodes.LabelArr[j];
     if (len > 0) CheckHip(hipMemcpy(Labels, labels.data(), labels.size() * sizeof(int32_t), hipMemcpyHostToDevice), "label copy");
     std::vector<int32_t> st, fi;
+    const int64_t tileInts = TSATTN_SPAN_TILE_INTS * tsattn_span_tiles_count(len);
     for (int k = 0; k < AttentionWidthCount; ++k) {
-        TS_VERIFY((int)Nodes.AttArr[k].GetSampleCount() == len, "span list %d has %d samples for %d nodes", k, (int)Nodes.AttArr[k].GetSampleCount(), len);
-        CausalPeriod[k] = FlattenSpans(Nodes.AttArr[k], &st, &fi);
-        if (len == 0) continue;
-        CheckHip(hipMemcpy(SpanStart[k], st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice), "span copy");
-        CheckHip(hipMemcpy(SpanFinish[k], fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice), "span copy");
-        Check(tsattn_build_span_tiles(Handle, len, SpanStart[k], SpanFinish[k], SpanTiles[k], nullptr), "tsattn_build_span_tiles");
+        const TAttentionInfo &att = Nodes.AttArr[k];
+        TS_VERIFY((int)att.GetSampleCount() == len, "span list %d has %d samples for %d nodes", k, (int)att.GetSampleCount(), len);
+        // rows may hold several spans (the reference's ComputeFragmentPredictions takes any TAttentionInfo,
+        // gpt_cpu.cpp:405-436): part i is every row's i-th span, walked by the one attention launch of the layer
+        int parts = 1;
+        for (int t = 0; t < len; ++t) parts = std::max(parts, att.SpanPtr[t + 1] - att.SpanPtr[t]);
+        TS_VERIFY(parts <= 64, "a node with %d spans; up to 64 are supported", parts);
+        if (parts > SpanPartCapacity[k]) CheckHip(hipDeviceSynchronize(), "before the span arrays grow");
+        ReserveSpans(k, parts);
+        SpanParts[k] = parts;
+        for (int i = 0; i < parts; ++i) {
+            const int period = FlattenSpans(att, &st, &fi, i, false);
+            CausalPeriod[k] = parts == 1 ? period : 0;
+            if (len == 0) continue;
+            int32_t *const ds = SpanStart[k] + (size_t)i * MaxNodeCount, *const df = SpanFinish[k] + (size_t)i * MaxNodeCount;
+            CheckHip(hipMemcpy(ds, st.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice), "span copy"); // (blocking: st, fi are reused)
+            CheckHip(hipMemcpy(df, fi.data(), sizeof(int32_t) * len, hipMemcpyHostToDevice), "span copy");
+            Check(tsattn_build_span_tiles(Handle, len, ds, df, SpanTiles[k] + i * tileInts, nullptr), "tsattn_build_span_tiles");
+        }
     }
     CheckHip(hipDeviceSynchronize(), "batch set-up");
 }
@@ -716,7 +752,7 @@ const uint8_t *TComputeContext::ComputeForward(void *stream)
     for (size_t d = 0; d < Model.LayerArr.size(); ++d) {
         const int k = LayerWidthId[d];
         Layer.AddLookupProductPrompt(Len, nullptr, Pos, RopeBuf, MaxNodeCount, Model.LayerArr[d], SpanStart[k], SpanFinish[k], SpanTiles[k],
-                                     CausalPeriod[k], nullptr, State, stream, true);
+                                     CausalPeriod[k], nullptr, State, stream, true, SpanParts[k], MaxNodeCount);
     }
     return Layer.FlushState(Len, State, stream);
 }

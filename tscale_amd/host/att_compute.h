@@ -98,6 +98,9 @@ class TAttentionComputer
     void Reserve(int parts);
 
   public:
+    // Rows with several spans: false = one launch that walks them (n_span_parts of tsattn_prefill_args), true = one launch
+    // per span of the rows and tsattn_merge_lookups.  The same result up to rounding.
+    bool MergeParts = false;
     // maxSeqs > 0 also provisions the handle for KV-cache decode of that many sequences
     TAttentionComputer(const TModelDims &dims, float alibiSlope, int deviceId, int maxLen, int maxSeqs = 0);
     ~TAttentionComputer();
@@ -221,7 +224,7 @@ class TLayerComputer
     void AddLookupProductPrompt(int len, const int32_t *seqOffset, const int32_t *pos, const float *ropeBuf, int64_t ropeLen,
                                 const TAttentionMatrices &att, const int32_t *spanStart, const int32_t *spanFinish,
                                 const int32_t *spanTiles, int64_t causalPeriod, TAttentionVecHistory *pKVCache, float *state,
-                                void *stream, bool deferStateUpdate = false);
+                                void *stream, bool deferStateUpdate = false, int nSpanParts = 1, int64_t spanPartStride = 0);
     const float *GetValLookup() const { return ValLookup; } // [rows][HeadCount*TTDim] of the last call
     // false: AddLookupProductPrompt does not write the attention output (its KVProduct, made by the same kernel, is all
     // the layer reads); GetValLookup() is then stale after that call
@@ -301,6 +304,8 @@ class TComputeContext
     int32_t *Labels = nullptr, *Pos = nullptr;
     std::vector<int32_t *> SpanStart, SpanFinish, SpanTiles; // per attention width, device
     std::vector<int> CausalPeriod;
+    std::vector<int> SpanParts, SpanPartCapacity; // per width: spans per row of the batch set, and what the arrays hold
+    void ReserveSpans(int k, int parts);
     float *State = nullptr, *RopeBuf = nullptr, *Prediction = nullptr;
 
     const uint8_t *ComputeForward(void *stream); // returns NormalizeState of the final state (device)
