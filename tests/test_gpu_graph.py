@@ -57,6 +57,28 @@ def eager_noise():
     return float((x * 2 + 1).sum())
 
 
+def test_long_span_prefill_replays(ctx):
+    """The long-span kernel and the kernel that writes its copy of V into the caller's workspace, as two nodes of a graph."""
+    dtype, H, d, n = capi.E4M3, 4, 128, 900
+    g0 = torch.Generator(device="cuda").manual_seed(6)
+    q, qs = ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g0), H, dtype)
+    k, ks = ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g0), H, dtype)
+    v, vs = ctx.quantize_rows(torch.randn((n, H * d), device="cuda", generator=g0), H, dtype)
+    off = torch.tensor([0, n], dtype=torch.int32, device="cuda")
+    st, fi = ctx.build_spans(off, n, 10 ** 6)
+    hint = capi.PREFILL_LONG_SPAN
+    want = ctx.compute_val_lookup(dtype, H, q, k, v, qs, ks, vs, st, fi, 0.0, span_len_hint=hint).clone()   # (allocates the workspace)
+    out = torch.zeros_like(want)
+    graph = capture(lambda: ctx.compute_val_lookup(dtype, H, q, k, v, qs, ks, vs, st, fi, 0.0, out=out, span_len_hint=hint))
+    for _ in range(3):
+        out.zero_()
+        ctx._workspace.fill_(0xFF)   # the copy of V is made again by every replay (0xFF..: NaN halves)
+        eager_noise()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+
+
 @pytest.mark.parametrize("dtype,window,slope", [(capi.E4M3, 10 ** 6, 0.0), (capi.I8, 64, 0.5)])
 def test_prefill_replays(ctx, dtype, window, slope):
     H, d, lens = 4, 128, [300, 77, 513]

@@ -74,6 +74,67 @@ def test_fused_append_through_the_static_entry_point(ctx):
                 assert torch.equal(getattr(a, name), getattr(b, name)), (call, window, name)
 
 
+def test_no_device_memory_is_taken(ctx):
+    """Free device memory, as the driver reports it, is the same before and after static calls -- the first one of the
+    process on this device included when this file runs alone (the array is part of the library's device image)."""
+    B, H, L, d = 8, 4, 600, 128
+    cache = filled_cache(ctx, 31, B, H, L, d, [L] * B)
+    q = torch.randn((B, H * d), device="cuda").to(torch.bfloat16)
+    out = torch.empty((B, H * d), dtype=torch.float32, device="cuda")
+    want = ctx.compute_val_lookup_decode(cache, q, None, 10 ** 6, 0.0, n_splits=4)   # (the kernels' code is loaded by now)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        ctx.compute_val_lookup_decode(cache, q, None, 10 ** 6, 0.0, n_splits=4, out=out, static_scratch=True)
+        torch.cuda.synchronize()
+        free1, _ = torch.cuda.mem_get_info()
+        assert free1 == free0, (free0, free1)
+    assert torch.equal(out, want)
+
+
+def test_static_fused_append_in_a_graph(ctx):
+    """The static entry point under stream capture, without help from a handle's buffers: a fused-append decode with one
+    split (window 64: the arrival counters in the array are used, and cleared by the fill kernel in front of the launch),
+    replayed three times with eager work between the replays, every replay against eager calls on a copy of the cache."""
+    B, H, L, d = 6, 4, 300, 128
+    rng = np.random.default_rng(77)
+    lens = [int(x) for x in rng.integers(70, L - 8, B)]
+    a = filled_cache(ctx, 23, B, H, L, d, lens)
+    b = clone_cache(ctx, a)
+    g0 = torch.Generator(device="cuda").manual_seed(300)
+    x = torch.randn((3, B, H * d), device="cuda", generator=g0)
+    q, qs = ctx.quantize_rows(x[0], H, capi.I8)
+    kn, kns = ctx.quantize_rows(x[1], H, capi.I8)
+    vn, vns = ctx.quantize_rows(x[2], H, capi.I8)
+    qs, kns, vns = (s.t().contiguous() for s in (qs, kns, vns))
+    out = torch.zeros((B, H * d), dtype=torch.float32, device="cuda")
+    step = lambda: ctx.compute_val_lookup_decode(b, q, qs, 64, 0.5, out=out, append=(kn, kns, vn, vns), static_scratch=True)
+    # warm up on a side stream (as torch asks), put the cache back, record
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for name in ("k", "v", "k_scale", "v_scale", "cache_len"):
+        getattr(b, name).copy_(getattr(a, name))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    torch.cuda.synchronize()
+    for name in ("k", "v", "k_scale", "v_scale", "cache_len"):   # (capture runs nothing, but the cache is put back all the same)
+        getattr(b, name).copy_(getattr(a, name))
+    for replay in range(3):
+        want = ctx.compute_val_lookup_decode(a, q, qs, 64, 0.5, append=(kn, kns, vn, vns))   # eager, handle path
+        float((torch.randn(1 << 16, device="cuda") * 2 + 1).sum())                           # eager work of the program's own
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+        for name in ("k", "v", "k_scale", "v_scale", "cache_len"):
+            assert torch.equal(getattr(a, name), getattr(b, name)), (replay, name)
+
+
 def test_limits_are_refused_with_a_clear_error(ctx):
     from tscale_amd import KVCache
     B, H, L, d = 40, 16, 64, 64

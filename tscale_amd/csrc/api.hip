@@ -172,6 +172,7 @@ int tsattn_create(const tsattn_config *cfg, tsattn_handle_t *out)
     e = hipSetDevice(cfg->device);
     if (e != hipSuccess) return hip_fail(e, "hipSetDevice");
     e = tsattn::prepare_matmul_i8();
+    if (e == hipSuccess) e = tsattn::prepare_prefill_long();
     if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute");
     tsattn_ctx *c = new tsattn_ctx();
     c->device = cfg->device;

@@ -89,6 +89,7 @@ constexpr int VT_PAD = 32;
 inline int64_t prefill_long_vt_pitch(int64_t n_tokens) { return (n_tokens + 63) / 64 * 64 + 256; }
 size_t prefill_long_workspace_bytes(int64_t n_tokens, int n_heads, int head_dim);
 hipError_t launch_prefill_long(const PrefillParams &p, int dtype, int out_dtype, hipStream_t st);
+hipError_t prepare_prefill_long(); // once per device, at handle creation: lets the kernels ask for their LDS
 
 hipError_t launch_quantize_rows(int src_dtype, int dst_dtype, const void *src, int64_t src_pitch, int64_t n_rows,
                                 int n_heads, int head_dim, void *dst, int64_t dst_pitch, float *scale,

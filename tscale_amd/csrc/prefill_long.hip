@@ -612,12 +612,6 @@ static hipError_t launch_long_do(const PrefillParams &p_in, hipStream_t st)
     p.ks_pitch = p.scale_pitch;
     p.map = wg_plan(n_qtiles, p.n_heads, PL_D, PF_BM, p.period_tiles, 3); // K as it is, V as f16
     auto kernel = prefill_long_kernel<DTYPE, PL_D, OUT_F16, QS_CONST>;
-    static bool attr_set = false; // (per instantiation; setting it again is harmless)
-    if (!attr_set) {
-        const hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, PL_LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
     const dim3 wgrid((unsigned)(p.vt_pitch / 64), (unsigned)p.n_heads);
     float *ksq = nullptr;
     const int64_t ksq_pitch = ksq_pitch_of(p.n_tokens);
@@ -636,6 +630,27 @@ static hipError_t launch_long_do(const PrefillParams &p_in, hipStream_t st)
     }
     hipLaunchKernelGGL(kernel, dim3((unsigned)(n_qtiles * p.n_heads)), dim3(PF_THREADS), PL_LDS_BYTES, st, p, n_qtiles);
     return hipGetLastError();
+}
+
+template <int DTYPE, bool OUT_F16, bool QS_CONST>
+static hipError_t allow_lds()
+{
+    return hipFuncSetAttribute((const void *)prefill_long_kernel<DTYPE, PL_D, OUT_F16, QS_CONST>, hipFuncAttributeMaxDynamicSharedMemorySize, PL_LDS_BYTES);
+}
+
+// The kernels use more LDS than a launch may ask for by default: said once per device (at handle creation), so that no
+// launch has to, also not the first one under a graph capture.
+hipError_t prepare_prefill_long()
+{
+    hipError_t e = allow_lds<TSATTN_E4M3, true, true>();
+    if (e == hipSuccess) e = allow_lds<TSATTN_E4M3, true, false>();
+    if (e == hipSuccess) e = allow_lds<TSATTN_E4M3, false, true>();
+    if (e == hipSuccess) e = allow_lds<TSATTN_E4M3, false, false>();
+    if (e == hipSuccess) e = allow_lds<TSATTN_I8, true, true>();
+    if (e == hipSuccess) e = allow_lds<TSATTN_I8, true, false>();
+    if (e == hipSuccess) e = allow_lds<TSATTN_I8, false, true>();
+    if (e == hipSuccess) e = allow_lds<TSATTN_I8, false, false>();
+    return e;
 }
 
 hipError_t launch_prefill_long(const PrefillParams &p, int dtype, int out_dtype, hipStream_t st)
