@@ -14,6 +14,9 @@ A "step" is one pass of the hot path over one batch of synthetic input, inputs r
       on the InitAlibi schedule, int8, batch 32, 2048-token prompt, 256 generated tokens).
   "cpu_reference_config": batch 1, seq 1024, 12 heads x 64, int8, full causal window, fp32 output: the shape the
       reference's CPU path is quoted on; the CPU leg of it runs on int8, as that configuration says.
+  "prefill_long_span": the two prefill kernels side by side on full-window layers of 32768 tokens at S = 4096, 8192, 16384.
+  "token_step_24_layers", "prompt_pass_24_layers": the whole 24-layer stack of the host mirror around those attention
+      calls (int8 projections, producer, attention, feed-forward), one generated token and one prompt pass.
 Algorithmic work: FLOPs = 4*d*sum_rows min(row, W) per (sequence, head) (masked tiles count zero,
 the zero vector adds none); decode bytes = K + V planes + both scale planes + q + out.
 
@@ -142,7 +145,7 @@ class PrefillWorkload:
         self.flops = sum(self.flops_layer)
         torch.cuda.synchronize()
 
-    def run_layer(self, i):
+    def run_layer(self, i, span_len_hint=None):
         (q, qs), (k, ks), (v, vs) = self.inputs[i]
         W, slope = self.layers[i]
         st, fi = self.spans[W]
@@ -150,7 +153,7 @@ class PrefillWorkload:
         # (and the layer's attention width: with long spans the library takes its workspace kernel)
         self.ctx.compute_val_lookup(self.dtype, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
                                     causal_period=self.S if W >= self.S else 0, span_tiles=self.span_tiles[W],
-                                    span_len_hint=min(W, self.S))
+                                    span_len_hint=min(W, self.S) if span_len_hint is None else span_len_hint)
 
     def step(self):
         for i in range(len(self.layers)):
@@ -251,13 +254,14 @@ class GenerationWorkload:
         return total
 
 
-def bench_generation(ctx, steps):
+def bench_generation(ctx, steps, facts=None):
     import torch
+    facts = facts or {}
     gw = GenerationWorkload(ctx)
     res = {"config": "24 layers (4 x W=1, 10 x W=64 slope 0.5, 10 x full), B32, prompt 2048 + 256 generated tokens, "
                      "H16 d128 int8 Q/K/V + per-row f32 scales; attention launches only"}
     first = {W: [i for i, (w, _) in enumerate(gw.sched) if w == W][0] for W in gw.kinds}
-    pre_ms = {W: gpu_time_ms(lambda i=i: gw.prefill_layer(i), max(3, steps // 10), 1) for W, i in first.items()}
+    pre_ms = {W: gpu_time_ms(lambda i=i: gw.prefill_layer(i), max(50 if W == max(gw.kinds) else 10, steps // 5), 1) for W, i in first.items()}
     total_ms = sum(pre_ms[w] for w, _ in gw.sched)
     total_flops = sum(gw.prefill_flops(i) for i in range(len(gw.sched)))
     wide = max(gw.kinds)
@@ -269,6 +273,11 @@ def bench_generation(ctx, steps):
                                    "achieved": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9, 2), "peak": PEAK_I8_TOPS,
                                    "unit": "TOP/s", "frac": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9 / PEAK_I8_TOPS, 5),
                                    "traffic": None, "launch_ms": round(pre_ms[wide], 5), "flops_per_launch": gw.prefill_flops(first[wide])}}
+    fact = facts.get("prefill_prompt_int8_full")
+    if fact:
+        res["prefill"]["roofline"].update({"traffic": fact.get("traffic_bytes"), "traffic_from": fact["profile"]})
+        if "mfma_util" in fact:
+            res["prefill"]["roofline"]["mfma_util"] = fact["mfma_util"]
     fill_ms = gpu_time_ms(gw.fill_caches, 2, 1)
     n = gw.B * gw.prompt
     fill_bytes = len(gw.caches) * 2 * (n * gw.H * gw.d * 2 + n * gw.H * 4 * 2)   # read + write of K, V and both scales
@@ -306,6 +315,34 @@ def bench_generation(ctx, steps):
                                     "bound": "hbm", "achieved": round(nbytes / gen_ms / 1e6, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                                     "frac": round(nbytes / gen_ms / 1e6 / PEAK_HBM_GBPS, 4), "traffic": None,
                                     "bytes_per_token": nbytes // gw.n_new}}
+    fact = facts.get("decode_fused_append_token")
+    if fact:   # (measured over the 24 launches of the token whose caches hold 2048 + 128 rows: the middle of the run)
+        res["generate"]["roofline"].update({"traffic": fact.get("traffic_bytes"), "traffic_from": fact["profile"]})
+    return res
+
+
+def bench_long_span(ctx, steps):
+    """The launch-time choice between the two prefill kernels (span_len_hint in the arguments): a full-window e4m3 layer of
+    32768 tokens, 16 heads x 128, at three sequence lengths, once with no hint (the standard kernel, which stages K and V
+    through its waves) and once with a hint of at least TSATTN_PREFILL_LONG_SPAN (the long-span kernel: K and V'^T by DMA
+    into LDS, its time includes the kernel that writes V'^T into the workspace)."""
+    import torch
+    from tscale_amd import capi
+    res = {"config": "32768 tokens, H16 d128 e4m3 + per-row f32 scales, full causal window, f16 out; ms per launch and TFLOP/s",
+           "threshold": capi.PREFILL_LONG_SPAN}
+    for B, S in ((8, 4096), (4, 8192), (2, 16384)):
+        wl = PrefillWorkload(ctx, capi.E4M3, B, S, 16, 128, 2, seed=1313 + 6, short=256)
+        n = max(50, steps)
+        std, lng = [], []
+        for _ in range(2):   # alternating, so that both see the same state of the clocks; the better of two
+            std.append(gpu_time_ms(lambda: wl.run_layer(1, span_len_hint=0), n, 5))
+            lng.append(gpu_time_ms(lambda: wl.run_layer(1, span_len_hint=max(S, capi.PREFILL_LONG_SPAN)), n, 5))
+        std, lng = min(std), min(lng)
+        res[f"B{B}_S{S}"] = {"standard_ms": round(std, 5), "long_span_ms": round(lng, 5),
+                             "standard_TFLOP/s": round(wl.flops_layer[1] / std / 1e9, 1), "long_span_TFLOP/s": round(wl.flops_layer[1] / lng / 1e9, 1),
+                             "library_picks": "long-span" if S >= capi.PREFILL_LONG_SPAN else "standard"}
+        del wl
+        torch.cuda.empty_cache()
     return res
 
 
@@ -777,7 +814,32 @@ def run_only(ctx, args):
         ms = gpu_time_ms(dw.step, args.steps, args.warmup)
         print(json.dumps({"only": name, "ms": ms, "GB/s": dw.bytes / ms / 1e6}))
         return
-    if name == "c1-int8":
+    if name in ("prompt-int8-full", "decode-append-token"):
+        import torch
+        gw = GenerationWorkload(ctx)
+        if name == "prompt-int8-full":   # the full-window prefill launch over the 1.5B-style prompt (B32 x 2048, int8, d128)
+            i = [j for j, (w, _) in enumerate(gw.sched) if w == max(gw.kinds)][0]
+            ms = gpu_time_ms(lambda: gw.prefill_layer(i), args.steps, args.warmup)
+            print(json.dumps({"only": name, "ms": ms, "TOP/s": gw.prefill_flops(i) / ms / 1e9}))
+            return
+        # one generated token in the middle of the run: 24 decode launches with the append fused, caches at 2048 + 128 rows
+        gw.fill_caches()
+        for c in gw.caches:
+            c.cache_len.fill_(gw.prompt + gw.n_new // 2)
+        lens = torch.full((gw.B,), gw.prompt + gw.n_new // 2, dtype=torch.int32, device="cuda")
+        def token():
+            for c in gw.caches:
+                c.cache_len.copy_(lens)
+            gw.decode_step()
+        ms = gpu_time_ms(token, args.steps, args.warmup)
+        n = gw.prompt + gw.n_new // 2 + 1
+        nbytes = sum(gw.B * gw.H * (min(n - 1, W) * (2 * gw.d + 8) + gw.d + 4 + 4 * gw.d) for W, _ in gw.sched)
+        print(json.dumps({"only": name, "ms_per_token": ms, "bytes_per_token": nbytes, "GB/s": nbytes / ms / 1e6}))
+        return
+    if name == "long-s8192":   # the long-span kernel's own shape: B4 S8192, full window
+        wl = PrefillWorkload(ctx, capi.E4M3, 4, 8192, 16, 128, 2, seed=1313 + 6, short=256)
+        li = 1
+    elif name == "c1-int8":
         wl = PrefillWorkload(ctx, capi.I8, 1, 1024, 12, 64, 2, seed=1313 + 1)
         li = 1
     elif name.startswith("c2"):
@@ -798,10 +860,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--extra", action="store_true",
-                    help="also time the producer, KVProduct, the int8 matrix products, the token step, the prompt pass and "
-                         "generation with the whole int8 model")
+                    help="also time the producer, KVProduct, the int8 matrix products and generation with the whole int8 model")
     ap.add_argument("--only", default=None,
-                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "producer", "matmul", "token-step", "prompt-pass", "generate-model", "prompt-then-generate"],
+                    choices=["c2-short", "c2-full", "c4-short", "c4-full", "c1-int8", "decode", "prompt-int8-full", "decode-append-token", "long-s8192", "producer", "matmul", "token-step", "prompt-pass", "generate-model", "prompt-then-generate"],
                     help="profiling aid: run just this launch --steps times and print its timing")
     ap.add_argument("--calibrate", action="store_true",
                     help="with --only: first run three 256 MiB device copies (counter calibration)")
@@ -826,7 +887,7 @@ def main():
     wl = PrefillWorkload(ctx, capi.E4M3, B, S, H, d, 2, seed=1313 + 4, short=256)
     ms = gpu_time_ms(wl.step, args.steps, args.warmup)
     tflops = wl.flops / (ms * 1e-3) / 1e12
-    lsteps = max(10, args.steps // 2)
+    lsteps = max(50, args.steps)   # the launch durations behind `roofline`: at least 50 launches each
     ms_short = gpu_time_ms(lambda: wl.run_layer(0), lsteps, 2)
     ms_wide = gpu_time_ms(lambda: wl.run_layer(1), lsteps, 2)
     ach = wl.flops_layer[1] / (ms_wide * 1e-3) / 1e12
@@ -902,7 +963,12 @@ def main():
         del dw
         torch.cuda.empty_cache()
         # ---- the attention calls of the 1.5B-style generation run ---------------------------------
-        result["generation_1p5B_style"] = bench_generation(ctx, args.steps)
+        result["generation_1p5B_style"] = bench_generation(ctx, args.steps, facts)
+        torch.cuda.empty_cache()
+        result["prefill_long_span"] = bench_long_span(ctx, args.steps)
+        # ---- the whole layer stack around the attention calls (a few seconds) ------------------------
+        result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
+        result["prompt_pass_24_layers"] = bench_prompt_pass(ctx, args.steps)
         torch.cuda.empty_cache()
 
     # ---- optional: 1.5B-style prefill shapes ---------------------------------------------------------
@@ -911,8 +977,6 @@ def main():
         torch.cuda.empty_cache()
         result["kv_product"] = bench_kv_product(ctx, args.steps)
         result["combiner_matmul"] = bench_matmul(ctx, args.steps)
-        result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
-        result["prompt_pass_24_layers"] = bench_prompt_pass(ctx, args.steps)
         result["generate_whole_model"] = bench_generate_model(ctx, args.steps)
         torch.cuda.empty_cache()
         result["prompt_then_generate_256"] = bench_prompt_then_generate(ctx)
