@@ -321,7 +321,7 @@ def bench_generation(ctx, steps, facts=None):
     return res
 
 
-def bench_long_span(ctx, steps):
+def bench_long_span(ctx, steps, facts=None):
     """The launch-time choice between the two prefill kernels (span_len_hint in the arguments): a full-window e4m3 layer of
     32768 tokens, 16 heads x 128, at three sequence lengths, once with no hint (the standard kernel, which stages K and V
     through its waves) and once with a hint of at least TSATTN_PREFILL_LONG_SPAN (the long-span kernel: K and V'^T by DMA
@@ -341,6 +341,9 @@ def bench_long_span(ctx, steps):
         res[f"B{B}_S{S}"] = {"standard_ms": round(std, 5), "long_span_ms": round(lng, 5),
                              "standard_TFLOP/s": round(wl.flops_layer[1] / std / 1e9, 1), "long_span_TFLOP/s": round(wl.flops_layer[1] / lng / 1e9, 1),
                              "library_picks": "long-span" if S >= capi.PREFILL_LONG_SPAN else "standard"}
+        if S == 8192:
+            res[f"B{B}_S{S}"]["roofline"] = roofline("prefill_long_kernel<e4m3, d128> + widen_v_kernel, full causal window", "mfma",
+                                                     wl.flops_layer[1] / lng / 1e9, wl.flops_layer[1], lng, (facts or {}).get("prefill_long_s8192"))
         del wl
         torch.cuda.empty_cache()
     return res
@@ -965,7 +968,7 @@ def main():
         # ---- the attention calls of the 1.5B-style generation run ---------------------------------
         result["generation_1p5B_style"] = bench_generation(ctx, args.steps, facts)
         torch.cuda.empty_cache()
-        result["prefill_long_span"] = bench_long_span(ctx, args.steps)
+        result["prefill_long_span"] = bench_long_span(ctx, args.steps, facts)
         # ---- the whole layer stack around the attention calls (a few seconds) ------------------------
         result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
         result["prompt_pass_24_layers"] = bench_prompt_pass(ctx, args.steps)
