@@ -66,6 +66,10 @@ def roofline(kernel, bound, achieved, flops_or_bytes, launch_ms, fact):
     peak, unit = (PEAK_FP8_TFLOPS, "TFLOP/s") if bound == "mfma" else (PEAK_HBM_GBPS, "GB/s")
     r = {"kernel": kernel, "bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
          "frac": round(achieved / peak, 5), "traffic": None, "launch_ms": round(launch_ms, 5)}
+    if bound == "mfma":
+        # half of the algorithmic FLOPs (P.V) run as f16 matrix instructions at half the fp8 rate: the matrix pipes are
+        # full at 2/3 of `peak`
+        r["frac_of_executed_mfma_peak"] = round(achieved / (peak * 2.0 / 3.0), 5)
     r["flops_per_launch" if bound == "mfma" else "bytes_per_launch"] = flops_or_bytes
     if fact:
         r["traffic"] = fact.get("traffic_bytes")
