@@ -122,6 +122,30 @@ def test_long_constant_query_scale(ctx, dtype, ks_plane, gscale):
     assert_within_tolerance(out, want, "constant query scale")
 
 
+@pytest.mark.parametrize("dtype", [capi.I8, capi.E4M3])
+def test_long_padded_rows_and_planes(ctx, dtype):
+    """Q, K, V and the output as column slices of wider arrays (row pitches larger than a row, each different), scale
+    planes with a pitch larger than the token count, one head: the kernel's row addresses come from the pitches."""
+    H, n = 1, 333
+    q, qs, k, ks, v, vs = make_qkv(21, n, H, D, dtype)
+    st, fi = orc.make_spans([200, 133], 10 ** 6)
+    want, want_swl = orc.prefill_q8(dtype, q, k, v, H, qs, ks, vs, st, fi, 0.0, want_swl=True)
+    def wide(a, extra, fill):
+        w = torch.full((a.shape[0], a.shape[1] + extra), fill, dtype=torch.uint8, device="cuda")
+        w[:, :a.shape[1]] = t(a)
+        return w[:, :a.shape[1]]
+    planes = torch.full((4, H, n + 40), 7.0, dtype=torch.float32, device="cuda")   # q, k, v scales and sum_weight_log
+    for i, sc in enumerate((qs, ks, vs)):
+        planes[i, :, :n] = t(sc)
+    out_w = torch.full((n, H * D + 48), -5.0, dtype=torch.float32, device="cuda")
+    out = ctx.compute_val_lookup(dtype, H, wide(q, 16, 0x7F), wide(k, 64, 0x7F), wide(v, 32, 0x7F), planes[0, :, :n], planes[1, :, :n], planes[2, :, :n],
+                                 t(st), t(fi), 0.0, out=out_w[:, :H * D], sum_weight_log=planes[3, :, :n], span_len_hint=8192)
+    torch.cuda.synchronize()
+    assert_within_tolerance(out.cpu().numpy(), want, "padded rows")
+    assert np.abs(planes[3, :, :n].cpu().numpy() - want_swl).max() < 1e-3
+    assert bool((out_w[:, H * D:] == -5.0).all()) and bool((planes[3, :, n:] == 7.0).all()), "nothing written outside the rows"
+
+
 def test_long_full_size_properties(ctx):
     """1.5B-style shape at full size (B8 S4096 H16 d128 e4m3): V = ones of scale 1 gives out = 1 - 2^-sum_weight_log in
     every column, row 0 of every sequence is zero, and the result equals the standard kernel's within the f16 rounding
