@@ -98,7 +98,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
     constexpr int SHORT_BYTES = PF_SHORT_KEYS * L::V_PITCH + PF_SHORT_KEYS * 4;
     constexpr bool HAS_SHORT = (D == 64) && !DUMP;
     // the common-tile loop with ALiBi only where it fits into the registers without spilling
-    constexpr bool FAST_LOOP = !DUMP && (!SLOPE || (D == 128 && DTYPE == TSATTN_E4M3));
+    constexpr bool FAST_LOOP = !DUMP && (!SLOPE || (D == 128 && DTYPE == TSATTN_E4M3 && !MULTI)); // (with ALiBi and a loop over parts it would spill)
     constexpr int LDS_BYTES = (HAS_SHORT && SHORT_BYTES > LOOP_BYTES) ? SHORT_BYTES : LOOP_BYTES;
     // the fused KVProduct exists where the reference has one: behind int8 attention with an f32 result (cpu_infer.cpp:509-511)
     constexpr bool KV_FUSED = DTYPE == TSATTN_I8 && !OUT_F16 && !DUMP;
@@ -848,7 +848,20 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read before the second half overwrites it
         }
     }
-    if (row_ok && p.sum_weight_log && g == 0) p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m_ref + __log2f(l_all);
+    if constexpr (!MULTI) {
+        if (p.sum_weight_log) {
+            // (the row's index from opaque copies again: kept in registers through the tile loops it costs the ALiBi
+            // kernels a spill; the kernels with a loop over parts around the tile loops fare better as they are)
+            int qi_e = lane & 31, g_e = lane >> 5, q0_e = tile * PF_BM + wave * 32;
+#if defined(__HIP_DEVICE_COMPILE__)
+            asm volatile("" : "+v"(qi_e), "+v"(g_e), "+v"(q0_e));
+#endif
+            const int from_e = q0_e + qi_e;
+            if (from_e < p.n_tokens && g_e == 0) p.sum_weight_log[(int64_t)head * p.scale_pitch + from_e] = m_ref + __log2f(l_all);
+        }
+    } else {
+        if (row_ok && p.sum_weight_log && g == 0) p.sum_weight_log[(int64_t)head * p.scale_pitch + from] = m_ref + __log2f(l_all);
+    }
 }
 
 template <int DTYPE, int D, bool OUT_F16>
