@@ -113,6 +113,30 @@ def test_prefill_constant_scales_and_global_key_scale(ctx):
     assert_within_tolerance(out, want, "constant scales")
 
 
+@pytest.mark.parametrize("dtype", [capi.I8, capi.E4M3])
+@pytest.mark.parametrize("d,window,slope,seq_lens", [
+    (128, 10 ** 6, 0.0, [700, 324]),     # the common-tile loop, tiles on the diagonal, a sequence boundary inside a tile
+    (128, 256, 0.5, [900]),              # ALiBi, both ends of the spans cut through tiles
+    (64, 10 ** 6, 0.0, [513, 255]),
+    (64, 64, 0.25, [400, 1, 130]),       # the short-range path of d = 64
+])
+def test_prefill_constant_query_scale(ctx, dtype, d, window, slope, seq_lens):
+    """TScale's own model passes one number as the query scale (VEC_SCALE, gpt_att_fp8.cuh:137): the kernels that fold it
+    into the staged key scales, per-row key and value scales as usual, f32 and f16 results, with sum_weight_log."""
+    H, n = 3, sum(seq_lens)
+    q, _, k, ks, v, vs = make_qkv(77, n, H, d, dtype)
+    VEC = np.float32(1.0 / 48 if dtype == capi.I8 else 1.0 / 96)   # (logits of the usual size for these rows)
+    st, fi = orc.make_spans(seq_lens, window)
+    want, want_swl = orc.prefill_q8(dtype, q, k, v, H, float(VEC), ks, vs, st, fi, slope, want_swl=True)
+    tt = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    for f16 in (False, True):
+        swl = torch.zeros((H, n), dtype=torch.float32, device="cuda")
+        out = ctx.compute_val_lookup(dtype, H, tt(q), tt(k), tt(v), float(VEC), tt(ks), tt(vs), tt(st), tt(fi), slope, out_f16=f16, sum_weight_log=swl)
+        torch.cuda.synchronize()
+        assert_within_tolerance(out.float().cpu().numpy(), want, f"constant query scale, f16 out {f16}")
+        assert np.abs(swl.cpu().numpy() - want_swl).max() < 1e-3
+
+
 @pytest.mark.parametrize("dtype,B,S,H,d,window,slope", [
     (capi.I8, 1, 1024, 12, 64, 1024, 0.0),     # the CPU-reference configuration, full size
     (capi.E4M3, 2, 1024, 12, 64, 64, 0.5),     # 125M-style short-window layer, reduced batch

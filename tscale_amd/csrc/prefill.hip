@@ -81,7 +81,9 @@ __device__ inline void widen_v_word(int w, v2h vs2, v2h &h0, v2h &h1)
 typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
 
 // MULTI: rows may have several spans (p.n_parts arrays of them); otherwise the one-span kernel, which needs fewer registers.
-template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP, bool MULTI>
+// QS_CONST: the query scale is one number for all rows (TScale's own model: VEC_SCALE, gpt_att_fp8.cuh:137); it is
+// multiplied into the key scales as they are staged and a logit costs one multiply-add instead of a multiply and one.
+template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP, bool MULTI, bool QS_CONST>
 __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefill_kernel(PrefillParams p, int n_qtiles)
 {
     typedef PfLayout<D> L;
@@ -137,10 +139,13 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
     Qk qk;
     if (row_ok) qk.load_q(p.q + (int64_t)from * p.q_pitch + hoff, g);
     else qk.clear_q();
-    const float qs = row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f;
+    const float qs = QS_CONST ? 1.0f : (row_ok ? (p.qs ? p.qs[(int64_t)head * p.scale_pitch + from] : p.qs_const) : 0.0f);
 
     float ads = att_dot_scale(D);
     if (p.k_global_scale) ads *= *p.k_global_scale;
+    if (QS_CONST) ads *= p.qs_const; // (rows past the end have zero operands: their logits are zero either way)
+    // a logit from an accumulator, its key's staged scale and what is added to it
+    auto logit = [&](float a, float k, float bias) __attribute__((always_inline)) { return QS_CONST ? fmaf(a, k, bias) : fmaf(a * k, qs, bias); };
 
     v16f o_acc[DT];
 #pragma unroll
@@ -331,8 +336,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
                             ((float *)p.dbg)[((int64_t)head * p.n_tokens + from) * p.dbg_pitch + key0 + off + 4 * g] = Qk::bits(acc, r);
                         }
                     }
-                    float x = Qk::to_float(acc, r) * ksv[j];
-                    float tv = fmaf(x, qs, bias);
+                    float tv = logit(Qk::to_float(acc, r), ksv[j], bias);
                     if (SLOPE) bias += (j == 3) ? slope5 : p.slope;
                     tv = in_span ? tv : -INFINITY;
                     t[r] = tv;
@@ -383,7 +387,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int off = 8 * c4 + j;
-                    const float tv = fmaf(Qk::to_float(acc, c4 * 4 + j) * ksv[j], qs, bias);
+                    const float tv = logit(Qk::to_float(acc, c4 * 4 + j), ksv[j], bias);
                     if (SLOPE) bias += (j == 3) ? slope5 : p.slope;
                     float pw = fast_exp2(tv);
                     if (LOW) pw = (lo <= off) ? pw : 0.0f;
@@ -458,10 +462,10 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
                 b2 = b1 + p.slope;
                 b3 = b2 + p.slope;
             }
-            const float p0 = fast_exp2(fmaf(Qk::to_float(acc, r) * ksv[0], qs, nbase));
-            const float p1 = fast_exp2(fmaf(Qk::to_float(acc, r + 1) * ksv[1], qs, b1));
-            const float p2 = fast_exp2(fmaf(Qk::to_float(acc, r + 2) * ksv[2], qs, b2));
-            const float p3 = fast_exp2(fmaf(Qk::to_float(acc, r + 3) * ksv[3], qs, b3));
+            const float p0 = fast_exp2(logit(Qk::to_float(acc, r), ksv[0], nbase));
+            const float p1 = fast_exp2(logit(Qk::to_float(acc, r + 1), ksv[1], b1));
+            const float p2 = fast_exp2(logit(Qk::to_float(acc, r + 2), ksv[2], b2));
+            const float p3 = fast_exp2(logit(Qk::to_float(acc, r + 3), ksv[3], b3));
             if (SLOPE) nbase = b3 + 5.0f * p.slope;
             s0 += p0;
             s1 += p1;
@@ -476,7 +480,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float bias = SLOPE ? bias0 + p.slope * (float)(8 * (r / 4) + (r & 3)) : bias0;
-                xs[r] = fmaf(Qk::to_float(acc, r) * ksp[8 * (r / 4) + (r & 3)], qs, bias);
+                xs[r] = logit(Qk::to_float(acc, r), ksp[8 * (r / 4) + (r & 3)], bias);
                 tmax = fmaxf(tmax, xs[r]);
             }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
@@ -875,16 +879,19 @@ static void launch_prefill_do(const PrefillParams &p_in, dim3 grid2, hipStream_t
     const bool slope = p.slope != 0.0f;
     dim3 block(PF_THREADS);
     const bool multi = p.n_parts > 1;
+    const bool qs_const = p.qs == nullptr && !dump && !multi; // (the rarer kernels exist in the general form only)
     if (dump) {
         // the debug variant always takes the general (slope) path
-        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, true>), grid, block, 0, st, p, n_qtiles);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, true, false>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, false, false>), grid, block, 0, st, p, n_qtiles);
     } else if (slope) {
-        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, true>), grid, block, 0, st, p, n_qtiles);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, true, false>), grid, block, 0, st, p, n_qtiles);
+        else if (qs_const) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false, true>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false, false>), grid, block, 0, st, p, n_qtiles);
     } else {
-        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, true>), grid, block, 0, st, p, n_qtiles);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, true, false>), grid, block, 0, st, p, n_qtiles);
+        else if (qs_const) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false, true>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false, false>), grid, block, 0, st, p, n_qtiles);
     }
 }
 
