@@ -148,12 +148,15 @@ class PrefillWorkload:
         self.flops_layer = [prefill_flops(B, S, H, d, W) for W, _ in self.layers]
         self.flops = sum(self.flops_layer)
         self.mean_qs = [float(inp[0][1].mean()) for inp in self.inputs]
+        self.mean_vs = [float(inp[2][1].mean()) for inp in self.inputs]
         torch.cuda.synchronize()
 
-    def run_layer(self, i, span_len_hint=None, const_q_scale=False):
+    def run_layer(self, i, span_len_hint=None, const_q_scale=False, const_v_scale=False):
         (q, qs), (k, ks), (v, vs) = self.inputs[i]
         if const_q_scale:   # one number as the query scale, as TScale's own model passes (gpt_att_fp8.cuh:137); of the planes' size
             qs = self.mean_qs[i]
+        if const_v_scale:   # ... and as the value scale (cpu_infer.cpp:454)
+            vs = self.mean_vs[i]
         W, slope = self.layers[i]
         st, fi = self.spans[W]
         # equal-length sequences: tell the library the causal period of the wide layers (a launch-order hint)
@@ -906,6 +909,7 @@ def main():
     ms_short = gpu_time_ms(lambda: wl.run_layer(0), lsteps, 2)
     ms_wide = gpu_time_ms(lambda: wl.run_layer(1), lsteps, 2)
     ms_wide_cq = gpu_time_ms(lambda: wl.run_layer(1, const_q_scale=True), lsteps, 2)
+    ms_wide_cqv = gpu_time_ms(lambda: wl.run_layer(1, const_q_scale=True, const_v_scale=True), lsteps, 2)
     ach = wl.flops_layer[1] / (ms_wide * 1e-3) / 1e12
     result = {
         "metric": "prefill attn TFLOP/s + decode attn HBM GB/s (% of MI355X peak), 1 GPU",
@@ -916,8 +920,10 @@ def main():
                                "(W=256, slope 0.5) + (W=4096, slope 0), f16 out; 616.19 GFLOP per step",
                    "frac_of_fp8_peak": round(tflops / PEAK_FP8_TFLOPS, 5),
                    "layer_ms": {"window256": round(ms_short, 5), "full": round(ms_wide, 5),
-                                # (not part of `value`: the same launch with one number as the query scale, as TScale's own model has)
-                                "full_with_constant_query_scale": round(ms_wide_cq, 5)},
+                                # (not part of `value`: the same launch with one number as the query scale, and as the value scale
+                                # too, which is what TScale's own model passes)
+                                "full_with_constant_query_scale": round(ms_wide_cq, 5),
+                                "full_with_constant_query_and_value_scales": round(ms_wide_cqv, 5)},
                    "layer_tflops": {"window256": round(wl.flops_layer[0] / ms_short / 1e9, 2),
                                     "full": round(wl.flops_layer[1] / ms_wide / 1e9, 2)}},
         # the dominant kernel: the full-window launch (549.62 of the step's 616.19 GFLOP), timed back to back on its own

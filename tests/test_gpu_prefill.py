@@ -127,14 +127,17 @@ def test_prefill_constant_query_scale(ctx, dtype, d, window, slope, seq_lens):
     q, _, k, ks, v, vs = make_qkv(77, n, H, d, dtype)
     VEC = np.float32(1.0 / 48 if dtype == capi.I8 else 1.0 / 96)   # (logits of the usual size for these rows)
     st, fi = orc.make_spans(seq_lens, window)
-    want, want_swl = orc.prefill_q8(dtype, q, k, v, H, float(VEC), ks, vs, st, fi, slope, want_swl=True)
     tt = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
-    for f16 in (False, True):
-        swl = torch.zeros((H, n), dtype=torch.float32, device="cuda")
-        out = ctx.compute_val_lookup(dtype, H, tt(q), tt(k), tt(v), float(VEC), tt(ks), tt(vs), tt(st), tt(fi), slope, out_f16=f16, sum_weight_log=swl)
-        torch.cuda.synchronize()
-        assert_within_tolerance(out.float().cpu().numpy(), want, f"constant query scale, f16 out {f16}")
-        assert np.abs(swl.cpu().numpy() - want_swl).max() < 1e-3
+    for v_const in (False, True):   # ... and one number as the value scale too (cpu_infer.cpp:454): V widened as it is
+        v_scale = float(np.float32(vs.mean())) if v_const else vs
+        want, want_swl = orc.prefill_q8(dtype, q, k, v, H, float(VEC), ks, v_scale, st, fi, slope, want_swl=True)
+        for f16 in (False, True):
+            swl = torch.zeros((H, n), dtype=torch.float32, device="cuda")
+            out = ctx.compute_val_lookup(dtype, H, tt(q), tt(k), tt(v), float(VEC), tt(ks), v_scale if v_const else tt(vs), tt(st), tt(fi), slope,
+                                         out_f16=f16, sum_weight_log=swl)
+            torch.cuda.synchronize()
+            assert_within_tolerance(out.float().cpu().numpy(), want, f"constant query scale, constant value scale {v_const}, f16 out {f16}")
+            assert np.abs(swl.cpu().numpy() - want_swl).max() < 1e-3
 
 
 @pytest.mark.parametrize("dtype,B,S,H,d,window,slope", [

@@ -36,7 +36,8 @@ struct PfLayout {
 // e4m3: v_cvt_scalef32_pk_f16_fp8 (exact widening, unit scale) then a packed f16 multiply.
 // int8: byte b -> f16 bits 0x6400 | (b ^ 0x80) = 1024 + (b + 128); a packed add of -1152 gives b
 //       exactly, then the packed multiply.
-template <int DTYPE>
+// SCALED = false: the values as they are (a scale that is one number for all rows is applied to the result instead).
+template <int DTYPE, bool SCALED = true>
 __device__ inline void widen_v(v4i raw, float vs, v8h &lo, v8h &hi)
 {
     const _Float16 vsh = (_Float16)vs;
@@ -50,11 +51,15 @@ __device__ inline void widen_v(v4i raw, float vs, v8h &lo, v8h &hi)
             const unsigned a = __builtin_amdgcn_perm(u, 0x64646464u, 0x00050004u);
             const unsigned b = __builtin_amdgcn_perm(u, 0x64646464u, 0x00070006u);
             const v2h off = v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
-            h[2 * i] = (__builtin_bit_cast(v2h, a) + off) * vs2;
-            h[2 * i + 1] = (__builtin_bit_cast(v2h, b) + off) * vs2;
+            h[2 * i] = __builtin_bit_cast(v2h, a) + off;
+            h[2 * i + 1] = __builtin_bit_cast(v2h, b) + off;
         } else {
-            h[2 * i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, false) * vs2;
-            h[2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, true) * vs2;
+            h[2 * i] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, false);
+            h[2 * i + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[i], 1.0f, true);
+        }
+        if (SCALED) {
+            h[2 * i] *= vs2;
+            h[2 * i + 1] *= vs2;
         }
     }
     lo = v8h{h[0][0], h[0][1], h[1][0], h[1][1], h[2][0], h[2][1], h[3][0], h[3][1]};
@@ -62,7 +67,7 @@ __device__ inline void widen_v(v4i raw, float vs, v8h &lo, v8h &hi)
 }
 
 // one 32-bit word (4 values) of the same: two packed pairs
-template <int DTYPE>
+template <int DTYPE, bool SCALED = true>
 __device__ inline void widen_v_word(int w, v2h vs2, v2h &h0, v2h &h1)
 {
     if (DTYPE == TSATTN_I8) {
@@ -70,24 +75,31 @@ __device__ inline void widen_v_word(int w, v2h vs2, v2h &h0, v2h &h1)
         const unsigned a = __builtin_amdgcn_perm(u, 0x64646464u, 0x00050004u);
         const unsigned b = __builtin_amdgcn_perm(u, 0x64646464u, 0x00070006u);
         const v2h off = v2h{(_Float16)-1152.0f, (_Float16)-1152.0f};
-        h0 = (__builtin_bit_cast(v2h, a) + off) * vs2;
-        h1 = (__builtin_bit_cast(v2h, b) + off) * vs2;
+        h0 = __builtin_bit_cast(v2h, a) + off;
+        h1 = __builtin_bit_cast(v2h, b) + off;
     } else {
-        h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false) * vs2;
-        h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true) * vs2;
+        h0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+        h1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+    }
+    if (SCALED) {
+        h0 *= vs2;
+        h1 *= vs2;
     }
 }
 
 typedef __attribute__((address_space(3))) v4s *lds_v4s_ptr;
 
 // MULTI: rows may have several spans (p.n_parts arrays of them); otherwise the one-span kernel, which needs fewer registers.
-// QS_CONST: the query scale is one number for all rows (TScale's own model: VEC_SCALE, gpt_att_fp8.cuh:137); it is
+// CONSTS >= 1: the query scale is one number for all rows (TScale's own model: VEC_SCALE, gpt_att_fp8.cuh:137); it is
 // multiplied into the key scales as they are staged and a logit costs one multiply-add instead of a multiply and one.
-template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP, bool MULTI, bool QS_CONST>
+// CONSTS == 2: the value scale is one number too (cpu_infer.cpp:454): V is widened as it is -- exactly -- and the
+// result multiplied by the scale.
+template <int DTYPE, int D, bool OUT_F16, bool SLOPE, bool DUMP, bool MULTI, int CONSTS>
 __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefill_kernel(PrefillParams p, int n_qtiles)
 {
     typedef PfLayout<D> L;
     typedef QkMma<DTYPE, D> Qk;
+    constexpr bool QS_CONST = CONSTS >= 1, VS_CONST = CONSTS == 2;
     constexpr int DT = D / 32;                               // 32-row tiles of O^T
     constexpr int CHUNKS = D / 16;                           // 16-byte chunks per 8-bit row
     constexpr int NLD = (PF_BN * CHUNKS + PF_THREADS - 1) / PF_THREADS;
@@ -285,7 +297,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
                 const int r = ch / CHUNKS, c = ch % CHUNKS;
                 *(v4i *)(k_lds(buf) + r * L::K_PITCH + c * 16) = rk[i];
                 v8h lo, hi;
-                widen_v<DTYPE>(rv[i], rvs[i], lo, hi);
+                widen_v<DTYPE, !VS_CONST>(rv[i], rvs[i], lo, hi);
                 *(v8h *)(v_lds(buf) + r * L::V_PITCH + c * 32) = lo;
                 *(v8h *)(v_lds(buf) + r * L::V_PITCH + c * 32 + 16) = hi;
             }
@@ -583,7 +595,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
                 o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[grp][dt], grp == 0 ? p1a : p1b, o_acc[dt], 0, 0, 0);
                 const int i = m / 4, w = m % 4;
                 const _Float16 vsh = (_Float16)rvs[i];
-                widen_v_word<DTYPE>(rv[i][w], v2h{vsh, vsh}, hh[i][2 * w], hh[i][2 * w + 1]);
+                widen_v_word<DTYPE, !VS_CONST>(rv[i][w], v2h{vsh, vsh}, hh[i][2 * w], hh[i][2 * w + 1]);
                 if (w == 3) {
                     const int ch = tid + i * PF_THREADS;
                     const int r = ch / CHUNKS, c = ch % CHUNKS;
@@ -645,7 +657,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
                     const int r = ch / CHUNKS, c = ch % CHUNKS;
                     if (r < n_keys) {
                         v8h lo, hi;
-                        widen_v<DTYPE>(svv[i], svs[i], lo, hi);
+                        widen_v<DTYPE, !VS_CONST>(svv[i], svs[i], lo, hi);
                         *(v8h *)(v_short + r * L::V_PITCH + c * 32) = lo;
                         *(v8h *)(v_short + r * L::V_PITCH + c * 32 + 16) = hi;
                     }
@@ -719,7 +731,7 @@ __global__ __launch_bounds__(PF_THREADS, (D == 64 && !MULTI) ? 3 : 2) void prefi
     l += l2;
     float l_all = l + __shfl_xor(l, 32, WAVE);
     l_all += fast_exp2(-m_ref);
-    const float inv = 1.0f / l_all;
+    const float inv = (VS_CONST ? p.vs_const : 1.0f) / l_all;
     if constexpr (KV_FUSED) if (p.kv_out) {
         // Fused consumer: KVProduct (gpt/train/cpu_infer.cpp:320-337) of the result, which is in registers, with the
         // rows of kv_k: kv[head][blk][x] = int8((k[x ^ blk] * value[x]) * mult).  x ^ blk stays inside an aligned group
@@ -879,19 +891,22 @@ static void launch_prefill_do(const PrefillParams &p_in, dim3 grid2, hipStream_t
     const bool slope = p.slope != 0.0f;
     dim3 block(PF_THREADS);
     const bool multi = p.n_parts > 1;
-    const bool qs_const = p.qs == nullptr && !dump && !multi; // (the rarer kernels exist in the general form only)
+    // 0: scales per row; 1: one query scale; 2: one query scale and one value scale (the rarer kernels exist in the general form only)
+    const int consts = (p.qs == nullptr && !dump && !multi) ? (p.vs == nullptr ? 2 : 1) : 0;
     if (dump) {
         // the debug variant always takes the general (slope) path
-        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, true, false>), grid, block, 0, st, p, n_qtiles);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, false, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, true, 0>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, true, false, 0>), grid, block, 0, st, p, n_qtiles);
     } else if (slope) {
-        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, true, false>), grid, block, 0, st, p, n_qtiles);
-        else if (qs_const) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false, true>), grid, block, 0, st, p, n_qtiles);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, true, 0>), grid, block, 0, st, p, n_qtiles);
+        else if (consts == 2) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false, 2>), grid, block, 0, st, p, n_qtiles);
+        else if (consts == 1) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false, 1>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, true, false, false, 0>), grid, block, 0, st, p, n_qtiles);
     } else {
-        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, true, false>), grid, block, 0, st, p, n_qtiles);
-        else if (qs_const) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false, true>), grid, block, 0, st, p, n_qtiles);
-        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false, false>), grid, block, 0, st, p, n_qtiles);
+        if (multi) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, true, 0>), grid, block, 0, st, p, n_qtiles);
+        else if (consts == 2) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false, 2>), grid, block, 0, st, p, n_qtiles);
+        else if (consts == 1) hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false, 1>), grid, block, 0, st, p, n_qtiles);
+        else hipLaunchKernelGGL((prefill_kernel<DTYPE, D, OUT_F16, false, false, false, 0>), grid, block, 0, st, p, n_qtiles);
     }
 }
 
