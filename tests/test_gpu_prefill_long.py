@@ -123,6 +123,19 @@ def test_long_constant_query_scale(ctx, dtype, ks_plane, gscale):
 
 
 @pytest.mark.parametrize("dtype", [capi.I8, capi.E4M3])
+def test_long_row_query_scales_with_constant_key_scale(ctx, dtype):
+    """Query scales per row, one number as the key scale and the device scalar on top of it (the general kernel, whose
+    key scales are then a constant in LDS and whose query scales carry the scalar)."""
+    H, n = 2, 450
+    q, qs, k, ks, v, vs = make_qkv(31, n, H, D, dtype)
+    kc = float(np.float32(ks.mean()))
+    st, fi = orc.make_spans([n], 10 ** 6)
+    want = orc.prefill_q8(dtype, q, k, v, H, qs, kc * np.float32(0.6), vs, st, fi, 0.0)
+    out = run_long(ctx, dtype, H, q, qs, k, kc, v, vs, st, fi, k_global_scale=torch.tensor([0.6], device="cuda"))
+    assert_within_tolerance(out, want, "row query scales, constant key scale, global scale")
+
+
+@pytest.mark.parametrize("dtype", [capi.I8, capi.E4M3])
 def test_long_padded_rows_and_planes(ctx, dtype):
     """Q, K, V and the output as column slices of wider arrays (row pitches larger than a row, each different), scale
     planes with a pitch larger than the token count, one head: the kernel's row addresses come from the pitches."""
