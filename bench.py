@@ -229,12 +229,13 @@ class GenerationWorkload:
         self.dout = torch.empty((B, H * d), dtype=torch.float32, device="cuda")
         self.kinds = sorted({w for w, _ in self.sched})
         self.mean_qs = float(self.qkv[0][1].mean())
+        self.mean_vs = float(self.qkv[2][1].mean())
         torch.cuda.synchronize()
 
     def prefill_layer(self, i, const_q_scale=False):
         (q, qs), (k, ks), (v, vs) = self.qkv
-        if const_q_scale:   # one number as the query scale, as the reference's own layer passes (cpu_infer.cpp:448)
-            qs = self.mean_qs
+        if const_q_scale:   # one number as the query scale and one as the value scale, as the reference's own layer passes (cpu_infer.cpp:448,454)
+            qs, vs = self.mean_qs, self.mean_vs
         W, slope = self.sched[i]
         st, fi = self.spans[W]
         self.ctx.compute_val_lookup(self.i8, self.H, q, k, v, qs, ks, vs, st, fi, slope, out=self.out,
@@ -287,7 +288,7 @@ def bench_generation(ctx, steps, facts=None):
                                    "unit": "TOP/s", "frac": round(gw.prefill_flops(first[wide]) / pre_ms[wide] / 1e9 / PEAK_I8_TOPS, 5),
                                    "traffic": None, "launch_ms": round(pre_ms[wide], 5), "flops_per_launch": gw.prefill_flops(first[wide])}}
     cq_ms = gpu_time_ms(lambda: gw.prefill_layer(first[wide], const_q_scale=True), max(50, steps // 5), 1)
-    res["prefill"]["full_layer_ms_with_constant_query_scale"] = round(cq_ms, 5)
+    res["prefill"]["full_layer_ms_with_constant_query_and_value_scales"] = round(cq_ms, 5)
     fact = facts.get("prefill_prompt_int8_full")
     if fact:
         res["prefill"]["roofline"].update({"traffic": fact.get("traffic_bytes"), "traffic_from": fact["profile"]})
