@@ -17,6 +17,8 @@ A "step" is one pass of the hot path over one batch of synthetic input, inputs r
   "prefill_long_span": the two prefill kernels side by side on full-window layers of 32768 tokens at S = 4096, 8192, 16384.
   "token_step_24_layers", "prompt_pass_24_layers": the whole 24-layer stack of the host mirror around those attention
       calls (int8 projections, producer, attention, feed-forward), one generated token and one prompt pass.
+  "prompt_then_generate_256": the last configuration end to end in one timed region (embedding, 24 int8 layers, final
+      layer, greedy choice): 32 prompts of 2048 tokens, then 256 generated tokens each.
 Algorithmic work: FLOPs = 4*d*sum_rows min(row, W) per (sequence, head) (masked tiles count zero,
 the zero vector adds none); decode bytes = K + V planes + both scale planes + q + out.
 
@@ -995,6 +997,9 @@ def main():
         result["token_step_24_layers"] = bench_token_step(ctx, args.steps)
         result["prompt_pass_24_layers"] = bench_prompt_pass(ctx, args.steps)
         torch.cuda.empty_cache()
+        # ---- the last configuration end to end: 32 prompts through the whole int8 model, then 256 greedy tokens each ----
+        result["prompt_then_generate_256"] = bench_prompt_then_generate(ctx)
+        torch.cuda.empty_cache()
 
     # ---- optional: 1.5B-style prefill shapes ---------------------------------------------------------
     if args.extra:
@@ -1004,7 +1009,6 @@ def main():
         result["combiner_matmul"] = bench_matmul(ctx, args.steps)
         result["generate_whole_model"] = bench_generate_model(ctx, args.steps)
         torch.cuda.empty_cache()
-        result["prompt_then_generate_256"] = bench_prompt_then_generate(ctx)
     print(json.dumps(result))
 
 
