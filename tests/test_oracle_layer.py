@@ -120,6 +120,12 @@ def real_layer(mats, scales, width, slope, t, rope, state, cache, mutate=None):
     """One token of one sequence.  cache: list of (qv vector [H*D], v vector [H*D]) of the rows before it."""
     W = {n: m.astype(np.float64) for n, m in mats.items()}
     qv_scale, comb_scale, contr_scale = scales
+    if mutate == "key_scale_10pct":
+        qv_scale *= 1.1
+    if mutate == "combiner_scale_10pct":
+        comb_scale *= 1.1
+    if mutate == "contract_scale_10pct":
+        contr_scale *= 1.1
     dim = state.size
     n, _ = _rms_norm(state, dim // 128)
     qk, qv, k, v = W["qk"] @ n, W["qv"] @ n, W["k"] @ n, W["v"] @ n
@@ -161,12 +167,13 @@ def real_layer(mats, scales, width, slope, t, rope, state, cache, mutate=None):
     return state, val
 
 
-def _run_both(mutate, n_tokens=6, width=100, slope=0.0, seed=21):
+def _run_both(mutate, n_tokens=6, width=100, slope=0.0, seed=21, rms=False, scales=(0.04, 0.03, 0.05)):
     """n_tokens tokens of B sequences through the oracle (one shared cache object, as the reference keeps it) and through
     the real-valued layer; both start every token from the oracle's state, so rounding does not pile up over tokens.
-    Returns the largest differences of the new state's update and of the attention output, relative to their rms."""
+    Returns the largest differences of the new state's update and of the attention output, relative to their rms; with
+    rms=True the rms of the update's difference over all tokens and sequences relative to the update's rms (the int8
+    rounding averages out in it, a scale that is off does not)."""
     mats = make_layer(seed)
-    scales = (0.04, 0.03, 0.05)
     rng = np.random.default_rng(seed + 1)
     state = rng.standard_normal((B, DIM)).astype(np.float32)
     k = np.zeros((B, H, MAXLEN, D), dtype=np.uint8)
@@ -176,6 +183,7 @@ def _run_both(mutate, n_tokens=6, width=100, slope=0.0, seed=21):
     rope = orc.fill_rope(D, 64)
     caches = [[] for _ in range(B)]
     worst_state, worst_val = 0.0, 0.0
+    sq_err, sq_ref = 0.0, 0.0
     for tok in range(n_tokens):
         t = np.full(B, tok, dtype=np.int32)
         new_state, val = orc.add_lookup_product(mats, scales, width, slope, H, D, t, rope, state, k, v, ks, cl)
@@ -184,9 +192,13 @@ def _run_both(mutate, n_tokens=6, width=100, slope=0.0, seed=21):
                                               caches[b], mutate)
             upd, want_upd = new_state[b] - state[b], want_state - state[b]
             worst_state = max(worst_state, np.abs(upd - want_upd).max() / np.sqrt((want_upd ** 2).mean()))
+            sq_err += float(((upd - want_upd) ** 2).sum())
+            sq_ref += float((want_upd ** 2).sum())
             if tok > 0:
                 worst_val = max(worst_val, np.abs(val[b] - want_val).max() / (np.sqrt((want_val ** 2).mean()) + 1e-30))
         state = new_state
+    if rms:
+        return np.sqrt(sq_err / sq_ref)
     return worst_state, worst_val
 
 
@@ -201,3 +213,19 @@ def test_a_wrong_composition_does_not(mutate):
     good_s, good_v = _run_both(None)
     bad_s, bad_v = _run_both(mutate)
     assert max(bad_s / good_s, bad_v / good_v) > 4.0, (mutate, good_s, good_v, bad_s, bad_v)
+
+
+@pytest.mark.parametrize("mutate", ["key_scale_10pct", "combiner_scale_10pct", "contract_scale_10pct"])
+def test_a_scale_ten_percent_off_shows(mutate):
+    """The largest-element figure of the state lets a mis-scaling of 10 % through.  For the two matrix scales that act on
+    the state the rms over everything does not: the int8 rounding leaves about 2 % there and averages out, a scale that is
+    off adds its share in full.  The key scale acts on the logits: the attention output's largest difference doubles."""
+    if mutate == "key_scale_10pct":
+        _, good = _run_both(None)
+        _, bad = _run_both(mutate)
+        assert good < 0.08 and bad > 1.8 * good, (mutate, good, bad)
+        return
+    good = _run_both(None, rms=True)
+    bad = _run_both(mutate, rms=True)
+    assert good < 0.05, good
+    assert bad > 1.5 * good, (mutate, good, bad)
